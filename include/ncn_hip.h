@@ -1,0 +1,150 @@
+/*
+ * ncn_hip.h -- C ABI of the MI355X (gfx950) NCN layer library, libncn_hip.so.
+ *
+ * The library replaces the reference's pybind11 module `ncn_cuda_module`
+ * (ncn_cuda/ncn_cuda.cpp:29-32, built from ncn_fwd_cuda_kernel.cu and ncn_bwd_cuda_kernel.cu).
+ * Differences of contract with that module, all deliberate:
+ *   - the caller owns every buffer (inputs, outputs, workspace); the library never allocates,
+ *     frees or keeps a pointer after a call returns        (reference: torch::zeros_like inside,
+ *     ncn_fwd_cuda_kernel.cu:128-129, ncn_bwd_cuda_kernel.cu:247-251);
+ *   - work is enqueued on the HIP stream passed in and the call returns without a host sync
+ *     (reference: default stream + cudaDeviceSynchronize, ncn_fwd_cuda_kernel.cu:158);
+ *   - every entry point returns 0 or an error code (reference: no checks at all);
+ *   - activations and gradients may be float32 or bfloat16 in memory; all arithmetic is float32;
+ *     W and dW are always float32;
+ *   - `m`, hard-coded to 0.9 in the reference (ncn_fwd_cuda_kernel.cu:72), is an argument;
+ *   - several consecutive stages can be run by one call (n_stages > 1), later stages in place.
+ *
+ * Tensors are row-major [batch, N, E] with E contiguous; a head is a slice of E/n_head features.
+ * Stage `l` of the layer groups the N axis into N/n_cache groups of n_cache rows through the
+ * stride permutation of torch_ref/ncn_pytorch.py:12-41 and runs the n_cache-step recurrence of
+ * torch_ref/ncn_pytorch.py:74-94 on each (batch, head, group).  W holds, per stage, 2E floats:
+ * W[0:E] multiplies the row itself (Wi), W[E:2E] the step's pivot row (Wj); a head uses its own
+ * slice of both halves (torch_ref/ncn_pytorch.py:60-61).
+ *
+ * All pointers are device pointers, 16-byte aligned.  Calls are re-entrant; two calls that write the
+ * same buffers must be ordered by the caller (same stream, or events).
+ */
+#ifndef NCN_HIP_H
+#define NCN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element types of activation / gradient buffers */
+#define NCN_F32 0
+#define NCN_BF16 1
+
+/* activation codes: those of the reference's CUDA surface (ncn_pytorch_wrapper_v2.py:111,
+ * ncn_fwd_cuda_kernel.cu:86-95): 0 tanh, 1 relu, 2 sigmoid, anything else the reference treats as
+ * linear; here only -1 is accepted for linear. */
+#define NCN_ACT_TANH 0
+#define NCN_ACT_RELU 1
+#define NCN_ACT_SIGMOID 2
+#define NCN_ACT_LINEAR (-1)
+
+/* error codes (negative: rejected before any GPU work; positive: a hipError_t from the runtime) */
+#define NCN_OK 0
+#define NCN_ERR_NULL (-1)        /* a required pointer is NULL */
+#define NCN_ERR_SHAPE (-2)       /* non-positive size, N % n_cache != 0, E % n_head != 0, bad stage range */
+#define NCN_ERR_DTYPE (-3)       /* unknown element type */
+#define NCN_ERR_ACTIVATION (-4)  /* unknown activation code */
+#define NCN_ERR_WORKSPACE (-5)   /* workspace missing or smaller than ncn_workspace_bytes() */
+#define NCN_ERR_UNSUPPORTED (-6) /* n_cache > 64, or head width too large for the generic kernel */
+#define NCN_ERR_ALIGN (-7)       /* a pointer is not 16-byte aligned */
+#define NCN_ERR_ALIAS (-8)       /* n_stages > 1 needs the state buffers the call would carry it in */
+
+/* Shape of one problem; shared by all entry points. */
+typedef struct ncn_shape {
+    int64_t batch;   /* X.size(0) */
+    int64_t N;       /* X.size(1), the mixing axis (reference: ctx_dim) */
+    int64_t E;       /* X.size(2) (reference: embed_dim) */
+    int32_t n_head;  /* heads; head width Ec = E / n_head (reference: nhead) */
+    int32_t n_cache; /* group size (reference: cache_dim) */
+} ncn_shape;
+
+/*
+ * Forward of stages first_stage .. first_stage+n_stages-1.
+ * Replaces: forward(X, Xa, W, alpha, activation, cache_dim, nhead, module_l) -> {Y, Ya}
+ *           ncn_cuda/ncn_cuda.cpp:3-12, ncn_fwd_cuda_kernel.cu:115-161 (one stage per call there).
+ * x, xa       in   [batch,N,E] of in_dtype
+ * y, ya       out  [batch,N,E] of out_dtype; may alias x, xa when the dtypes are equal (each row is
+ *                  read and written by exactly one wavefront).  With n_stages > 1 the later stages
+ *                  run in place on y, ya.
+ * y32, ya32   out  optional (NULL to skip) float32 copies of the final y, ya: what a bf16 caller saves
+ *                  for the reversible backward.
+ * W           in   [n_stages, 2E] float32
+ */
+int ncn_forward(const void* x, const void* xa, int in_dtype,
+                void* y, void* ya, int out_dtype,
+                float* y32, float* ya32,
+                const float* W,
+                const ncn_shape* shape, int first_stage, int n_stages,
+                float alpha, float m, int activation, void* stream);
+
+/*
+ * Reversible backward of stages first_stage+n_stages-1 .. first_stage, from the OUTPUTS of the last
+ * of them.
+ * Replaces: backward(Y, Ya, dY, dYa, W, alpha, activation, cache_dim, nhead, module_l)
+ *           -> {X, Xa, dX, dXa, dW[batch,N,2E]}  ncn_cuda/ncn_cuda.cpp:14-25,
+ *           ncn_bwd_cuda_kernel.cu:232-288, plus the torch.sum(dW,(0,1)) of
+ *           ncn_pytorch_wrapper_v2.py:48, which is done here.
+ * y, ya       in   [batch,N,E] of y_dtype: outputs of the last stage (use float32: the inversion
+ *                  amplifies rounding by (1/m)^n_cache per stage)
+ * dy, dya     in   [batch,N,E] of dy_dtype; dya may be NULL, meaning zeros
+ * dx, dxa     out  [batch,N,E] of dx_dtype
+ * x_rec,xa_rec out float32 [batch,N,E], reconstructed inputs of first_stage; may be NULL when
+ *                  n_stages == 1.  With n_stages > 1 they are required, dx_dtype must be NCN_F32, and
+ *                  the four of x_rec, xa_rec, dx, dxa carry the state between stages in place.
+ * W           in   [n_stages, 2E] float32
+ * dW          out  [n_stages, 2E] float32, overwritten (summed over batch, groups and rows)
+ * workspace        scratch of at least ncn_workspace_bytes(shape) bytes
+ */
+int ncn_backward(const void* y, const void* ya, int y_dtype,
+                 const void* dy, const void* dya, int dy_dtype,
+                 void* dx, void* dxa, int dx_dtype,
+                 float* x_rec, float* xa_rec,
+                 const float* W, float* dW,
+                 void* workspace, size_t workspace_bytes,
+                 const ncn_shape* shape, int first_stage, int n_stages,
+                 float alpha, float m, int activation, void* stream);
+
+/*
+ * Inverse of stages first_stage+n_stages-1 .. first_stage: x, xa such that ncn_forward(x, xa) = y, ya.
+ * Follows NCNFunctionPytorch.invert (torch_ref/ncn_pytorch_invertible.py:87-113), which the
+ * reference's CUDA module only runs inside backward (ncn_bwd_cuda_kernel.cu:88-115).
+ * May run in place (x == y, xa == ya) when the dtypes are equal.
+ */
+int ncn_inverse(const void* y, const void* ya, int in_dtype,
+                void* x, void* xa, int out_dtype,
+                const float* W,
+                const ncn_shape* shape, int first_stage, int n_stages,
+                float alpha, float m, int activation, void* stream);
+
+/* Bytes of scratch ncn_backward needs for this shape (0 on an invalid shape).  No reference counterpart:
+ * the reference allocates a [batch,N,2E] partial-dW tensor per call (ncn_bwd_cuda_kernel.cu:251). */
+size_t ncn_workspace_bytes(const ncn_shape* shape);
+
+/* 2: hand-tuned register kernel, 1: generic LDS kernel, 0: not supported (n_cache > 64, or the
+ * head width does not fit the generic kernel's LDS).  No reference counterpart. */
+int ncn_kernel_path(const ncn_shape* shape);
+
+/* Validates arguments exactly as the entry points do, without touching the GPU.  Returns NCN_OK or
+ * the error the corresponding call would return before launching.  No reference counterpart (the
+ * reference validates nothing). */
+int ncn_check_shape(const ncn_shape* shape, int first_stage, int n_stages, int activation);
+
+/* Human-readable text for a code returned by the functions above. */
+const char* ncn_error_string(int code);
+
+/* Library version, "major.minor". */
+const char* ncn_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NCN_HIP_H */

@@ -1,0 +1,65 @@
+"""ctypes binding of libncn_hip.so (C ABI declared in include/ncn_hip.h).
+
+There is no fallback: if the library is missing or a symbol is absent, loading raises.
+"""
+import ctypes
+import os
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(PKG_DIR, "libncn_hip.so")
+
+NCN_F32, NCN_BF16 = 0, 1
+ACT_TANH, ACT_RELU, ACT_SIGMOID, ACT_LINEAR = 0, 1, 2, -1
+
+EXPORTS = ("ncn_forward", "ncn_backward", "ncn_inverse", "ncn_workspace_bytes", "ncn_kernel_path",
+           "ncn_check_shape", "ncn_error_string", "ncn_version")
+
+
+class NcnShape(ctypes.Structure):
+    _fields_ = [("batch", ctypes.c_int64), ("N", ctypes.c_int64), ("E", ctypes.c_int64),
+                ("n_head", ctypes.c_int32), ("n_cache", ctypes.c_int32)]
+
+
+_lib = None
+
+
+def load():
+    """Load the shared library once and declare the prototypes."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `python -m ncn_cuda_amd._build` "
+            "(or __graft_entry__.build()); there is no CPU or PyTorch fallback for the NCN kernels")
+    lib = ctypes.CDLL(LIB_PATH)
+    vp, f32p, shp = ctypes.c_void_p, ctypes.c_void_p, ctypes.POINTER(NcnShape)
+    i, fl = ctypes.c_int, ctypes.c_float
+    lib.ncn_forward.restype = i
+    lib.ncn_forward.argtypes = [vp, vp, i, vp, vp, i, f32p, f32p, f32p, shp, i, i, fl, fl, i, vp]
+    lib.ncn_backward.restype = i
+    lib.ncn_backward.argtypes = [vp, vp, i, vp, vp, i, vp, vp, i, f32p, f32p, f32p, f32p, vp, ctypes.c_size_t,
+                                 shp, i, i, fl, fl, i, vp]
+    lib.ncn_inverse.restype = i
+    lib.ncn_inverse.argtypes = [vp, vp, i, vp, vp, i, f32p, shp, i, i, fl, fl, i, vp]
+    lib.ncn_workspace_bytes.restype = ctypes.c_size_t
+    lib.ncn_workspace_bytes.argtypes = [shp]
+    lib.ncn_kernel_path.restype = i
+    lib.ncn_kernel_path.argtypes = [shp]
+    lib.ncn_check_shape.restype = i
+    lib.ncn_check_shape.argtypes = [shp, i, i, i]
+    lib.ncn_error_string.restype = ctypes.c_char_p
+    lib.ncn_error_string.argtypes = [i]
+    lib.ncn_version.restype = ctypes.c_char_p
+    lib.ncn_version.argtypes = []
+    _lib = lib
+    return lib
+
+
+def error_string(code):
+    return load().ncn_error_string(int(code)).decode()
+
+
+def check(code, what):
+    if code != 0:
+        raise RuntimeError(f"{what} failed: {error_string(code)} (code {code})")

@@ -1,0 +1,226 @@
+// C ABI of libncn_hip.so: argument validation, stage sequencing and launches.  See include/ncn_hip.h.
+#include <hip/hip_runtime.h>
+
+#include "../../include/ncn_hip.h"
+#include "ncn_launch.h"
+
+namespace {
+
+using namespace ncn;
+
+bool known_activation(int a) {
+    return a == NCN_ACT_TANH || a == NCN_ACT_RELU || a == NCN_ACT_SIGMOID || a == NCN_ACT_LINEAR;
+}
+bool known_dtype(int d) { return d == NCN_F32 || d == NCN_BF16; }
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// 2 = register kernels, 1 = generic LDS kernels, 0 = unsupported
+int kernel_path(const ncn_shape* sh, int activation) {
+    if (sh->n_cache < 1 || sh->n_cache > 64) return 0;
+    const int64_t ec = sh->E / sh->n_head;
+    if (activation == NCN_ACT_TANH && ec <= 64 && fast_fpl(sh->n_cache, (int)ec) != 0) return 2;
+    if (ec <= kGenericMaxHeadDim) return 1;
+    return 0;
+}
+
+int check_shape(const ncn_shape* sh, int first_stage, int n_stages, int activation) {
+    if (!sh) return NCN_ERR_NULL;
+    if (sh->batch <= 0 || sh->N <= 0 || sh->E <= 0 || sh->n_head <= 0 || sh->n_cache <= 0) return NCN_ERR_SHAPE;
+    if (sh->N % sh->n_cache != 0 || sh->E % sh->n_head != 0) return NCN_ERR_SHAPE;
+    if (first_stage < 0 || n_stages < 1) return NCN_ERR_SHAPE;
+    if (!known_activation(activation)) return NCN_ERR_ACTIVATION;
+    if (kernel_path(sh, activation) == 0) return NCN_ERR_UNSUPPORTED;
+    // 32-bit tile and block arithmetic inside the kernels
+    const int64_t groups = sh->N / sh->n_cache;
+    if (groups > (int64_t)1 << 24) return NCN_ERR_UNSUPPORTED;
+    if (sh->batch * groups > (int64_t)1 << 30) return NCN_ERR_UNSUPPORTED;
+    return NCN_OK;
+}
+
+// 2^(stage-1) mod groups without overflow (torch_ref/ncn_pytorch.py:38 uses Python big integers)
+uint32_t stage_stride(int stage, uint32_t groups) {
+    if (stage == 0) return 0;
+    uint64_t s = 1 % groups;
+    for (int k = 1; k < stage; ++k) s = (s * 2) % groups;
+    return (uint32_t)s;
+}
+
+struct Plan {
+    int path;
+    int groups_per_tile;
+    uint32_t groups, tiles_per_inst, total_tiles;
+    int grid_x;
+};
+
+Plan make_plan(const ncn_shape* sh, int activation) {
+    Plan p;
+    p.path = kernel_path(sh, activation);
+    const int ec = (int)(sh->E / sh->n_head);
+    p.groups_per_tile = (p.path == 2) ? fast_groups_per_tile(sh->n_cache, ec) : generic_groups_per_tile(sh->n_cache);
+    p.groups = (uint32_t)(sh->N / sh->n_cache);
+    p.tiles_per_inst = (p.groups + p.groups_per_tile - 1) / p.groups_per_tile;
+    p.total_tiles = (uint32_t)(sh->batch * p.tiles_per_inst);
+    const int tiles_per_block = (p.path == 2) ? 4 : 1;
+    const int64_t blocks = ((int64_t)p.total_tiles + tiles_per_block - 1) / tiles_per_block;
+    p.grid_x = (int)(blocks < kMaxGridX ? blocks : kMaxGridX);
+    return p;
+}
+
+void fill_common(StageArgs& a, const ncn_shape* sh, const Plan& p, int stage, float alpha, float m, int activation) {
+    a.N = sh->N;
+    a.E = sh->E;
+    a.total_tiles = p.total_tiles;
+    a.tiles_per_inst = p.tiles_per_inst;
+    a.groups = p.groups;
+    a.stride = stage_stride(stage, p.groups);
+    a.groups_pow2 = (p.groups & (p.groups - 1)) == 0 ? 1u : 0u;
+    a.n_cache = sh->n_cache;
+    a.head_dim = (int)(sh->E / sh->n_head);
+    a.activation = activation;
+    a.alpha = alpha;
+    a.m = m;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* ncn_version(void) { return "0.1"; }
+
+const char* ncn_error_string(int code) {
+    switch (code) {
+        case NCN_OK: return "ok";
+        case NCN_ERR_NULL: return "a required pointer is NULL";
+        case NCN_ERR_SHAPE: return "bad shape: sizes must be positive, N % n_cache == 0, E % n_head == 0, n_stages >= 1";
+        case NCN_ERR_DTYPE: return "unknown element type (0 = float32, 1 = bfloat16)";
+        case NCN_ERR_ACTIVATION: return "unknown activation code (0 tanh, 1 relu, 2 sigmoid, -1 linear)";
+        case NCN_ERR_WORKSPACE: return "workspace is NULL or smaller than ncn_workspace_bytes()";
+        case NCN_ERR_UNSUPPORTED: return "unsupported shape: n_cache must be <= 64 and the head width <= 64";
+        case NCN_ERR_ALIGN: return "a pointer is not 16-byte aligned";
+        case NCN_ERR_ALIAS: return "n_stages > 1 needs float32 x_rec, xa_rec, dx, dxa to carry the state";
+        default: break;
+    }
+    if (code > 0) return hipGetErrorString((hipError_t)code);
+    return "unknown error";
+}
+
+int ncn_check_shape(const ncn_shape* shape, int first_stage, int n_stages, int activation) {
+    return check_shape(shape, first_stage, n_stages, activation);
+}
+
+int ncn_kernel_path(const ncn_shape* shape) {
+    if (!shape || shape->batch <= 0 || shape->N <= 0 || shape->E <= 0 || shape->n_head <= 0 || shape->n_cache <= 0)
+        return 0;
+    if (shape->E % shape->n_head != 0) return 0;
+    return kernel_path(shape, NCN_ACT_TANH);
+}
+
+size_t ncn_workspace_bytes(const ncn_shape* shape) {
+    if (check_shape(shape, 0, 1, NCN_ACT_TANH) != NCN_OK) return 0;
+    return (size_t)kMaxGridX * 2 * (size_t)shape->E * sizeof(float);
+}
+
+int ncn_forward(const void* x, const void* xa, int in_dtype, void* y, void* ya, int out_dtype, float* y32, float* ya32,
+                const float* W, const ncn_shape* shape, int first_stage, int n_stages, float alpha, float m,
+                int activation, void* stream) {
+    int rc = check_shape(shape, first_stage, n_stages, activation);
+    if (rc != NCN_OK) return rc;
+    if (!x || !xa || !y || !ya || !W) return NCN_ERR_NULL;
+    if ((y32 == nullptr) != (ya32 == nullptr)) return NCN_ERR_NULL;
+    if (!known_dtype(in_dtype) || !known_dtype(out_dtype)) return NCN_ERR_DTYPE;
+    if (!aligned16(x) || !aligned16(xa) || !aligned16(y) || !aligned16(ya) || !aligned16(W) || !aligned16(y32) ||
+        !aligned16(ya32))
+        return NCN_ERR_ALIGN;
+    const Plan p = make_plan(shape, activation);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    for (int k = 0; k < n_stages; ++k) {
+        StageArgs a{};
+        fill_common(a, shape, p, first_stage + k, alpha, m, activation);
+        a.in0 = k == 0 ? x : y;
+        a.in1 = k == 0 ? xa : ya;
+        a.in_dtype = k == 0 ? in_dtype : out_dtype;
+        a.out0 = y;
+        a.out1 = ya;
+        a.out_dtype = out_dtype;
+        const bool last = (k == n_stages - 1);
+        a.aux0 = last ? y32 : nullptr;
+        a.aux1 = last ? ya32 : nullptr;
+        a.W = W + (int64_t)k * 2 * shape->E;
+        hipError_t err = (p.path == 2) ? launch_fast_forward(kForward, a, shape->n_head, p.grid_x, s)
+                                       : launch_generic(kForward, a, shape->n_head, p.grid_x, s);
+        if (err != hipSuccess) return (int)err;
+    }
+    return NCN_OK;
+}
+
+int ncn_inverse(const void* y, const void* ya, int in_dtype, void* x, void* xa, int out_dtype, const float* W,
+                const ncn_shape* shape, int first_stage, int n_stages, float alpha, float m, int activation,
+                void* stream) {
+    int rc = check_shape(shape, first_stage, n_stages, activation);
+    if (rc != NCN_OK) return rc;
+    if (!x || !xa || !y || !ya || !W) return NCN_ERR_NULL;
+    if (!known_dtype(in_dtype) || !known_dtype(out_dtype)) return NCN_ERR_DTYPE;
+    if (!aligned16(x) || !aligned16(xa) || !aligned16(y) || !aligned16(ya) || !aligned16(W)) return NCN_ERR_ALIGN;
+    const Plan p = make_plan(shape, activation);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    for (int k = n_stages - 1; k >= 0; --k) {
+        StageArgs a{};
+        fill_common(a, shape, p, first_stage + k, alpha, m, activation);
+        const bool first = (k == n_stages - 1);
+        a.in0 = first ? y : x;
+        a.in1 = first ? ya : xa;
+        a.in_dtype = first ? in_dtype : out_dtype;
+        a.out0 = x;
+        a.out1 = xa;
+        a.out_dtype = out_dtype;
+        a.W = W + (int64_t)k * 2 * shape->E;
+        hipError_t err = (p.path == 2) ? launch_fast_forward(kInverse, a, shape->n_head, p.grid_x, s)
+                                       : launch_generic(kInverse, a, shape->n_head, p.grid_x, s);
+        if (err != hipSuccess) return (int)err;
+    }
+    return NCN_OK;
+}
+
+int ncn_backward(const void* y, const void* ya, int y_dtype, const void* dy, const void* dya, int dy_dtype, void* dx,
+                 void* dxa, int dx_dtype, float* x_rec, float* xa_rec, const float* W, float* dW, void* workspace,
+                 size_t workspace_bytes, const ncn_shape* shape, int first_stage, int n_stages, float alpha, float m,
+                 int activation, void* stream) {
+    int rc = check_shape(shape, first_stage, n_stages, activation);
+    if (rc != NCN_OK) return rc;
+    if (!y || !ya || !dy || !dx || !dxa || !W || !dW) return NCN_ERR_NULL;
+    if ((x_rec == nullptr) != (xa_rec == nullptr)) return NCN_ERR_NULL;
+    if (!known_dtype(y_dtype) || !known_dtype(dy_dtype) || !known_dtype(dx_dtype)) return NCN_ERR_DTYPE;
+    if (n_stages > 1 && (!x_rec || dx_dtype != NCN_F32)) return NCN_ERR_ALIAS;
+    if (!workspace || workspace_bytes < ncn_workspace_bytes(shape)) return NCN_ERR_WORKSPACE;
+    if (!aligned16(y) || !aligned16(ya) || !aligned16(dy) || !aligned16(dya) || !aligned16(dx) || !aligned16(dxa) ||
+        !aligned16(x_rec) || !aligned16(xa_rec) || !aligned16(W) || !aligned16(dW) || !aligned16(workspace))
+        return NCN_ERR_ALIGN;
+    const Plan p = make_plan(shape, activation);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    for (int k = n_stages - 1; k >= 0; --k) {
+        StageArgs a{};
+        fill_common(a, shape, p, first_stage + k, alpha, m, activation);
+        const bool top = (k == n_stages - 1);
+        a.in0 = top ? y : x_rec;
+        a.in1 = top ? ya : xa_rec;
+        a.in_dtype = top ? y_dtype : NCN_F32;
+        a.g0 = top ? dy : dx;
+        a.g1 = top ? dya : dxa;
+        a.g_dtype = top ? dy_dtype : NCN_F32;
+        a.out0 = dx;
+        a.out1 = dxa;
+        a.out_dtype = dx_dtype;
+        a.aux0 = x_rec;
+        a.aux1 = xa_rec;
+        a.W = W + (int64_t)k * 2 * shape->E;
+        a.dw_partials = static_cast<float*>(workspace);
+        hipError_t err = (p.path == 2) ? launch_fast_backward(a, shape->n_head, p.grid_x, s)
+                                       : launch_generic(kBackward, a, shape->n_head, p.grid_x, s);
+        if (err != hipSuccess) return (int)err;
+        err = launch_reduce_dw(a.dw_partials, p.grid_x, 2 * shape->E, dW + (int64_t)k * 2 * shape->E, s);
+        if (err != hipSuccess) return (int)err;
+    }
+    return NCN_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,21 @@
+// Instantiations and dispatch of the register-resident reversible backward stage kernel.
+#include "ncn_configs.h"
+#include "ncn_launch.h"
+#include "ncn_stage_kernels.h"
+
+namespace ncn {
+
+hipError_t launch_fast_backward(const StageArgs& a, int n_head, int grid_x, hipStream_t s) {
+    const dim3 grid(grid_x, n_head), block(kBlockThreads);
+#define NCN_CASE(NC, EC, FPL)                                                                  \
+    static_assert(fast_fpl(NC, EC) == FPL, "config list disagrees with fast_fpl()");          \
+    if (a.n_cache == NC && a.head_dim == EC) {                                                 \
+        hipLaunchKernelGGL((stage_backward_kernel<NC, EC, FPL>), grid, block, 0, s, a);        \
+        return hipGetLastError();                                                              \
+    }
+    NCN_FOR_EACH_FAST_CONFIG(NCN_CASE)
+#undef NCN_CASE
+    return hipErrorInvalidConfiguration;
+}
+
+}  // namespace ncn

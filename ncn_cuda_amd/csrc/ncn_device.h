@@ -1,0 +1,185 @@
+// Device-side building blocks shared by the NCN stage kernels (gfx950, wave64).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/ncn_hip.h"
+
+namespace ncn {
+
+// Everything one stage launch needs.  Which pointer means what depends on the kernel:
+//   forward : in0,in1 = x,xa        out0,out1 = y,ya      aux0,aux1 = optional float32 copies of y,ya
+//   inverse : in0,in1 = y,ya        out0,out1 = x,xa
+//   backward: in0,in1 = y,ya        g0,g1 = dy,dya (g1 may be null = zeros)
+//             out0,out1 = dx,dxa    aux0,aux1 = optional float32 reconstructed x,xa
+struct StageArgs {
+    const void* in0;
+    const void* in1;
+    const void* g0;
+    const void* g1;
+    void* out0;
+    void* out1;
+    float* aux0;
+    float* aux1;
+    const float* W;      // [2E] of this stage
+    float* dw_partials;  // backward: [gridDim.x][2E]
+    int64_t N, E;
+    uint32_t total_tiles;     // batch * tiles_per_instance
+    uint32_t tiles_per_inst;  // ceil(groups / groups-per-wave-tile)
+    uint32_t groups;          // N / n_cache
+    uint32_t stride;          // stride of this stage in blocks: 0, or 2^(stage-1) mod groups
+    uint32_t groups_pow2;     // 1 when `groups` is a power of two
+    int32_t n_cache, head_dim;
+    int32_t in_dtype, g_dtype, out_dtype;
+    int32_t activation;
+    float alpha, m;
+};
+
+// ---------------------------------------------------------------------------------------------
+// bfloat16 <-> float32 (round to nearest even; NaN stays NaN)
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ float bf16_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+
+__device__ __forceinline__ uint32_t f32_to_bf16(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+
+// Row fragment of FPL consecutive features, element offset `off` into a buffer of type `dtype`.
+template <int FPL>
+__device__ __forceinline__ void load_frag(const void* base, int dtype, int64_t off, bool valid, float (&v)[FPL]) {
+    static_assert(FPL % 4 == 0, "fragment must be a multiple of 4 features");
+    if (!valid) {
+#pragma unroll
+        for (int f = 0; f < FPL; ++f) v[f] = 0.f;
+        return;
+    }
+    if (dtype == NCN_F32) {
+        const float4* p = reinterpret_cast<const float4*>(static_cast<const float*>(base) + off);
+#pragma unroll
+        for (int k = 0; k < FPL / 4; ++k) {
+            float4 t = p[k];
+            v[4 * k + 0] = t.x; v[4 * k + 1] = t.y; v[4 * k + 2] = t.z; v[4 * k + 3] = t.w;
+        }
+    } else {
+        const uint2* p = reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(base) + off);
+#pragma unroll
+        for (int k = 0; k < FPL / 4; ++k) {
+            uint2 t = p[k];
+            v[4 * k + 0] = bf16_to_f32(t.x & 0xffffu); v[4 * k + 1] = bf16_to_f32(t.x >> 16);
+            v[4 * k + 2] = bf16_to_f32(t.y & 0xffffu); v[4 * k + 3] = bf16_to_f32(t.y >> 16);
+        }
+    }
+}
+
+template <int FPL>
+__device__ __forceinline__ void store_frag(void* base, int dtype, int64_t off, bool valid, const float (&v)[FPL]) {
+    if (!valid) return;
+    if (dtype == NCN_F32) {
+        float4* p = reinterpret_cast<float4*>(static_cast<float*>(base) + off);
+#pragma unroll
+        for (int k = 0; k < FPL / 4; ++k) p[k] = make_float4(v[4 * k], v[4 * k + 1], v[4 * k + 2], v[4 * k + 3]);
+    } else {
+        uint2* p = reinterpret_cast<uint2*>(static_cast<uint16_t*>(base) + off);
+#pragma unroll
+        for (int k = 0; k < FPL / 4; ++k) {
+            uint2 t;
+            t.x = f32_to_bf16(v[4 * k + 0]) | (f32_to_bf16(v[4 * k + 1]) << 16);
+            t.y = f32_to_bf16(v[4 * k + 2]) | (f32_to_bf16(v[4 * k + 3]) << 16);
+            p[k] = t;
+        }
+    }
+}
+
+__device__ __forceinline__ float load_elem(const void* base, int dtype, int64_t off) {
+    if (dtype == NCN_F32) return static_cast<const float*>(base)[off];
+    return bf16_to_f32(static_cast<const uint16_t*>(base)[off]);
+}
+
+__device__ __forceinline__ void store_elem(void* base, int dtype, int64_t off, float v) {
+    if (dtype == NCN_F32) static_cast<float*>(base)[off] = v;
+    else static_cast<uint16_t*>(base)[off] = static_cast<uint16_t>(f32_to_bf16(v));
+}
+
+// ---------------------------------------------------------------------------------------------
+// cross-lane moves inside one 64-wide wavefront
+// ---------------------------------------------------------------------------------------------
+// value of lane (lane ^ S)
+template <int S>
+__device__ __forceinline__ float lane_xor(float v) {
+    static_assert(S == 1 || S == 2 || S == 4 || S == 8 || S == 16 || S == 32, "power of two below 64");
+    int x = __float_as_int(v);
+    if constexpr (S == 1) {
+        x = __builtin_amdgcn_mov_dpp(x, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
+    } else if constexpr (S == 2) {
+        x = __builtin_amdgcn_mov_dpp(x, 0x4E, 0xF, 0xF, true);  // quad_perm [2,3,0,1]
+    } else if constexpr (S < 32) {
+        x = __builtin_amdgcn_ds_swizzle(x, (S << 10) | 0x1F);   // bit mode: lane' = lane ^ S inside 32
+    } else {
+        const int lane = __lane_id();
+        x = __builtin_amdgcn_ds_bpermute((lane ^ 32) << 2, x);
+    }
+    return __int_as_float(x);
+}
+
+// sum over the lanes {lane ^ k*LO : k} for strides LO, 2*LO, .. < HI  (LO, HI powers of two)
+template <int LO, int HI>
+__device__ __forceinline__ float lane_sum(float v) {
+    if constexpr (LO < HI) {
+        v += lane_xor<LO>(v);
+        return lane_sum<LO * 2, HI>(v);
+    } else {
+        return v;
+    }
+}
+
+// value held by lane `src_lane` (any lane of the wave; computed at run time)
+__device__ __forceinline__ float lane_read(float v, int src_lane) {
+    return __int_as_float(__builtin_amdgcn_ds_bpermute(src_lane << 2, __float_as_int(v)));
+}
+
+// ---------------------------------------------------------------------------------------------
+// activation: F(T) and dF/dT.  Codes of the reference's CUDA kernels
+// (ncn_fwd_cuda_kernel.cu:86-95, ncn_bwd_cuda_kernel.cu:137-150).
+// ---------------------------------------------------------------------------------------------
+// tanh(T) = 1 - 2/(1 + e^{2T}) with the hardware exp2 and reciprocal (about 1 ulp each): the absolute
+// error of F stays near 1e-7 over the whole range, and the saturated ends come out exactly +-1.
+__device__ __forceinline__ void tanh_fd(float T, float& F, float& dF) {
+    const float t = __builtin_amdgcn_exp2f(T * 2.8853900817779268f);
+    const float r = __builtin_amdgcn_rcpf(t + 1.0f);
+    F = fmaf(-2.0f, r, 1.0f);
+    dF = 4.0f * r * (1.0f - r);  // 1 - F^2
+}
+
+__device__ __forceinline__ float tanh_f(float T) {
+    const float t = __builtin_amdgcn_exp2f(T * 2.8853900817779268f);
+    const float r = __builtin_amdgcn_rcpf(t + 1.0f);
+    return fmaf(-2.0f, r, 1.0f);
+}
+
+__device__ __forceinline__ void act_fd(int code, float T, float& F, float& dF) {
+    if (code == NCN_ACT_TANH) {
+        tanh_fd(T, F, dF);
+    } else if (code == NCN_ACT_RELU) {
+        F = fmaxf(T, 0.f);
+        dF = F > 0.f ? 1.f : 0.f;
+    } else if (code == NCN_ACT_SIGMOID) {
+        const float t = __builtin_amdgcn_exp2f(-T * 1.4426950408889634f);
+        F = __builtin_amdgcn_rcpf(1.0f + t);
+        dF = F * (1.0f - F);
+    } else {
+        F = T;
+        dF = 1.f;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// stride permutation (torch_ref/ncn_pytorch.py:38-40): block that slot `slot` of group `group` reads
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ uint32_t stage_block(const StageArgs& A, uint32_t group, uint32_t slot) {
+    const uint32_t t = group + slot * A.stride;  // < 65 * groups, checked on the host to fit 32 bits
+    return A.groups_pow2 ? (t & (A.groups - 1u)) : (t % A.groups);
+}
+
+}  // namespace ncn

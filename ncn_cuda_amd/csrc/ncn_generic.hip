@@ -1,0 +1,216 @@
+// Generic stage kernels: any n_cache <= 64 and any head width up to kGenericMaxHeadDim, all four
+// activations.  One 64-lane wavefront per block, one lane per row, floor(64/n_cache) groups per
+// wave tile; the per-row state lives in LDS as [feature][lane] arrays so that the pivot row of a step
+// and the sum over a group's rows are plain LDS reads.  This is the slow, shape-agnostic path; the
+// register kernels in ncn_stage_kernels.h cover the shapes that matter for speed.
+// Same arithmetic as there; see that file for the formulas and their reference citations.
+#include "ncn_launch.h"
+
+namespace ncn {
+
+namespace {
+
+struct GenericLane {
+    bool valid;
+    int64_t off;   // element offset of this lane's row, feature 0 of the head
+    int row;       // slot inside the group
+    int base;      // lane of slot 0 of this lane's group
+};
+
+__device__ __forceinline__ GenericLane generic_lane(const StageArgs& A, uint32_t t, int lane, int head) {
+    GenericLane L;
+    const int n = A.n_cache;
+    const int gpw = 64 / n;
+    const int gw = lane / n;
+    L.row = lane - gw * n;
+    L.base = gw * n;
+    const uint32_t b = t / A.tiles_per_inst;
+    const uint32_t tile = t - b * A.tiles_per_inst;
+    const uint32_t group = tile * gpw + gw;
+    L.valid = (gw < gpw) && (group < A.groups);
+    const uint32_t blk = stage_block(A, L.valid ? group : 0u, (uint32_t)L.row);
+    const int64_t pos = (int64_t)blk * n + L.row;
+    L.off = ((int64_t)b * A.N + pos) * A.E + (int64_t)head * A.head_dim;
+    if (!L.valid) L.base = lane, L.row = 0;  // idle lanes talk to themselves only
+    return L;
+}
+
+#define LDS(arr, f) lds[((arr) * ec + (f)) * 64 + lane]
+#define LDS_AT(arr, f, l) lds[((arr) * ec + (f)) * 64 + (l)]
+
+// pass 0: forward, pass 1: inverse
+__global__ void __launch_bounds__(64) generic_forward_kernel(const StageArgs A, const int inverse) {
+    extern __shared__ float lds[];
+    const int lane = threadIdx.x, head = blockIdx.y, ec = A.head_dim, n = A.n_cache;
+    const float alpha = A.alpha, m = A.m, om = 1.f - A.m, oa = 1.f - A.alpha;
+    const float inv_m = 1.f / m, k_ba = om / m;
+    const float* Wi = A.W + (int64_t)head * ec;
+    const float* Wj = Wi + A.E;
+    enum { X = 0, XA = 1 };
+    for (uint32_t t = blockIdx.x; t < A.total_tiles; t += gridDim.x) {
+        const GenericLane L = generic_lane(A, t, lane, head);
+        for (int f = 0; f < ec; ++f) {
+            LDS(X, f) = L.valid ? load_elem(A.in0, A.in_dtype, L.off + f) : 0.f;
+            LDS(XA, f) = L.valid ? load_elem(A.in1, A.in_dtype, L.off + f) : 0.f;
+        }
+        __syncthreads();
+        for (int step = 0; step < n; ++step) {
+            const int j = inverse ? n - 1 - step : step;
+            const int jl = L.valid ? L.base + j : lane;
+            if (inverse) {
+                for (int f = 0; f < ec; ++f) LDS(X, f) = fmaf(LDS(X, f), inv_m, -k_ba * LDS(XA, f));
+                __syncthreads();
+            }
+            float s = 0.f;
+            for (int f = 0; f < ec; ++f) s += LDS(X, f) * Wi[f] + LDS_AT(X, f, jl) * Wj[f];
+            const float c = oa * s;
+            if (inverse) {
+                for (int f = 0; f < ec; ++f) {
+                    float F, dF;
+                    act_fd(A.activation, fmaf(alpha, LDS(X, f), c * LDS_AT(X, f, jl)), F, dF);
+                    LDS(XA, f) = fmaf(LDS(XA, f), inv_m, -k_ba * F);
+                }
+            } else {
+                for (int f = 0; f < ec; ++f) {
+                    const float xj = LDS_AT(X, f, jl), xv = LDS(X, f);
+                    float F, dF;
+                    act_fd(A.activation, fmaf(alpha, xv, c * xj), F, dF);
+                    const float a2 = fmaf(m, LDS(XA, f), om * F);
+                    __syncthreads();  // every lane has read the pivot row's feature f
+                    LDS(XA, f) = a2;
+                    LDS(X, f) = fmaf(m, xv, om * a2);
+                }
+            }
+            __syncthreads();
+        }
+        if (L.valid) {
+            for (int f = 0; f < ec; ++f) {
+                store_elem(A.out0, A.out_dtype, L.off + f, LDS(X, f));
+                store_elem(A.out1, A.out_dtype, L.off + f, LDS(XA, f));
+                if (A.aux0) {
+                    A.aux0[L.off + f] = LDS(X, f);
+                    A.aux1[L.off + f] = LDS(XA, f);
+                }
+            }
+        }
+        __syncthreads();
+    }
+}
+
+__global__ void __launch_bounds__(64) generic_backward_kernel(const StageArgs A) {
+    extern __shared__ float lds[];
+    const int lane = threadIdx.x, head = blockIdx.y, ec = A.head_dim, n = A.n_cache;
+    const float alpha = A.alpha, m = A.m, om = 1.f - A.m, oa = 1.f - A.alpha;
+    const float inv_m = 1.f / m, k_ba = om / m, k1 = om * om, k2 = om, kh1 = m * om;
+    const float* Wi = A.W + (int64_t)head * ec;
+    const float* Wj = Wi + A.E;
+    enum { X = 0, XA = 1, G = 2, H = 3, U = 4, DWI = 5, DWJ = 6 };
+    for (int f = 0; f < ec; ++f) LDS(DWI, f) = LDS(DWJ, f) = 0.f;
+    for (uint32_t t = blockIdx.x; t < A.total_tiles; t += gridDim.x) {
+        const GenericLane L = generic_lane(A, t, lane, head);
+        for (int f = 0; f < ec; ++f) {
+            LDS(X, f) = L.valid ? load_elem(A.in0, A.in_dtype, L.off + f) : 0.f;
+            LDS(XA, f) = L.valid ? load_elem(A.in1, A.in_dtype, L.off + f) : 0.f;
+            LDS(G, f) = L.valid ? load_elem(A.g0, A.g_dtype, L.off + f) : 0.f;
+            LDS(H, f) = (L.valid && A.g1) ? load_elem(A.g1, A.g_dtype, L.off + f) : 0.f;
+        }
+        __syncthreads();
+        for (int j = n - 1; j >= 0; --j) {
+            const int jl = L.valid ? L.base + j : lane;
+            for (int f = 0; f < ec; ++f) LDS(X, f) = fmaf(LDS(X, f), inv_m, -k_ba * LDS(XA, f));
+            __syncthreads();
+            float s = 0.f;
+            for (int f = 0; f < ec; ++f) s += LDS(X, f) * Wi[f] + LDS_AT(X, f, jl) * Wj[f];
+            const float c = oa * s;
+            float r = 0.f;
+            for (int f = 0; f < ec; ++f) {
+                const float xj = LDS_AT(X, f, jl);
+                float F, dF;
+                act_fd(A.activation, fmaf(alpha, LDS(X, f), c * xj), F, dF);
+                LDS(XA, f) = fmaf(LDS(XA, f), inv_m, -k_ba * F);
+                const float u = fmaf(k1, LDS(G, f), k2 * LDS(H, f)) * dF;
+                LDS(U, f) = u;
+                r = fmaf(u, xj, r);
+            }
+            const float cr = oa * r;
+            for (int f = 0; f < ec; ++f) {
+                const float xj = LDS_AT(X, f, jl), u = LDS(U, f), g = LDS(G, f);
+                LDS(DWI, f) = fmaf(r, LDS(X, f), LDS(DWI, f));
+                LDS(DWJ, f) = fmaf(r, xj, LDS(DWJ, f));
+                LDS(G, f) = fmaf(m, g, fmaf(alpha, u, cr * Wi[f]));
+                LDS(H, f) = fmaf(kh1, g, m * LDS(H, f));
+                LDS(U, f) = fmaf(cr, Wj[f], c * u);  // this row's share of the pivot row's gradient
+            }
+            __syncthreads();
+            if (L.valid && L.row == j) {
+                for (int f = 0; f < ec; ++f) {
+                    float v = 0.f;
+                    for (int k = 0; k < n; ++k) v += LDS_AT(U, f, L.base + k);
+                    LDS(G, f) += v;
+                }
+            }
+            __syncthreads();
+        }
+        if (L.valid) {
+            for (int f = 0; f < ec; ++f) {
+                store_elem(A.out0, A.out_dtype, L.off + f, LDS(G, f));
+                store_elem(A.out1, A.out_dtype, L.off + f, LDS(H, f));
+                if (A.aux0) {
+                    A.aux0[L.off + f] = LDS(X, f);
+                    A.aux1[L.off + f] = LDS(XA, f);
+                }
+            }
+        }
+        __syncthreads();
+    }
+    // one partial row per block: sum the 64 lanes' accumulators
+    for (int k = lane; k < 2 * ec; k += 64) {
+        const int half = k / ec, f = k - half * ec;
+        float sum = 0.f;
+        for (int l = 0; l < 64; ++l) sum += LDS_AT(half ? DWJ : DWI, f, l);
+        A.dw_partials[(int64_t)blockIdx.x * (2 * A.E) + (int64_t)half * A.E + (int64_t)head * ec + f] = oa * sum;
+    }
+}
+
+// dW[col] = sum over rows of partials[row][col].  64 columns x 4 row lanes per block.
+__global__ void __launch_bounds__(256) reduce_dw_kernel(const float* __restrict__ partials, int rows, int64_t cols,
+                                                        float* __restrict__ dW) {
+    __shared__ float red[4][64];
+    const int cx = threadIdx.x & 63, ry = threadIdx.x >> 6;
+    const int64_t col = (int64_t)blockIdx.x * 64 + cx;
+    float sum = 0.f;
+    if (col < cols)
+        for (int r = ry; r < rows; r += 4) sum += partials[(int64_t)r * cols + col];
+    red[ry][cx] = sum;
+    __syncthreads();
+    if (ry == 0 && col < cols) dW[col] = (red[0][cx] + red[1][cx]) + (red[2][cx] + red[3][cx]);
+}
+
+}  // namespace
+
+hipError_t launch_generic(Pass pass, const StageArgs& a, int n_head, int grid_x, hipStream_t s) {
+    const int arrays = (pass == kBackward) ? kGenericArrays : 2;
+    const size_t lds_bytes = (size_t)arrays * a.head_dim * 64 * sizeof(float);
+    const dim3 grid(grid_x, n_head), block(64);
+    hipError_t err;
+    if (pass == kBackward) {
+        err = hipFuncSetAttribute(reinterpret_cast<const void*>(generic_backward_kernel),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if (err != hipSuccess) return err;
+        hipLaunchKernelGGL(generic_backward_kernel, grid, block, lds_bytes, s, a);
+    } else {
+        err = hipFuncSetAttribute(reinterpret_cast<const void*>(generic_forward_kernel),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if (err != hipSuccess) return err;
+        hipLaunchKernelGGL(generic_forward_kernel, grid, block, lds_bytes, s, a, pass == kInverse ? 1 : 0);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_reduce_dw(const float* partials, int rows, int64_t cols, float* dW, hipStream_t s) {
+    const dim3 grid((unsigned)((cols + 63) / 64)), block(256);
+    hipLaunchKernelGGL(reduce_dw_kernel, grid, block, 0, s, partials, rows, cols, dW);
+    return hipGetLastError();
+}
+
+}  // namespace ncn

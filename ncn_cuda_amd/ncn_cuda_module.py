@@ -1,0 +1,196 @@
+"""Tensor-level entry points with the signatures of the reference's pybind11 module.
+
+The reference builds `ncn_cuda_module` from ncn_cuda/ncn_cuda.cpp:29-32 and exposes
+
+    forward(X, Xa, W, alpha, activation, cache_dim, nhead, module_l)            -> [Y, Ya]
+    backward(Y, Ya, dY, dYa, W, alpha, activation, cache_dim, nhead, module_l)  -> [X, Xa, dX, dXa, dW]
+
+This module offers the same two callables (plus `inverse` and the multi-stage variants) on top of
+libncn_hip.so.  Tensors are allocated here with torch.empty; the library itself never allocates.
+Deviations from the reference module, all visible in the signatures or return values:
+  * `dW` comes back already summed over batch and positions, shaped [1, 1, 2E], so that the
+    reference wrapper's `torch.sum(dW, dim=(0, 1))` (ncn_pytorch_wrapper_v2.py:48) still yields
+    the [2E] gradient (the reference returns per-row partials [batch, N, 2E]);
+  * float32 and bfloat16 activations are accepted (reference: float32 only); W may be either and is
+    used as float32;
+  * launches go to the current PyTorch stream and do not synchronise the host;
+  * invalid arguments raise ValueError/TypeError instead of reading out of bounds.
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+
+M_DEFAULT = 0.9  # hard-coded by the reference: ncn_fwd_cuda_kernel.cu:72, ncn_pytorch.py:89
+
+_DTYPES = {torch.float32: _lib.NCN_F32, torch.bfloat16: _lib.NCN_BF16}
+_ACT_CODES = (_lib.ACT_TANH, _lib.ACT_RELU, _lib.ACT_SIGMOID, _lib.ACT_LINEAR)
+
+
+def validate(x, xa, W, n_cache, n_head, activation, module_l=0, n_stages=1, what="x"):
+    """Host-side argument checks (no GPU needed).  Raises TypeError / ValueError."""
+    if not (isinstance(x, torch.Tensor) and isinstance(xa, torch.Tensor) and isinstance(W, torch.Tensor)):
+        raise TypeError("x, xa and W must be torch tensors")
+    if x.dim() != 3:
+        raise ValueError(f"{what} must be [batch, N, E], got shape {tuple(x.shape)}")
+    if xa.shape != x.shape:
+        raise ValueError(f"{what} and its companion must have the same shape, got {tuple(x.shape)} and {tuple(xa.shape)}")
+    if x.dtype not in _DTYPES or xa.dtype != x.dtype:
+        raise TypeError(f"activations must both be float32 or bfloat16, got {x.dtype} and {xa.dtype}")
+    if W.dtype not in _DTYPES:
+        raise TypeError(f"W must be float32 or bfloat16, got {W.dtype}")
+    batch, N, E = x.shape
+    n_cache, n_head, module_l, n_stages = int(n_cache), int(n_head), int(module_l), int(n_stages)
+    if batch <= 0 or N <= 0 or E <= 0:
+        raise ValueError(f"empty tensor of shape {tuple(x.shape)}")
+    if n_cache <= 0 or N % n_cache != 0:
+        raise ValueError(f"block_size must divide N (N={N}, n_cache={n_cache})")
+    if n_head <= 0 or E % n_head != 0:
+        raise ValueError(f"n_head must divide E (E={E}, n_head={n_head})")
+    if module_l < 0 or n_stages < 1:
+        raise ValueError(f"bad stage range: first stage {module_l}, {n_stages} stages")
+    if W.numel() != n_stages * 2 * E:
+        raise ValueError(f"W must hold {n_stages} x 2E = {n_stages * 2 * E} values, got {W.numel()}")
+    if int(activation) not in _ACT_CODES:
+        raise ValueError(f"unknown activation code {activation} (0 tanh, 1 relu, 2 sigmoid, -1 linear)")
+    shape = _lib.NcnShape(batch, N, E, n_head, n_cache)
+    rc = _lib.load().ncn_check_shape(ctypes.byref(shape), module_l, n_stages, int(activation))
+    if rc != 0:
+        raise ValueError(f"unsupported NCN problem {tuple(x.shape)}, n_cache={n_cache}, n_head={n_head}: "
+                         f"{_lib.error_string(rc)}")
+    return shape
+
+
+def _require_gpu(*tensors):
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError("the NCN kernels run on the GPU only: got a CPU tensor (there is no CPU fallback)")
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise RuntimeError(f"all tensors must live on one device, got {dev} and {t.device}")
+    return dev
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+def _prep(t):
+    """Contiguous, 16-byte aligned view or copy."""
+    t = t.contiguous()
+    if t.data_ptr() % 16 != 0:
+        t = t.clone(memory_format=torch.contiguous_format)
+    return t
+
+
+def _w32(W):
+    return _prep(W.detach().reshape(-1).to(torch.float32))
+
+
+def _stream(dev):
+    return ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+
+def forward_stages(x, xa, W, alpha, activation, cache_dim, nhead, first_stage, n_stages, *, m=M_DEFAULT,
+                   out_dtype=None, save_fp32=False, out=None):
+    """Stages first_stage .. first_stage+n_stages-1 in one call.  W: [n_stages, 2E] (any shape with that many
+    values).  Returns (y, ya) or, with save_fp32, (y, ya, y32, ya32) where y32/ya32 are float32 copies."""
+    shape = validate(x, xa, W, cache_dim, nhead, activation, first_stage, n_stages)
+    dev = _require_gpu(x, xa, W)
+    x, xa, w = _prep(x.detach()), _prep(xa.detach()), _w32(W)
+    out_dtype = x.dtype if out_dtype is None else out_dtype
+    if out is not None:
+        y, ya = out
+    else:
+        y = torch.empty(x.shape, dtype=out_dtype, device=dev)
+        ya = torch.empty(x.shape, dtype=out_dtype, device=dev)
+    y32 = ya32 = None
+    if save_fp32:
+        if out_dtype == torch.float32:
+            y32, ya32 = y, ya
+        else:
+            y32 = torch.empty(x.shape, dtype=torch.float32, device=dev)
+            ya32 = torch.empty(x.shape, dtype=torch.float32, device=dev)
+    aux = (y32, ya32) if (save_fp32 and out_dtype != torch.float32) else (None, None)
+    with torch.cuda.device(dev):
+        rc = _lib.load().ncn_forward(_ptr(x), _ptr(xa), _DTYPES[x.dtype], _ptr(y), _ptr(ya), _DTYPES[out_dtype],
+                                     _ptr(aux[0]), _ptr(aux[1]), _ptr(w), ctypes.byref(shape),
+                                     int(first_stage), int(n_stages), float(alpha), float(m), int(activation),
+                                     _stream(dev))
+    _lib.check(rc, "ncn_forward")
+    return (y, ya, y32, ya32) if save_fp32 else (y, ya)
+
+
+def backward_stages(y, ya, dy, dya, W, alpha, activation, cache_dim, nhead, first_stage, n_stages, *, m=M_DEFAULT,
+                    grad_dtype=None, want_inputs=True):
+    """Reversible backward of stages first_stage+n_stages-1 .. first_stage from the outputs y, ya of the last one.
+    dya may be None (zeros).  Returns (x_rec, xa_rec, dx, dxa, dW[n_stages, 2E]); x_rec/xa_rec are None when
+    want_inputs is False and n_stages == 1."""
+    shape = validate(y, ya, W, cache_dim, nhead, activation, first_stage, n_stages, what="y")
+    if dy.shape != y.shape or (dya is not None and dya.shape != y.shape):
+        raise ValueError("dy/dya must have the shape of y")
+    if dy.dtype not in _DTYPES or (dya is not None and dya.dtype != dy.dtype):
+        raise TypeError("dy and dya must both be float32 or bfloat16")
+    dev = _require_gpu(y, ya, dy, dya, W)
+    y, ya, dy, w = _prep(y.detach()), _prep(ya.detach()), _prep(dy.detach()), _w32(W)
+    dya = _prep(dya.detach()) if dya is not None else None
+    grad_dtype = dy.dtype if grad_dtype is None else grad_dtype
+    need_state = want_inputs or n_stages > 1
+    if n_stages > 1 and grad_dtype != torch.float32:
+        raise ValueError("multi-stage backward carries its state in float32: use grad_dtype=torch.float32")
+    dx = torch.empty(y.shape, dtype=grad_dtype, device=dev)
+    dxa = torch.empty(y.shape, dtype=grad_dtype, device=dev)
+    x_rec = torch.empty(y.shape, dtype=torch.float32, device=dev) if need_state else None
+    xa_rec = torch.empty(y.shape, dtype=torch.float32, device=dev) if need_state else None
+    E = y.shape[2]
+    dW = torch.empty(n_stages, 2 * E, dtype=torch.float32, device=dev)
+    lib = _lib.load()
+    ws_bytes = lib.ncn_workspace_bytes(ctypes.byref(shape))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        rc = lib.ncn_backward(_ptr(y), _ptr(ya), _DTYPES[y.dtype], _ptr(dy), _ptr(dya), _DTYPES[dy.dtype],
+                              _ptr(dx), _ptr(dxa), _DTYPES[grad_dtype], _ptr(x_rec), _ptr(xa_rec), _ptr(w), _ptr(dW),
+                              _ptr(ws), ctypes.c_size_t(ws_bytes), ctypes.byref(shape), int(first_stage),
+                              int(n_stages), float(alpha), float(m), int(activation), _stream(dev))
+    _lib.check(rc, "ncn_backward")
+    return x_rec, xa_rec, dx, dxa, dW
+
+
+def inverse_stages(y, ya, W, alpha, activation, cache_dim, nhead, first_stage, n_stages, *, m=M_DEFAULT,
+                   out_dtype=None):
+    """x, xa with forward_stages(x, xa, ...) == (y, ya)."""
+    shape = validate(y, ya, W, cache_dim, nhead, activation, first_stage, n_stages, what="y")
+    dev = _require_gpu(y, ya, W)
+    y, ya, w = _prep(y.detach()), _prep(ya.detach()), _w32(W)
+    out_dtype = y.dtype if out_dtype is None else out_dtype
+    x = torch.empty(y.shape, dtype=out_dtype, device=dev)
+    xa = torch.empty(y.shape, dtype=out_dtype, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.load().ncn_inverse(_ptr(y), _ptr(ya), _DTYPES[y.dtype], _ptr(x), _ptr(xa), _DTYPES[out_dtype],
+                                     _ptr(w), ctypes.byref(shape), int(first_stage), int(n_stages), float(alpha),
+                                     float(m), int(activation), _stream(dev))
+    _lib.check(rc, "ncn_inverse")
+    return x, xa
+
+
+# ---- the reference module's two callables (ncn_cuda/ncn_cuda.cpp:3-25) -------------------------------------
+def forward(X, Xa, W, alpha, activation, cache_dim, nhead, module_l):
+    y, ya = forward_stages(X, Xa, W, alpha, activation, cache_dim, nhead, module_l, 1)
+    return [y, ya]
+
+
+def backward(Y, Ya, dY, dYa, W, alpha, activation, cache_dim, nhead, module_l):
+    x, xa, dx, dxa, dW = backward_stages(Y, Ya, dY, dYa, W, alpha, activation, cache_dim, nhead, module_l, 1)
+    return [x, xa, dx, dxa, dW.reshape(1, 1, -1)]
+
+
+def inverse(Y, Ya, W, alpha, activation, cache_dim, nhead, module_l):
+    """Inputs of stage module_l from its outputs (NCNFunctionPytorch.invert,
+    torch_ref/ncn_pytorch_invertible.py:87-113, applied for j = cache_dim-1 .. 0)."""
+    x, xa = inverse_stages(Y, Ya, W, alpha, activation, cache_dim, nhead, module_l, 1)
+    return [x, xa]

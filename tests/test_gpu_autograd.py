@@ -1,0 +1,87 @@
+"""The reference's autograd / nn.Module surface on the GPU: same names, same call pattern as
+grad_test_bench.py:116-134, results against the CPU oracle."""
+import pytest
+import torch
+
+from oracle import ncn_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def pkg():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    import ncn_cuda_amd
+    return ncn_cuda_amd
+
+
+def test_net_test_cuda_like_reference_script(pkg):
+    # the reference script's own configuration, grad_test_bench.py:22-32
+    batch, n_head, N, E, alpha, n, L = 4, 4, 256, 128, 0.9, 32, 3
+    g = torch.Generator().manual_seed(0)
+    x = (0.5 * torch.randn(batch, N, E, generator=g))
+    xa = torch.zeros(batch, N, E)
+    Ws = [0.5 * torch.randn(2 * E, generator=g) for _ in range(L)]
+    dyi = torch.randn(batch, N, E, generator=g)
+    d = torch.float64
+    ref_yi, ref_ya, ref_dx, ref_dxa, ref_dWs = O.net_autograd(x.to(d), xa.to(d), [w.to(d) for w in Ws], dyi.to(d),
+                                                              torch.zeros_like(dyi, dtype=d), alpha, n, n_head)
+    gx = x.cuda().requires_grad_()
+    gxa = xa.cuda().requires_grad_()
+    gWs = [w.cuda().requires_grad_() for w in Ws]
+    net = pkg.NCNNetTestCuda(alpha, "tanh", n, n_head, L, gWs)
+    yi, ya = net(gx, gxa)
+    yi.backward(dyi.cuda())
+    assert O.rel_err(yi, ref_yi) < 1e-5
+    assert O.rel_err(ya, ref_ya) < 1e-5
+    # n_cache = 32 amplifies inversion rounding by (1/0.9)^32 = 29: the reference's own check uses atol=1e-2
+    # (grad_test_bench.py:161); float32 still lands near 1e-5 relative
+    assert O.rel_err(gx.grad, ref_dx) < 3e-5
+    assert O.rel_err(gxa.grad, ref_dxa) < 3e-5
+    for l in range(L):
+        assert O.rel_err(gWs[l].grad, ref_dWs[l]) < 3e-5
+
+
+def test_net_cuda_module_list_and_state_dict(pkg):
+    alpha, n, C, L, E = 0.9, 4, 4, 3, 32
+    torch.manual_seed(0)
+    net = pkg.NCNNetCuda(alpha, "tanh", n, C, L, E).cuda()
+    assert sorted(net.state_dict().keys()) == [f"ncn_modules.{l}.weight" for l in range(L)]
+    with torch.no_grad():
+        for mod in net.ncn_modules:
+            mod.weight.normal_(0, 0.5)
+    x = torch.randn(2, 64, E, device="cuda", requires_grad=True)
+    xa = torch.randn(2, 64, E, device="cuda", requires_grad=True)
+    yi, ya = net(x, xa)
+    (yi.sum() + 2 * ya.sum()).backward()
+    d = torch.float64
+    Ws = [mod.weight.detach().cpu().to(d) for mod in net.ncn_modules]
+    ones = torch.ones(2, 64, E, dtype=d)
+    ref_yi, ref_ya, ref_dx, ref_dxa, ref_dWs = O.net_autograd(x.detach().cpu().to(d), xa.detach().cpu().to(d), Ws,
+                                                              ones, 2 * ones, alpha, n, C)
+    assert O.rel_err(yi, ref_yi) < 1e-5
+    assert O.rel_err(x.grad, ref_dx) < 1e-5
+    assert O.rel_err(xa.grad, ref_dxa) < 1e-5
+    for l in range(L):
+        assert O.rel_err(net.ncn_modules[l].weight.grad, ref_dWs[l]) < 1e-5
+
+
+def test_bf16_autograd(pkg):
+    batch, N, E, C, n, L, alpha = 2, 128, 128, 4, 16, 3, 0.9
+    x, xa, Ws, dyi, dya = O.make_inputs(batch, N, E, L, n, seed=4, xa_zero=True, dtype=torch.bfloat16)
+    f = torch.float32
+    ref_yi, ref_ya, ref_dx, ref_dxa, ref_dWs = O.net_autograd(x.to(f), xa.to(f), [w.to(f) for w in Ws], dyi.to(f),
+                                                              dya.to(f), alpha, n, C)
+    gx, gxa = x.cuda().requires_grad_(), xa.cuda().requires_grad_()
+    gWs = [w.cuda().requires_grad_() for w in Ws]
+    net = pkg.NCNNetTestCuda(alpha, "tanh", n, C, L, gWs)
+    yi, ya = net(gx, gxa)
+    assert yi.dtype == torch.bfloat16
+    torch.autograd.backward([yi, ya], [dyi.cuda(), dya.cuda()])
+    assert O.rel_err(yi, ref_yi) < 2e-2
+    assert O.rel_err(gx.grad, ref_dx) < 2e-2
+    assert O.rel_err(gxa.grad, ref_dxa) < 2e-2
+    for l in range(L):
+        assert gWs[l].grad.dtype == torch.bfloat16
+        assert O.rel_err(gWs[l].grad, ref_dWs[l]) < 2e-2

@@ -1,0 +1,210 @@
+"""Parity of the HIP path with the CPU oracle and with the reference's golden vectors.
+
+Every call goes through the C ABI of libncn_hip.so (ctypes, via ncn_cuda_amd.ncn_cuda_module).
+Tolerances: float32 1e-5 relative (max |diff| / max |ref|), bfloat16 storage with float32
+arithmetic 2e-2 relative; integer work (the index map) is exact by construction of the outputs.
+"""
+import pytest
+import torch
+
+from conftest import GOLDEN_CASES, load_golden
+from oracle import ncn_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+TOL_F32 = 1e-5
+TOL_BF16 = 2e-2
+
+
+@pytest.fixture(scope="module")
+def M():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from ncn_cuda_amd import ncn_cuda_module
+    return ncn_cuda_module
+
+
+def _dev(*ts):
+    return [t.cuda() if t is not None else None for t in ts]
+
+
+def _stack_forward(M, x, xa, Ws, alpha, n, C, act=0):
+    outs = []
+    for l, W in enumerate(Ws):
+        x, xa = M.forward(x, xa, W, alpha, act, n, C, l)
+        outs.append((x, xa))
+    return outs
+
+
+def _stack_backward(M, outs, dy, dya, Ws, alpha, n, C, act=0):
+    dWs = [None] * len(Ws)
+    for l in range(len(Ws) - 1, -1, -1):
+        y, ya = outs[l]
+        xr, xar, dy, dya, dW = M.backward(y, ya, dy, dya, Ws[l], alpha, act, n, C, l)
+        dWs[l] = dW.reshape(-1)
+    return xr, xar, dy, dya, dWs
+
+
+@pytest.mark.parametrize("name", GOLDEN_CASES)
+def test_golden_forward_backward(M, name):
+    """Reference vectors (float64 run of torch_ref) vs the GPU in float32, per-stage saved outputs."""
+    g = load_golden(name)
+    mt = g["meta"]
+    n, C, L, alpha = mt["n"], mt["C"], mt["L"], g["alpha"]
+    x, xa, dyi, dya = _dev(g["x"], g["xa"], g["dyi"], g["dya"])
+    Ws = _dev(*[g[f"W{l}"] for l in range(L)])
+    outs = _stack_forward(M, x, xa, Ws, alpha, n, C)
+    assert O.rel_err(outs[-1][0], g["ref_f64_yi"]) < TOL_F32
+    assert O.rel_err(outs[-1][1], g["ref_f64_ya"]) < TOL_F32
+    xr, xar, dx, dxa, dWs = _stack_backward(M, outs, dyi, dya, Ws, alpha, n, C)
+    assert O.rel_err(dx, g["ref_f64_dx"]) < TOL_F32
+    assert O.rel_err(dxa, g["ref_f64_dxa"]) < TOL_F32
+    for l in range(L):
+        assert O.rel_err(dWs[l], g[f"ref_f64_dW{l}"]) < TOL_F32, f"dW{l}"
+    # reconstruction of the stack input by the last inversion
+    assert O.rel_err(xr, g["x"]) < TOL_F32
+    assert (xar.cpu() - g["xa"]).abs().max().item() < TOL_F32 * max(1.0, g["x"].abs().max().item())
+
+
+# (batch, N, E, C, n, L): every register-kernel head width and group size, ragged tails, the generic kernel
+SHAPES = [
+    (3, 64, 16, 4, 2, 4),      # Ec=4
+    (2, 96, 32, 4, 4, 3),      # Ec=8, groups=24 (not a power of two)
+    (2, 128, 64, 4, 8, 5),     # Ec=16
+    (2, 256, 128, 4, 16, 3),   # Ec=32, n=16: the headline tile
+    (1, 256, 128, 4, 32, 3),   # the reference script's shape family (n_cache == Ec == 32)
+    (2, 64, 128, 2, 4, 4),     # Ec=64
+    (5, 40, 32, 1, 2, 3),      # Ec=32, one head, 20 groups: partial wave tile
+    (2, 64, 64, 4, 16, 6),     # stride wraps to 0 again (L > log2(groups)+1)
+    (2, 36, 20, 2, 3, 3),      # generic kernel: n=3, Ec=10
+    (1, 128, 6, 2, 64, 2),     # generic kernel: n=64, Ec=3
+    (2, 14, 12, 4, 1, 2),      # generic kernel: n=1
+]
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "b%d_N%d_E%d_C%d_n%d_L%d" % s)
+def test_forward_backward_inverse_vs_oracle(M, shape):
+    batch, N, E, C, n, L = shape
+    alpha = 0.9
+    x, xa, Ws, dyi, dya = O.make_inputs(batch, N, E, L, n, seed=11, xa_zero=False)
+    d = torch.float64
+    ref_yi, ref_ya, ref_dx, ref_dxa, ref_dWs = O.net_autograd(x.to(d), xa.to(d), [w.to(d) for w in Ws],
+                                                              dyi.to(d), dya.to(d), alpha, n, C)
+    gx, gxa, gdyi, gdya = _dev(x, xa, dyi, dya)
+    gWs = _dev(*Ws)
+    outs = _stack_forward(M, gx, gxa, gWs, alpha, n, C)
+    assert O.rel_err(outs[-1][0], ref_yi) < TOL_F32
+    assert O.rel_err(outs[-1][1], ref_ya) < TOL_F32
+    # the reversible backward divides by m at each of the n steps of a stage: float32 rounding grows like
+    # (1/m)^n (5x at n = 16, 29x at n = 32, 850x at n = 64), which only matters above n = 16
+    tol_inv = max(TOL_F32, 3e-6 * (1 / 0.9) ** n)
+    tol_bwd = TOL_F32 if n <= 32 else tol_inv
+    xr, xar, dx, dxa, dWs = _stack_backward(M, outs, gdyi, gdya, gWs, alpha, n, C)
+    assert O.rel_err(dx, ref_dx) < tol_bwd
+    assert O.rel_err(dxa, ref_dxa) < tol_bwd
+    for l in range(L):
+        assert O.rel_err(dWs[l], ref_dWs[l]) < tol_bwd, f"dW{l}"
+    # stand-alone inverse of the last stage reproduces the previous stage's output
+    prev = outs[-2] if L > 1 else (gx, gxa)
+    ix, ixa = M.inverse(outs[-1][0], outs[-1][1], gWs[-1], alpha, 0, n, C, L - 1)
+    assert O.rel_err(ix, prev[0]) < tol_inv
+    assert O.rel_err(ixa, prev[1]) < tol_inv
+
+
+def test_multi_stage_calls_match_single_stage_calls(M):
+    batch, N, E, C, n, L = 2, 128, 64, 2, 8, 3
+    alpha = 0.8
+    x, xa, Ws, dyi, dya = O.make_inputs(batch, N, E, L, n, seed=5, xa_zero=False)
+    gx, gxa, gdyi, gdya = _dev(x, xa, dyi, dya)
+    gWs = _dev(*Ws)
+    Wst = torch.stack(gWs)
+    outs = _stack_forward(M, gx, gxa, gWs, alpha, n, C)
+    y, ya = M.forward_stages(gx, gxa, Wst, alpha, 0, n, C, 0, L)
+    assert torch.equal(y, outs[-1][0]) and torch.equal(ya, outs[-1][1])
+    # whole-stack reversible backward (state carried in place) against the float64 oracle
+    d = torch.float64
+    _, _, ref_dx, ref_dxa, ref_dWs = O.net_autograd(x.to(d), xa.to(d), [w.to(d) for w in Ws], dyi.to(d), dya.to(d),
+                                                    alpha, n, C)
+    xr, xar, dx, dxa, dW = M.backward_stages(y, ya, gdyi, gdya, Wst, alpha, 0, n, C, 0, L)
+    amp = (1 / 0.9) ** (n * L)
+    assert O.rel_err(dx, ref_dx) < 5e-7 * amp
+    assert O.rel_err(dxa, ref_dxa) < 5e-7 * amp
+    for l in range(L):
+        assert O.rel_err(dW[l], ref_dWs[l]) < 5e-7 * amp
+    assert O.rel_err(xr, x) < 5e-7 * amp
+    ix, ixa = M.inverse_stages(y, ya, Wst, alpha, 0, n, C, 0, L)
+    assert O.rel_err(ix, x) < 5e-7 * amp
+    assert torch.equal(ix, xr)
+
+
+def test_dya_none_equals_zeros(M):
+    batch, N, E, C, n = 2, 64, 32, 4, 4
+    x, xa, Ws, dyi, _ = O.make_inputs(batch, N, E, 1, n, seed=3)
+    gx, gxa, gdyi, gW = _dev(x, xa, dyi, Ws[0])
+    y, ya = M.forward(gx, gxa, gW, 0.9, 0, n, C, 1)
+    a = M.backward_stages(y, ya, gdyi, None, gW, 0.9, 0, n, C, 1, 1)
+    b = M.backward_stages(y, ya, gdyi, torch.zeros_like(gdyi), gW, 0.9, 0, n, C, 1, 1)
+    for u, v in zip(a, b):
+        assert torch.equal(u, v)
+
+
+@pytest.mark.parametrize("act", [1, 2, -1], ids=["relu", "sigmoid", "linear"])
+def test_other_activations_vs_oracle(M, act):
+    """relu / sigmoid / linear run on the generic kernel; the oracle for them is pinned by autograd only."""
+    batch, N, E, C, n, L = 2, 32, 16, 2, 4, 3
+    alpha = 0.9
+    x, xa, Ws, dyi, dya = O.make_inputs(batch, N, E, L, n, seed=21, xa_zero=False)
+    d = torch.float64
+    ref_yi, ref_ya, ref_dx, ref_dxa, ref_dWs = O.net_autograd(x.to(d), xa.to(d), [w.to(d) for w in Ws], dyi.to(d),
+                                                              dya.to(d), alpha, n, C, activation=act)
+    gx, gxa, gdyi, gdya = _dev(x, xa, dyi, dya)
+    gWs = _dev(*Ws)
+    outs = _stack_forward(M, gx, gxa, gWs, alpha, n, C, act)
+    assert O.rel_err(outs[-1][0], ref_yi) < TOL_F32
+    assert O.rel_err(outs[-1][1], ref_ya) < TOL_F32
+    if act == 1:
+        return  # relu's kink makes the reversible recomputation flip F' for |T| ~ eps: gradients not compared
+    _, _, dx, dxa, dWs = _stack_backward(M, outs, gdyi, gdya, gWs, alpha, n, C, act)
+    assert O.rel_err(dx, ref_dx) < TOL_F32
+    assert O.rel_err(dxa, ref_dxa) < TOL_F32
+    for l in range(L):
+        assert O.rel_err(dWs[l], ref_dWs[l]) < TOL_F32
+
+
+def test_bf16_storage_fp32_arithmetic(M):
+    """bf16 activations and weights, float32 arithmetic: compared with the oracle run in float32 on the
+    same bf16-rounded inputs.  Tolerance 2e-2 relative."""
+    batch, N, E, C, n, L = 4, 256, 128, 4, 16, 3
+    alpha = 0.9
+    x, xa, Ws, dyi, dya = O.make_inputs(batch, N, E, L, n, seed=0, xa_zero=True, dtype=torch.bfloat16)
+    f = torch.float32
+    ref_yi, ref_ya, ref_dx, ref_dxa, ref_dWs = O.net_autograd(x.to(f), xa.to(f), [w.to(f) for w in Ws], dyi.to(f),
+                                                              dya.to(f), alpha, n, C)
+    gx, gxa, gdyi, gdya = _dev(x, xa, dyi, dya)
+    gWs = _dev(*Ws)
+    saved = []
+    cx, cxa = gx, gxa
+    for l in range(L):
+        cx, cxa, y32, ya32 = M.forward_stages(cx, cxa, gWs[l], alpha, 0, n, C, l, 1, save_fp32=True)
+        assert cx.dtype == torch.bfloat16 and y32.dtype == torch.float32
+        saved.append((y32, ya32))
+    assert O.rel_err(cx, ref_yi) < TOL_BF16
+    assert O.rel_err(cxa, ref_ya) < TOL_BF16
+    dy, dya_ = gdyi, gdya
+    for l in range(L - 1, -1, -1):
+        _, _, dy, dya_, dW = M.backward_stages(saved[l][0], saved[l][1], dy, dya_, gWs[l], alpha, 0, n, C, l, 1,
+                                               grad_dtype=torch.bfloat16, want_inputs=False)
+        assert O.rel_err(dW[0], ref_dWs[l]) < TOL_BF16, f"dW{l}"
+    assert dy.dtype == torch.bfloat16
+    assert O.rel_err(dy, ref_dx) < TOL_BF16
+    assert O.rel_err(dya_, ref_dxa) < TOL_BF16
+
+
+def test_in_place_forward_and_inverse(M):
+    batch, N, E, C, n = 2, 128, 128, 4, 16
+    x, xa, Ws, _, _ = O.make_inputs(batch, N, E, 1, n, seed=9, xa_zero=False)
+    gx, gxa, gW = _dev(x, xa, Ws[0])
+    y, ya = M.forward(gx, gxa, gW, 0.9, 0, n, C, 2)
+    bx, bxa = gx.clone(), gxa.clone()
+    M.forward_stages(bx, bxa, gW, 0.9, 0, n, C, 2, 1, out=(bx, bxa))
+    assert torch.equal(bx, y) and torch.equal(bxa, ya)
