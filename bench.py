@@ -1,0 +1,179 @@
+#!/usr/bin/env python3
+"""Headline benchmark: NCN forward + backward of the full stage stack on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg3|cfg2|cfg4|cfg5] [--no-cpu]
+
+One step = forward of all L stages (each stage saving its outputs, like the reference's autograd
+node) + reversible backward of all L stages producing dx, dxa and every dW_l, on inputs that are
+already resident in HBM.  The default workload is the configuration the metric is quoted on:
+B=16384, D=4096, g=16, bf16 storage / float32 arithmetic, i.e. [batch=128, N=4096, E=128],
+4 heads of 32, n_cache=16, 3 stages.
+
+Prints ONE JSON line.  `roofline` describes the dominant kernel (the backward stage kernel):
+algorithmic bytes of one launch divided by its average duration, measured with HIP events on the
+launch stream inside the timed region.  `cpu_baseline` times the CPU oracle on a bounded batch
+slice of the same workload on the host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+# config label -> (batch, N, E, n_head, n_cache, L, io dtype, w_scale)   (B = batch*E tokens, D = N, g = n_cache)
+CONFIGS = {
+    "cfg2": dict(batch=32, N=1024, E=128, C=4, n=4, L=5, dtype="f32", w_scale=1.0),
+    "cfg3": dict(batch=128, N=4096, E=128, C=4, n=16, L=3, dtype="bf16", w_scale=1.0),
+    "cfg4": dict(batch=128, N=8192, E=128, C=4, n=2, L=13, dtype="f32", w_scale=1.0),
+    "cfg5": dict(batch=64, N=2048, E=128, C=4, n=8, L=4, dtype="f32", w_scale=0.1),
+}
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
+VALU_PEAK_TFLOPS = 157.3   # MI355X FP32 vector peak (packed); 78.6 without packed FP32
+# float32 operations per element-step of the kernels as written (FMA = 2), counted from
+# ncn_stage_kernels.h: forward 13 + exp2 + rcp, backward 41 + exp2 + rcp (+ log2(n) adds of the row sum)
+FLOPS_FWD_PER_ELEM_STEP = 15.0
+FLOPS_BWD_PER_ELEM_STEP = 43.0
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", default="cfg3", choices=sorted(CONFIGS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (the layer shards over batch; "
+              "only dW [L,2E] would need an all-reduce). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from ncn_cuda_amd import ncn_cuda_module as M
+    from oracle import ncn_oracle as O
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    cfg = CONFIGS[args.config]
+    batch, N, E, C, n, L = cfg["batch"], cfg["N"], cfg["E"], cfg["C"], cfg["n"], cfg["L"]
+    io_dtype = torch.bfloat16 if cfg["dtype"] == "bf16" else torch.float32
+    alpha = 0.9
+    tokens = batch * E
+    P = batch * N * E
+    sbytes = 2 if cfg["dtype"] == "bf16" else 4
+
+    x, xa, Ws, dyi, dya = O.make_inputs(batch, N, E, L, n, seed=0, xa_zero=True, w_scale=cfg["w_scale"],
+                                        dtype=io_dtype)
+    dev = torch.device("cuda:0")
+    gx, gxa, gdyi = x.to(dev), xa.to(dev), dyi.to(dev)
+    gWs = [w.to(dev) for w in Ws]
+    bf16 = io_dtype == torch.bfloat16
+
+    def step(events=None):
+        saved = []
+        cx, cxa = gx, gxa
+        for l in range(L):
+            if bf16:
+                cx, cxa, y32, ya32 = M.forward_stages(cx, cxa, gWs[l], alpha, 0, n, C, l, 1, save_fp32=True)
+                saved.append((y32, ya32))
+            else:
+                cx, cxa = M.forward_stages(cx, cxa, gWs[l], alpha, 0, n, C, l, 1)
+                saved.append((cx, cxa))
+        dy, dya_ = gdyi, None  # the reference script back-propagates through yi only (grad_test_bench.py:121)
+        dWs = [None] * L
+        for l in range(L - 1, -1, -1):
+            if events is not None:
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+            _, _, dy, dya_, dWs[l] = M.backward_stages(saved[l][0], saved[l][1], dy, dya_, gWs[l], alpha, 0, n, C, l,
+                                                       1, grad_dtype=io_dtype, want_inputs=False)
+            if events is not None:
+                e1.record()
+                events.append((e0, e1))
+        return cx, cxa, dy, dya_, dWs
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    events = []
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out = step(events)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    value = tokens / (ms_per_step * 1e-3)
+
+    # dominant kernel: backward stage launch (its event bracket also holds the microsecond-scale dW reduce)
+    bwd_ms = sum(e0.elapsed_time(e1) for e0, e1 in events) / len(events)
+    bytes_bwd_launch = 6.0 * P * sbytes            # read y, ya, dy, dya; write dx, dxa
+    achieved = bytes_bwd_launch / (bwd_ms * 1e-3) / 1e9
+    elem_steps_stage = float(P) * n
+    flops_step = (FLOPS_FWD_PER_ELEM_STEP + FLOPS_BWD_PER_ELEM_STEP) * elem_steps_stage * L
+    result = {
+        "metric": "NCN fwd+bwd tokens/sec and achieved HBM GB/s (% roofline), B=16384 D=4096 g=16",
+        "value": value,
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32" if not bf16 else "f32 arithmetic, bf16 storage",
+        "data": "synthetic",
+        "config": {"workload": f"{args.config}: B={tokens} D={N} g={n} -> x[batch={batch},N={N},E={E}], "
+                               f"{C} heads of {E // C}, n_cache={n}, {L} stages, alpha=0.9, m=0.9, tanh, "
+                               f"{cfg['dtype']} storage", "positions_per_s": batch * N / (ms_per_step * 1e-3)},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": f"stage_backward_kernel<{n},{E // C}>", "avg_launch_ms": bwd_ms,
+                     "algorithmic_bytes_per_launch": bytes_bwd_launch},
+        "stack": {"algorithmic_bytes_fused": 10.0 * P * sbytes,
+                  "achieved_GBps_fused_bytes": 10.0 * P * sbytes / (ms_per_step * 1e-3) / 1e9,
+                  "algorithmic_bytes_per_stage_launches": 10.0 * P * sbytes * L,
+                  "achieved_GBps_per_stage_bytes": 10.0 * P * sbytes * L / (ms_per_step * 1e-3) / 1e9,
+                  "fp32_flops_per_step": flops_step,
+                  "achieved_TFLOPs": flops_step / (ms_per_step * 1e-3) / 1e12,
+                  "frac_of_fp32_vector_peak": flops_step / (ms_per_step * 1e-3) / 1e12 / VALU_PEAK_TFLOPS,
+                  "note": "the step is bound by float32 VALU + exp2/rcp issue, not by HBM or MFMA: "
+                          "each element takes n_cache sequential tanh steps per stage"},
+    }
+
+    if not args.no_cpu:
+        ncores = os.cpu_count() or 1
+        threads = min(ncores, 16)
+        torch.set_num_threads(threads)
+        f = torch.float32
+
+        def cpu_run(b):
+            xs, xas, dys = x[:b].to(f), xa[:b].to(f), dyi[:b].to(f)
+            w32 = [w.to(f) for w in Ws]
+            t = time.perf_counter()
+            O.net_backward_checkpointed(xs, xas, dys, torch.zeros_like(dys), w32, alpha, n, C, save_every=1)
+            return time.perf_counter() - t
+
+        probe_b = min(batch, 2)
+        cpu_run(1)
+        tp = cpu_run(probe_b)
+        sample_b = int(max(probe_b, min(batch, round(6.0 / max(tp / probe_b, 1e-6)))))
+        ts = cpu_run(sample_b)
+        cpu_tokens_s = sample_b * E / ts
+        result["cpu_baseline"] = {"value": cpu_tokens_s, "unit": "tokens/s", "cores": threads, "kind": "port",
+                                  "sample": f"first {sample_b} of {batch} batch entries of the same workload "
+                                            f"({sample_b * E} of {tokens} tokens), float32, vectorised PyTorch "
+                                            f"restatement of torch_ref (forward + reversible backward), "
+                                            f"{ts:.1f} s wall",
+                                  "host_cpus_visible": ncores}
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
