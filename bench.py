@@ -33,10 +33,11 @@ CONFIGS = {
 }
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 VALU_PEAK_TFLOPS = 157.3   # MI355X FP32 vector peak (packed); 78.6 without packed FP32
-# float32 operations per element-step of the kernels as written (FMA = 2), counted from
-# ncn_stage_kernels.h: forward 13 + exp2 + rcp, backward 41 + exp2 + rcp (+ log2(n) adds of the row sum)
-FLOPS_FWD_PER_ELEM_STEP = 15.0
-FLOPS_BWD_PER_ELEM_STEP = 43.0
+# float32 operations per element and step of the kernels as written in ncn_stage_kernels.h (FMA = 2, exp2 and
+# rcp = 1 each), without the per-row and per-lane bookkeeping: forward 1 FMA (dot) + 2 (z) + 1 (t+1) + 2 FMA (xa)
+# + 2 (x) + exp2 + rcp = 13; backward 11 FMA + 4 mul/add + exp2 + rcp = 28.
+FLOPS_FWD_PER_ELEM_STEP = 13.0
+FLOPS_BWD_PER_ELEM_STEP = 28.0
 
 
 def main():

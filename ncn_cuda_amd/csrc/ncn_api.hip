@@ -1,6 +1,8 @@
 // C ABI of libncn_hip.so: argument validation, stage sequencing and launches.  See include/ncn_hip.h.
 #include <hip/hip_runtime.h>
 
+#include <cmath>
+
 #include "../../include/ncn_hip.h"
 #include "ncn_launch.h"
 
@@ -18,7 +20,7 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 int kernel_path(const ncn_shape* sh, int activation) {
     if (sh->n_cache < 1 || sh->n_cache > 64) return 0;
     const int64_t ec = sh->E / sh->n_head;
-    if (activation == NCN_ACT_TANH && ec <= 64 && fast_fpl(sh->n_cache, (int)ec) != 0) return 2;
+    if (activation == NCN_ACT_TANH && ec <= 64 && fast_tile(sh->n_cache, (int)ec).r != 0) return 2;
     if (ec <= kGenericMaxHeadDim) return 1;
     return 0;
 }
@@ -79,6 +81,16 @@ void fill_common(StageArgs& a, const ncn_shape* sh, const Plan& p, int stage, fl
     a.activation = activation;
     a.alpha = alpha;
     a.m = m;
+    const double md = m, al = alpha, k2l = 2.8853900817779268;
+    a.m_pow_n = (float)std::pow(md, (double)sh->n_cache);
+    a.inv_m_pow_n = (float)std::pow(md, -(double)sh->n_cache);
+    for (int t = 0; t < 64; ++t) {
+        const double im = std::pow(md, -(double)(t + 1));
+        a.step[t].lam = (float)(k2l * al * im);
+        a.step[t].kc2 = (float)(k2l * (1.0 - al) * im * im);
+        a.step[t].kap = (float)((1.0 - md) * std::pow(md, (double)t));
+        a.step[t].krho = (float)(4.0 * (1.0 - md) / md * (1.0 - al) * im);
+    }
 }
 
 }  // namespace
@@ -117,7 +129,7 @@ int ncn_kernel_path(const ncn_shape* shape) {
 
 size_t ncn_workspace_bytes(const ncn_shape* shape) {
     if (check_shape(shape, 0, 1, NCN_ACT_TANH) != NCN_OK) return 0;
-    return (size_t)kMaxGridX * 2 * (size_t)shape->E * sizeof(float);
+    return (size_t)(kMaxGridX + kReduceLevel1Rows) * 2 * (size_t)shape->E * sizeof(float);
 }
 
 int ncn_forward(const void* x, const void* xa, int in_dtype, void* y, void* ya, int out_dtype, float* y32, float* ya32,
@@ -217,7 +229,8 @@ int ncn_backward(const void* y, const void* ya, int y_dtype, const void* dy, con
         hipError_t err = (p.path == 2) ? launch_fast_backward(a, shape->n_head, p.grid_x, s)
                                        : launch_generic(kBackward, a, shape->n_head, p.grid_x, s);
         if (err != hipSuccess) return (int)err;
-        err = launch_reduce_dw(a.dw_partials, p.grid_x, 2 * shape->E, dW + (int64_t)k * 2 * shape->E, s);
+        err = launch_reduce_dw(a.dw_partials, p.grid_x, 2 * shape->E, a.dw_partials + (int64_t)kMaxGridX * 2 * shape->E,
+                               dW + (int64_t)k * 2 * shape->E, s);
         if (err != hipSuccess) return (int)err;
     }
     return NCN_OK;

@@ -33,6 +33,14 @@ struct StageArgs {
     int32_t in_dtype, g_dtype, out_dtype;
     int32_t activation;
     float alpha, m;
+    float m_pow_n, inv_m_pow_n;  // m^n_cache and its reciprocal
+    // Per-step scalars of the reversible backward, index t = number of inversion steps already done
+    // (t = 0 is the stage's last step).  Computed on the host in double precision:
+    //   im = m^-(t+1),  lam = 2 log2(e) alpha im,  kc2 = 2 log2(e) (1-alpha) im^2,
+    //   kap = (1-m) m^t,  krho = 4 (1-m)/m (1-alpha) im
+    struct StepScalars {
+        float lam, kc2, kap, krho;
+    } step[64];
 };
 
 // ---------------------------------------------------------------------------------------------
@@ -134,9 +142,35 @@ __device__ __forceinline__ float lane_sum(float v) {
     }
 }
 
-// value held by lane `src_lane` (any lane of the wave; computed at run time)
+// value held by lane `src_lane` (any lane of the wave; computed at run time).  ds_bpermute is several times
+// slower than ds_swizzle/DPP on gfx950: keep it off hot paths.
 __device__ __forceinline__ float lane_read(float v, int src_lane) {
     return __int_as_float(__builtin_amdgcn_ds_bpermute(src_lane << 2, __float_as_int(v)));
+}
+
+// Lane bits [log2(LF), log2(LF*LR)) hold a "row lane" index; every lane receives the F-register fragment of the
+// lane that has the same other bits and row lane index `jo` (uniform, known only at run time).
+// Through LDS: every lane stores its fragment into its own slot of a wave-private buffer and loads the slot of
+// its source lane (one ds_write + one ds_read of 16 bytes per 4 registers; a wave's LDS operations complete in
+// issue order, so no barrier is needed).  ds_bpermute would do the same without memory but costs about six
+// times an FMA per register on gfx950, and a switch over ds_swizzle patterns wrecks register allocation.
+template <int LF, int LR, int F>
+__device__ __forceinline__ void row_lane_broadcast(const float (&v)[F], float (&out)[F], int jo, int lane,
+                                                   float4* wave_slots) {
+    if constexpr (LR == 1) {
+#pragma unroll
+        for (int f = 0; f < F; ++f) out[f] = v[f];
+    } else {
+        static_assert(F % 4 == 0, "fragments are stored as float4");
+        const int src = (lane & ~((LR - 1) * LF)) | (jo * LF);
+#pragma unroll
+        for (int k = 0; k < F / 4; ++k) wave_slots[k * 64 + lane] = make_float4(v[4 * k], v[4 * k + 1], v[4 * k + 2], v[4 * k + 3]);
+#pragma unroll
+        for (int k = 0; k < F / 4; ++k) {
+            const float4 t = wave_slots[k * 64 + src];
+            out[4 * k] = t.x; out[4 * k + 1] = t.y; out[4 * k + 2] = t.z; out[4 * k + 3] = t.w;
+        }
+    }
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -7,11 +7,11 @@ namespace ncn {
 
 hipError_t launch_fast_forward(Pass pass, const StageArgs& a, int n_head, int grid_x, hipStream_t s) {
     const dim3 grid(grid_x, n_head), block(kBlockThreads);
-#define NCN_CASE(NC, EC, FPL)                                                                        \
-    static_assert(fast_fpl(NC, EC) == FPL, "config list disagrees with fast_fpl()");                \
+#define NCN_CASE(NC, EC, R, F)                                                                        \
+    static_assert(fast_tile(NC, EC).r == R && fast_tile(NC, EC).f == F, "duplicate config entry");                \
     if (a.n_cache == NC && a.head_dim == EC) {                                                       \
-        if (pass == kInverse) hipLaunchKernelGGL((stage_inverse_kernel<NC, EC, FPL>), grid, block, 0, s, a); \
-        else hipLaunchKernelGGL((stage_forward_kernel<NC, EC, FPL>), grid, block, 0, s, a);          \
+        if (pass == kInverse) hipLaunchKernelGGL((stage_inverse_kernel<NC, EC, R, F>), grid, block, 0, s, a); \
+        else hipLaunchKernelGGL((stage_forward_kernel<NC, EC, R, F>), grid, block, 0, s, a);          \
         return hipGetLastError();                                                                    \
     }
     NCN_FOR_EACH_FAST_CONFIG(NCN_CASE)

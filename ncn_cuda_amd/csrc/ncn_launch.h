@@ -2,29 +2,30 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include "ncn_configs.h"
 #include "ncn_device.h"
 
 namespace ncn {
 
 enum Pass { kForward = 0, kInverse = 1, kBackward = 2 };
 
-// Features per lane the register kernels use for (n_cache, head width); 0 = no register kernel.
-constexpr int fast_fpl(int nc, int ec) {
-    if (!(nc == 2 || nc == 4 || nc == 8 || nc == 16 || nc == 32)) return 0;
-    int fpl = 0;
-    switch (ec) {
-        case 4: fpl = 4; break;
-        case 8: fpl = 8; break;
-        case 16: fpl = 16; break;
-        case 32: fpl = 16; break;
-        case 64: fpl = 16; break;
-        default: return 0;
-    }
-    return (nc * (ec / fpl) <= 64) ? fpl : 0;
+// Register tile (rows x features per lane) the register kernels use for (n_cache, head width); {0,0} = none.
+struct TileShape {
+    int r, f;
+};
+constexpr TileShape fast_tile(int nc, int ec) {
+#define NCN_MATCH(NC, EC, R, F) \
+    if (nc == NC && ec == EC) return TileShape{R, F};
+    NCN_FOR_EACH_FAST_CONFIG(NCN_MATCH)
+#undef NCN_MATCH
+    return TileShape{0, 0};
 }
 
 // Groups that one 64-lane wave tile carries on each path.
-inline int fast_groups_per_tile(int nc, int ec) { return 64 / (nc * (ec / fast_fpl(nc, ec))); }
+inline int fast_groups_per_tile(int nc, int ec) {
+    const TileShape t = fast_tile(nc, ec);
+    return 64 / ((nc / t.r) * (ec / t.f));
+}
 inline int generic_groups_per_tile(int nc) { return 64 / nc; }
 
 // Largest head width the generic LDS kernel can hold (7 float arrays of [Ec][64] in 160 KB of LDS).
@@ -33,10 +34,13 @@ constexpr int kGenericArrays = 7;
 
 // Upper bound on gridDim.x of a stage launch == rows of the dW partial buffer.
 constexpr int kMaxGridX = 2048;
+// dW partial rows are summed in two levels: chunks of kReduceRowsPerBlock rows, then the chunk sums.
+constexpr int kReduceRowsPerBlock = 32;
+constexpr int kReduceLevel1Rows = kMaxGridX / kReduceRowsPerBlock;
 
 hipError_t launch_fast_forward(Pass pass, const StageArgs& a, int n_head, int grid_x, hipStream_t s);
 hipError_t launch_fast_backward(const StageArgs& a, int n_head, int grid_x, hipStream_t s);
 hipError_t launch_generic(Pass pass, const StageArgs& a, int n_head, int grid_x, hipStream_t s);
-hipError_t launch_reduce_dw(const float* partials, int rows, int64_t cols, float* dW, hipStream_t s);
+hipError_t launch_reduce_dw(const float* partials, int rows, int64_t cols, float* level1, float* dW, hipStream_t s);
 
 }  // namespace ncn

@@ -1,19 +1,26 @@
 // Register-resident stage kernels: forward, inverse and reversible backward of ONE stage.
 //
 // Work decomposition.  A (batch, head, group) triple is an independent problem: n_cache rows of Ec
-// features (torch_ref/ncn_pytorch.py:50-97).  A row is split over LPR = Ec/FPL adjacent lanes that each
-// keep FPL features of x and xa (and of the two gradients) in registers; the n_cache rows of a group
-// occupy n_cache*LPR adjacent lanes, so one 64-wide wavefront carries 64/(n_cache*LPR) whole groups
-// ("a wave tile") and no step of the recurrence ever needs a workgroup barrier:
-//   * the pivot row x_j of a step reaches the other rows with one ds_bpermute per register,
-//   * <x_i,Wi> + <x_j,Wj> and <u_i,x_j> are in-lane FMAs plus log2(LPR) cross-lane adds,
-//   * the sum over rows that feeds the pivot row's gradient is log2(n_cache) cross-lane adds.
+// features (torch_ref/ncn_pytorch.py:50-97).  Each lane keeps an R x F register tile of it: R
+// consecutive rows of the group times F consecutive features of the head.  A row is thus spread
+// over LF = Ec/F adjacent lanes and a group over LR = n_cache/R "row lanes" of LF lanes each, so
+// one 64-wide wavefront carries 64/(LF*LR) whole groups ("a wave tile") and no step of the recurrence
+// needs a workgroup barrier:
+//   * the pivot row x_j of a step lives in row lane j/R, register row j%R; the other row lanes get
+//     it through a wave-private LDS slot array (nothing to do when LR == 1),
+//   * <x_i,Wi> + <x_j,Wj> and <u_i,x_j> are in-lane FMAs over F features plus log2(LF) DPP adds,
+//   * the sum over rows that feeds the pivot row's gradient is an in-lane FMA chain over the R rows
+//     plus log2(LR) cross-lane adds per feature register,
+//   * <x_j,Wj> costs F FMAs per lane and step, i.e. 1/R per element.
+// The step loop runs over j/R at run time and is unrolled over j%R, so register rows are addressed
+// statically while the code stays R steps long.
 // A wave loops over wave tiles of one head (blockIdx.y), keeps that head's slices of Wi, Wj in
 // registers, and in backward accumulates dWi, dWj in registers over all its tiles; they are reduced
 // across lanes and waves once per block and leave as one [2*Ec] partial per block.
 //
-// Memory: a lane reads and writes only its own FPL-feature fragment of its own row (16-byte vector
-// accesses; a row of one head is one contiguous Ec*4-byte segment), each row exactly once per stage.
+// Memory: a lane reads and writes only its own F-feature fragments of its own R rows (16-byte vector
+// accesses; the LF lanes of a row cover its contiguous Ec-element head slice), each row exactly once
+// per stage.
 #pragma once
 #include "ncn_device.h"
 
@@ -21,244 +28,332 @@ namespace ncn {
 
 constexpr int kWavesPerBlock = 4;
 constexpr int kBlockThreads = 64 * kWavesPerBlock;
+constexpr float kTwoLog2e = 2.8853900817779268f;  // exp(2T) = exp2(kTwoLog2e * T)
 
-template <int NC, int EC, int FPL>
+template <int NC, int EC, int R, int F>
 struct Tile {
-    static_assert(EC % FPL == 0, "FPL must divide the head width");
-    static constexpr int LPR = EC / FPL;       // lanes per row
-    static constexpr int LPG = NC * LPR;       // lanes per group
+    static_assert(EC % F == 0 && NC % R == 0, "tile must divide the group");
+    static constexpr int LF = EC / F;      // lanes per row
+    static constexpr int LR = NC / R;      // row lanes per group
+    static constexpr int LPG = LF * LR;    // lanes per group
     static_assert(LPG <= 64 && 64 % LPG == 0, "a group must fit one wavefront");
-    static constexpr int GPW = 64 / LPG;       // groups per wave tile
-    static constexpr int ROWMASK = (NC - 1) * LPR;
+    static constexpr int GPW = 64 / LPG;   // groups per wave tile
+    static constexpr int RLMASK = (LR - 1) * LF;
 };
 
-// Position of this lane's row and validity, for wave tile `t`.
-template <int NC, int EC, int FPL>
-__device__ __forceinline__ bool tile_row_offset(const StageArgs& A, uint32_t t, int lane, int head, int64_t& off) {
-    using T = Tile<NC, EC, FPL>;
-    const int q = lane % T::LPR;
-    const int i = (lane / T::LPR) % NC;
+// Element offsets of this lane's R row fragments for wave tile `t`; false when the lane's group is past the end.
+template <int NC, int EC, int R, int F>
+__device__ __forceinline__ bool tile_offsets(const StageArgs& A, uint32_t t, int lane, int head, int64_t (&off)[R]) {
+    using T = Tile<NC, EC, R, F>;
+    const int fl = lane % T::LF;
+    const int rl = (lane / T::LF) % T::LR;
     const int gw = lane / T::LPG;
     const uint32_t b = t / A.tiles_per_inst;
     const uint32_t tile = t - b * A.tiles_per_inst;
     const uint32_t group = tile * T::GPW + gw;
     const bool valid = group < A.groups;
-    const uint32_t blk = stage_block(A, valid ? group : 0u, (uint32_t)i);
-    const int64_t pos = (int64_t)blk * NC + i;
-    off = ((int64_t)b * A.N + pos) * A.E + (int64_t)head * EC + q * FPL;
+    const int64_t base = (int64_t)b * A.N * A.E + (int64_t)head * EC + fl * F;
+#pragma unroll
+    for (int rr = 0; rr < R; ++rr) {
+        const uint32_t i = rl * R + rr;
+        const uint32_t blk = stage_block(A, valid ? group : 0u, i);
+        off[rr] = base + ((int64_t)blk * NC + i) * A.E;
+    }
     return valid;
 }
 
-template <int FPL>
-__device__ __forceinline__ void load_w(const StageArgs& A, int head, int ec, int q, float (&wi)[FPL], float (&wj)[FPL]) {
-    const float* w = A.W + (int64_t)head * ec + q * FPL;
+template <int F>
+__device__ __forceinline__ void load_w(const StageArgs& A, int head, int ec, int fl, float (&wi)[F], float (&wj)[F]) {
+    const float* w = A.W + (int64_t)head * ec + fl * F;
 #pragma unroll
-    for (int f = 0; f < FPL; ++f) {
+    for (int f = 0; f < F; ++f) {
         wi[f] = w[f];
         wj[f] = w[A.E + f];
     }
 }
 
+template <int F>
+__device__ __forceinline__ float dot_frag(const float (&a)[F], const float (&b)[F]) {
+    float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+    for (int f = 0; f < F; f += 2) {
+        s0 = fmaf(a[f], b[f], s0);
+        if (f + 1 < F) s1 = fmaf(a[f + 1], b[f + 1], s1);
+    }
+    return s0 + s1;
+}
+
 // ---------------------------------------------------------------------------------------------
 // forward (torch_ref/ncn_pytorch.py:74-94)
+//   s_i = <x_i,Wi> + <x_j,Wj>      T = alpha x_i + (1-alpha) s_i x_j      F = tanh T = 1 - 2r,
+//   r = 1/(1 + exp(2T))            a' = m a + (1-m) F                     x' = m x + (1-m) a'
 // ---------------------------------------------------------------------------------------------
-template <int NC, int EC, int FPL>
-__global__ void __launch_bounds__(kBlockThreads) stage_forward_kernel(const StageArgs A) {
-    using T = Tile<NC, EC, FPL>;
+template <int NC, int EC, int R, int F, int WPE = 1>
+__global__ void __launch_bounds__(kBlockThreads, WPE) stage_forward_kernel(const StageArgs A) {
+    using T = Tile<NC, EC, R, F>;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int head = blockIdx.y;
-    const int q = lane % T::LPR;
-    const float alpha = A.alpha, m = A.m, om = 1.0f - A.m, oa = 1.0f - A.alpha;
+    __shared__ float4 bcast_lds[T::LR == 1 ? 1 : kWavesPerBlock * (F / 4) * 64];
+    float4* slots = bcast_lds + (T::LR == 1 ? 0 : wave * (F / 4) * 64);
+    const int fl = lane % T::LF;
+    const float m = A.m, om = 1.0f - A.m;
+    const float ka = kTwoLog2e * A.alpha, kc = kTwoLog2e * (1.0f - A.alpha);
+    const float m2om = -2.0f * om;
 
-    float wi[FPL], wj[FPL];
-    load_w<FPL>(A, head, EC, q, wi, wj);
+    float wi[F], wj[F];
+    load_w<F>(A, head, EC, fl, wi, wj);
 
     const uint32_t nwaves = gridDim.x * kWavesPerBlock;
     for (uint32_t t = blockIdx.x * kWavesPerBlock + wave; t < A.total_tiles; t += nwaves) {
-        int64_t off;
-        const bool valid = tile_row_offset<NC, EC, FPL>(A, t, lane, head, off);
-        float x[FPL], a[FPL];
-        load_frag<FPL>(A.in0, A.in_dtype, off, valid, x);
-        load_frag<FPL>(A.in1, A.in_dtype, off, valid, a);
+        int64_t off[R];
+        const bool valid = tile_offsets<NC, EC, R, F>(A, t, lane, head, off);
+        float x[R][F], a[R][F];
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) {
+            load_frag<F>(A.in0, A.in_dtype, off[rr], valid, x[rr]);
+            load_frag<F>(A.in1, A.in_dtype, off[rr], valid, a[rr]);
+        }
 
 #pragma unroll 1
-        for (int j = 0; j < NC; ++j) {
-            const int src = (lane & ~T::ROWMASK) | (j * T::LPR);
-            float xj[FPL];
-            float d = 0.f, e = 0.f;
+        for (int jo = 0; jo < T::LR; ++jo) {
 #pragma unroll
-            for (int f = 0; f < FPL; ++f) {
-                xj[f] = lane_read(x[f], src);
-                d = fmaf(x[f], wi[f], d);
-                e = fmaf(xj[f], wj[f], e);
-            }
-            const float s = lane_sum<1, T::LPR>(d + e);
-            const float c = oa * s;
+            for (int jr = 0; jr < R; ++jr) {
+                float xj[F];
+                row_lane_broadcast<T::LF, T::LR, F>(x[jr], xj, jo, lane, slots);
+                const float e = dot_frag<F>(xj, wj);
+                // pivot row last: its registers are the source of xj when LR == 1
 #pragma unroll
-            for (int f = 0; f < FPL; ++f) {
-                const float Tv = fmaf(alpha, x[f], c * xj[f]);
-                const float F = tanh_f(Tv);
-                a[f] = fmaf(m, a[f], om * F);
-                x[f] = fmaf(m, x[f], om * a[f]);
+                for (int k = 1; k <= R; ++k) {
+                    const int rr = (jr + k) % R;
+                    const float s = lane_sum<1, T::LF>(dot_frag<F>(x[rr], wi) + e);
+                    const float c = kc * s;
+#pragma unroll
+                    for (int f = 0; f < F; ++f) {
+                        const float z = fmaf(c, xj[f], ka * x[rr][f]);
+                        const float r = __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(z) + 1.0f);
+                        a[rr][f] = fmaf(m2om, r, fmaf(m, a[rr][f], om));
+                        x[rr][f] = fmaf(om, a[rr][f], m * x[rr][f]);
+                    }
+                }
             }
         }
-        store_frag<FPL>(A.out0, A.out_dtype, off, valid, x);
-        store_frag<FPL>(A.out1, A.out_dtype, off, valid, a);
-        if (A.aux0) {
-            store_frag<FPL>(A.aux0, NCN_F32, off, valid, x);
-            store_frag<FPL>(A.aux1, NCN_F32, off, valid, a);
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) {
+            store_frag<F>(A.out0, A.out_dtype, off[rr], valid, x[rr]);
+            store_frag<F>(A.out1, A.out_dtype, off[rr], valid, a[rr]);
+            if (A.aux0) {
+                store_frag<F>(A.aux0, NCN_F32, off[rr], valid, x[rr]);
+                store_frag<F>(A.aux1, NCN_F32, off[rr], valid, a[rr]);
+            }
         }
     }
 }
 
 // ---------------------------------------------------------------------------------------------
 // inverse (torch_ref/ncn_pytorch_invertible.py:87-113), steps j = n_cache-1 .. 0
+//   x = (y - (1-m) b)/m       recompute r from x        a = (b - (1-m) F)/m
 // ---------------------------------------------------------------------------------------------
-template <int NC, int EC, int FPL>
-__global__ void __launch_bounds__(kBlockThreads) stage_inverse_kernel(const StageArgs A) {
-    using T = Tile<NC, EC, FPL>;
+template <int NC, int EC, int R, int F, int WPE = 1>
+__global__ void __launch_bounds__(kBlockThreads, WPE) stage_inverse_kernel(const StageArgs A) {
+    using T = Tile<NC, EC, R, F>;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int head = blockIdx.y;
-    const int q = lane % T::LPR;
-    const float alpha = A.alpha, oa = 1.0f - A.alpha;
-    const float inv_m = 1.0f / A.m, k_ba = (1.0f - A.m) / A.m;
+    __shared__ float4 bcast_lds[T::LR == 1 ? 1 : kWavesPerBlock * (F / 4) * 64];
+    float4* slots = bcast_lds + (T::LR == 1 ? 0 : wave * (F / 4) * 64);
+    const int fl = lane % T::LF;
+    const float om = 1.0f - A.m;
+    const float ka = kTwoLog2e * A.alpha, kc = kTwoLog2e * (1.0f - A.alpha);
+    const float inv_m = 1.0f / A.m, k_ba = om / A.m;
 
-    float wi[FPL], wj[FPL];
-    load_w<FPL>(A, head, EC, q, wi, wj);
+    float wi[F], wj[F];
+    load_w<F>(A, head, EC, fl, wi, wj);
 
     const uint32_t nwaves = gridDim.x * kWavesPerBlock;
     for (uint32_t t = blockIdx.x * kWavesPerBlock + wave; t < A.total_tiles; t += nwaves) {
-        int64_t off;
-        const bool valid = tile_row_offset<NC, EC, FPL>(A, t, lane, head, off);
-        float y[FPL], b[FPL];
-        load_frag<FPL>(A.in0, A.in_dtype, off, valid, y);
-        load_frag<FPL>(A.in1, A.in_dtype, off, valid, b);
+        int64_t off[R];
+        const bool valid = tile_offsets<NC, EC, R, F>(A, t, lane, head, off);
+        float y[R][F], b[R][F];
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) {
+            load_frag<F>(A.in0, A.in_dtype, off[rr], valid, y[rr]);
+            load_frag<F>(A.in1, A.in_dtype, off[rr], valid, b[rr]);
+        }
 
 #pragma unroll 1
-        for (int j = NC - 1; j >= 0; --j) {
-            const int src = (lane & ~T::ROWMASK) | (j * T::LPR);
-            float xj[FPL];
-            float d = 0.f, e = 0.f;
+        for (int jo = T::LR - 1; jo >= 0; --jo) {
 #pragma unroll
-            for (int f = 0; f < FPL; ++f) y[f] = fmaf(y[f], inv_m, -k_ba * b[f]);  // x of this step
+            for (int jr = R - 1; jr >= 0; --jr) {
 #pragma unroll
-            for (int f = 0; f < FPL; ++f) {
-                xj[f] = lane_read(y[f], src);
-                d = fmaf(y[f], wi[f], d);
-                e = fmaf(xj[f], wj[f], e);
-            }
-            const float s = lane_sum<1, T::LPR>(d + e);
-            const float c = oa * s;
+                for (int rr = 0; rr < R; ++rr)
 #pragma unroll
-            for (int f = 0; f < FPL; ++f) {
-                const float Tv = fmaf(alpha, y[f], c * xj[f]);
-                const float F = tanh_f(Tv);
-                b[f] = fmaf(b[f], inv_m, -k_ba * F);  // xa of this step
+                    for (int f = 0; f < F; ++f) y[rr][f] = fmaf(y[rr][f], inv_m, -k_ba * b[rr][f]);
+                float xj[F];
+                row_lane_broadcast<T::LF, T::LR, F>(y[jr], xj, jo, lane, slots);
+                const float e = dot_frag<F>(xj, wj);
+#pragma unroll
+                for (int rr = 0; rr < R; ++rr) {
+                    const float s = lane_sum<1, T::LF>(dot_frag<F>(y[rr], wi) + e);
+                    const float c = kc * s;
+#pragma unroll
+                    for (int f = 0; f < F; ++f) {
+                        const float z = fmaf(c, xj[f], ka * y[rr][f]);
+                        const float r = __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(z) + 1.0f);
+                        b[rr][f] = fmaf(2.0f * k_ba, r, fmaf(b[rr][f], inv_m, -k_ba));
+                    }
+                }
             }
         }
-        store_frag<FPL>(A.out0, A.out_dtype, off, valid, y);
-        store_frag<FPL>(A.out1, A.out_dtype, off, valid, b);
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) {
+            store_frag<F>(A.out0, A.out_dtype, off[rr], valid, y[rr]);
+            store_frag<F>(A.out1, A.out_dtype, off[rr], valid, b[rr]);
+        }
     }
 }
 
 // ---------------------------------------------------------------------------------------------
 // reversible backward: per step, invert (ncn_bwd_cuda_kernel.cu:88-115), then the closed-form
-// vector-Jacobian product (the vectorised statement is ncn_triton/ncn_triton.py:198-246):
-//   q = (1-m)^2 g + (1-m) h      u = q * F'(T)       r_i = <u_i, x_j>
-//   dWi += (1-a) r_i x_i         dWj += (1-a) r_i x_j
-//   g_i <- m g_i + a u_i + (1-a) r_i Wi  [+ sum_k ((1-a) r_k Wj + (1-a) s_k u_k) on the pivot row]
-//   h_i <- m (1-m) g_i + m h_i
+// vector-Jacobian product (vectorised statement: ncn_triton/ncn_triton.py:198-246).  With g = dL/dx',
+// h = dL/da' and p = (1-m) g + h carried instead of h:
+//   u_i  = (1-m) p_i F'(T_i),   F' = 1 - F^2 = 4 r (1 - r)          r_i = <u_i, x_j>
+//   dWi += (1-a) r_i x_i        dWj += (1-a) (sum_i r_i) x_j
+//   g_i <- m g_i + a u_i + (1-a) r_i Wi   [+ sum_k ((1-a) r_k Wj + (1-a) s_k u_k) on the pivot row j]
+//   p_i <- (1-m) g_i(new) + m p_i          (equivalent to h_i <- m (1-m) g_i + m h_i)
+//
+// The divisions by m of the inversion and the multiplications by m of the gradient recurrences are
+// folded into per-step scalars: after t inversion steps the registers hold
+//   Y = m^t x,   B = m^t xa,   G = g / m^t,   P = p / m^t,
+// which turns  x <- (y - (1-m) b)/m  into  Y <- Y - (1-m) B,   g <- m g + ..  into  G <- G + ../m^(t+1)
+// and  p <- (1-m) g + m p  into  P <- P + (1-m) G  (one FMA each); the powers of m are kept in double.
 // ---------------------------------------------------------------------------------------------
-template <int NC, int EC, int FPL>
-__global__ void __launch_bounds__(kBlockThreads) stage_backward_kernel(const StageArgs A) {
-    using T = Tile<NC, EC, FPL>;
+template <int NC, int EC, int R, int F, int WPE = 1>
+__global__ void __launch_bounds__(kBlockThreads, WPE) stage_backward_kernel(const StageArgs A) {
+    using T = Tile<NC, EC, R, F>;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int head = blockIdx.y;
-    const int q = lane % T::LPR;
-    const int row = (lane / T::LPR) % NC;
-    const float alpha = A.alpha, m = A.m, om = 1.0f - A.m, oa = 1.0f - A.alpha;
-    const float inv_m = 1.0f / m, k_ba = om / m;
-    const float k1 = om * om, k2 = om, kh1 = m * om;
+    __shared__ float4 bcast_lds[T::LR == 1 ? 1 : kWavesPerBlock * (F / 4) * 64];
+    float4* slots = bcast_lds + (T::LR == 1 ? 0 : wave * (F / 4) * 64);
+    const int fl = lane % T::LF;
+    const int rl = (lane / T::LF) % T::LR;
+    const float alpha = A.alpha, om = 1.0f - A.m;
+    const float ku = 4.0f * om / A.m * alpha;  // G += ku * U        (U = P (r - r^2))
+    const float nom = -om;
 
-    float wi[FPL], wj[FPL];
-    load_w<FPL>(A, head, EC, q, wi, wj);
-    float dwi[FPL], dwj[FPL];
+    float wi[F], wj[F];
+    load_w<F>(A, head, EC, fl, wi, wj);
+    float dwi[F], dwj[F];
 #pragma unroll
-    for (int f = 0; f < FPL; ++f) dwi[f] = dwj[f] = 0.f;
+    for (int f = 0; f < F; ++f) dwi[f] = dwj[f] = 0.f;
 
     const uint32_t nwaves = gridDim.x * kWavesPerBlock;
     for (uint32_t t = blockIdx.x * kWavesPerBlock + wave; t < A.total_tiles; t += nwaves) {
-        int64_t off;
-        const bool valid = tile_row_offset<NC, EC, FPL>(A, t, lane, head, off);
-        float y[FPL], b[FPL], g[FPL], h[FPL];
-        load_frag<FPL>(A.in0, A.in_dtype, off, valid, y);
-        load_frag<FPL>(A.in1, A.in_dtype, off, valid, b);
-        load_frag<FPL>(A.g0, A.g_dtype, off, valid, g);
-        load_frag<FPL>(A.g1, A.g_dtype, off, valid && A.g1 != nullptr, h);
-
+        int64_t off[R];
+        const bool valid = tile_offsets<NC, EC, R, F>(A, t, lane, head, off);
+        float Y[R][F], B[R][F], G[R][F], P[R][F];
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) {
+            load_frag<F>(A.in0, A.in_dtype, off[rr], valid, Y[rr]);
+            load_frag<F>(A.in1, A.in_dtype, off[rr], valid, B[rr]);
+            load_frag<F>(A.g0, A.g_dtype, off[rr], valid, G[rr]);
+            load_frag<F>(A.g1, A.g_dtype, off[rr], valid && A.g1 != nullptr, P[rr]);
+#pragma unroll
+            for (int f = 0; f < F; ++f) P[rr][f] = fmaf(om, G[rr][f], P[rr][f]);
+        }
 #pragma unroll 1
-        for (int j = NC - 1; j >= 0; --j) {
-            const int src = (lane & ~T::ROWMASK) | (j * T::LPR);
-            float xj[FPL], u[FPL];
-            float d = 0.f, e = 0.f;
+        for (int jo = T::LR - 1; jo >= 0; --jo) {
+            const float sel = (T::LR == 1 || rl == jo) ? 1.0f : 0.0f;  // this lane holds the pivot row
 #pragma unroll
-            for (int f = 0; f < FPL; ++f) y[f] = fmaf(y[f], inv_m, -k_ba * b[f]);  // x of this step
+            for (int jr = R - 1; jr >= 0; --jr) {
+                const int ts = (T::LR - 1 - jo) * R + (R - 1 - jr);   // inversion steps done so far
+                const float lam = A.step[ts].lam;     // z = lam Y_i + chat_i Yj
+                const float kc2 = A.step[ts].kc2;     // chat_i = kc2 S_i
+                const float kap = A.step[ts].kap;     // B <- B - kap F
+                const float krho = A.step[ts].krho;   // rho_i = krho <U_i, Yj>
 #pragma unroll
-            for (int f = 0; f < FPL; ++f) {
-                xj[f] = lane_read(y[f], src);
-                d = fmaf(y[f], wi[f], d);
-                e = fmaf(xj[f], wj[f], e);
-            }
-            const float s = lane_sum<1, T::LPR>(d + e);
-            const float c = oa * s;
-            float r = 0.f;
+                for (int rr = 0; rr < R; ++rr)
 #pragma unroll
-            for (int f = 0; f < FPL; ++f) {
-                const float Tv = fmaf(alpha, y[f], c * xj[f]);
-                float F, dF;
-                tanh_fd(Tv, F, dF);
-                b[f] = fmaf(b[f], inv_m, -k_ba * F);  // xa of this step
-                const float qq = fmaf(k1, g[f], k2 * h[f]);
-                u[f] = qq * dF;
-                r = fmaf(u[f], xj[f], r);
-            }
-            r = lane_sum<1, T::LPR>(r);
-            const float cr = oa * r;
-            const bool pivot = (row == j);
+                    for (int f = 0; f < F; ++f) Y[rr][f] = fmaf(nom, B[rr][f], Y[rr][f]);  // m^(t+1) x of this step
+                float xj[F], v[F];
+                row_lane_broadcast<T::LF, T::LR, F>(Y[jr], xj, jo, lane, slots);
 #pragma unroll
-            for (int f = 0; f < FPL; ++f) {
-                dwi[f] = fmaf(r, y[f], dwi[f]);
-                dwj[f] = fmaf(r, xj[f], dwj[f]);
-                float v = fmaf(cr, wj[f], c * u[f]);
-                v = lane_sum<T::LPR, T::LPG>(v);  // over the rows of the group
-                const float gn = fmaf(m, g[f], fmaf(alpha, u[f], cr * wi[f]));
-                h[f] = fmaf(kh1, g[f], m * h[f]);
-                g[f] = pivot ? gn + v : gn;
+                for (int f = 0; f < F; ++f) v[f] = 0.f;
+                const float e = dot_frag<F>(xj, wj);
+                float rhosum = 0.f;
+#pragma unroll
+                for (int rr = 0; rr < R; ++rr) {
+                    const float S = lane_sum<1, T::LF>(dot_frag<F>(Y[rr], wi) + e);
+                    const float chat = kc2 * S;
+                    float u[F];
+                    float rh = 0.f;
+#pragma unroll
+                    for (int f = 0; f < F; ++f) {
+                        const float z = fmaf(chat, xj[f], lam * Y[rr][f]);
+                        const float r = __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(z) + 1.0f);
+                        B[rr][f] = fmaf(2.0f * kap, r, B[rr][f] - kap);   // m^(t+1) xa of this step
+                        u[f] = P[rr][f] * fmaf(-r, r, r);
+                        rh = fmaf(u[f], xj[f], rh);
+                    }
+                    rh = lane_sum<1, T::LF>(rh);
+                    const float rho = krho * rh;     // (1-alpha) r_i / m^(t+1)
+                    const float c4 = krho * S;       // (1-alpha) s_i u-scale / m^(t+1)
+                    rhosum += rho;
+#pragma unroll
+                    for (int f = 0; f < F; ++f) {
+                        dwi[f] = fmaf(rho, Y[rr][f], dwi[f]);
+                        v[f] = fmaf(c4, u[f], v[f]);
+                        G[rr][f] = fmaf(rho, wi[f], fmaf(ku, u[f], G[rr][f]));
+                        if (rr != jr) P[rr][f] = fmaf(om, G[rr][f], P[rr][f]);
+                    }
+                }
+#pragma unroll
+                for (int f = 0; f < F; ++f) {
+                    dwj[f] = fmaf(rhosum, xj[f], dwj[f]);
+                    const float vt = lane_sum<T::LF, T::LPG>(fmaf(rhosum, wj[f], v[f]));  // over the group's row lanes
+                    G[jr][f] = fmaf(sel, vt, G[jr][f]);
+                    P[jr][f] = fmaf(om, G[jr][f], P[jr][f]);
+                }
+                __builtin_amdgcn_sched_barrier(0);  // keep steps apart: interleaving them only costs registers
             }
         }
-        store_frag<FPL>(A.out0, A.out_dtype, off, valid, g);
-        store_frag<FPL>(A.out1, A.out_dtype, off, valid, h);
-        if (A.aux0) {
-            store_frag<FPL>(A.aux0, NCN_F32, off, valid, y);
-            store_frag<FPL>(A.aux1, NCN_F32, off, valid, b);
+        // undo the scalings: t = NC steps done
+        const float up = A.inv_m_pow_n;   // m^-NC
+        const float dn = A.m_pow_n;       // m^NC
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) {
+#pragma unroll
+            for (int f = 0; f < F; ++f) {
+                G[rr][f] *= dn;
+                P[rr][f] = fmaf(P[rr][f], dn, nom * G[rr][f]);  // back to h = p - (1-m) g
+            }
+            store_frag<F>(A.out0, A.out_dtype, off[rr], valid, G[rr]);
+            store_frag<F>(A.out1, A.out_dtype, off[rr], valid, P[rr]);
+            if (A.aux0) {
+#pragma unroll
+                for (int f = 0; f < F; ++f) {
+                    Y[rr][f] *= up;
+                    B[rr][f] *= up;
+                }
+                store_frag<F>(A.aux0, NCN_F32, off[rr], valid, Y[rr]);
+                store_frag<F>(A.aux1, NCN_F32, off[rr], valid, B[rr]);
+            }
         }
     }
 
-    // dW: lanes holding the same feature chunk q -> one value; then across the block's waves.
+    // dW: lanes holding the same feature chunk -> one value; then across the block's waves.
     __shared__ float red[kWavesPerBlock][2][EC];
 #pragma unroll
-    for (int f = 0; f < FPL; ++f) {
-        dwi[f] = lane_sum<T::LPR, 64>(dwi[f]);
-        dwj[f] = lane_sum<T::LPR, 64>(dwj[f]);
+    for (int f = 0; f < F; ++f) {
+        dwi[f] = lane_sum<T::LF, 64>(dwi[f]);
+        dwj[f] = lane_sum<T::LF, 64>(dwj[f]);
     }
-    if (lane < T::LPR) {
+    if (lane < T::LF) {
 #pragma unroll
-        for (int f = 0; f < FPL; ++f) {
-            red[wave][0][q * FPL + f] = dwi[f];
-            red[wave][1][q * FPL + f] = dwj[f];
+        for (int f = 0; f < F; ++f) {
+            red[wave][0][fl * F + f] = dwi[f];
+            red[wave][1][fl * F + f] = dwj[f];
         }
     }
     __syncthreads();
@@ -267,7 +362,7 @@ __global__ void __launch_bounds__(kBlockThreads) stage_backward_kernel(const Sta
         float sum = 0.f;
 #pragma unroll
         for (int w = 0; w < kWavesPerBlock; ++w) sum += red[w][half][f];
-        A.dw_partials[(int64_t)blockIdx.x * (2 * A.E) + (int64_t)half * A.E + (int64_t)head * EC + f] = oa * sum;
+        A.dw_partials[(int64_t)blockIdx.x * (2 * A.E) + (int64_t)half * A.E + (int64_t)head * EC + f] = sum;
     }
 }
 
