@@ -90,6 +90,10 @@ void fill_common(StageArgs& a, const ncn_shape* sh, const Plan& p, int stage, fl
         a.step[t].kc2 = (float)(k2l * (1.0 - al) * im * im);
         a.step[t].kap = (float)((1.0 - md) * std::pow(md, (double)t));
         a.step[t].krho = (float)(4.0 * (1.0 - md) / md * (1.0 - al) * im);
+        const double mt = std::pow(md, (double)t);
+        a.step[t].flam = (float)(k2l * al * mt);
+        a.step[t].fkc = (float)(k2l * (1.0 - al) * mt * mt);
+        a.step[t].fkap = (float)((1.0 - md) * im);
     }
 }
 

@@ -38,8 +38,11 @@ struct StageArgs {
     // (t = 0 is the stage's last step).  Computed on the host in double precision:
     //   im = m^-(t+1),  lam = 2 log2(e) alpha im,  kc2 = 2 log2(e) (1-alpha) im^2,
     //   kap = (1-m) m^t,  krho = 4 (1-m)/m (1-alpha) im
+    // and of the forward, index t = number of steps already done:
+    //   flam = 2 log2(e) alpha m^t,  fkc = 2 log2(e) (1-alpha) m^2t,  fkap = (1-m) / m^(t+1)
     struct StepScalars {
         float lam, kc2, kap, krho;
+        float flam, fkc, fkap;
     } step[64];
 };
 
@@ -52,6 +55,14 @@ __device__ __forceinline__ uint32_t f32_to_bf16(float f) {
     uint32_t u = __float_as_uint(f);
     if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
     return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+
+// two floats -> packed bf16 pair (lo in bits 0..15): one v_cvt_pk_bf16_f32 on gfx950, round to nearest even
+typedef __bf16 ncn_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float ncn_floatx2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    const ncn_floatx2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, ncn_bf16x2));
 }
 
 // Row fragment of FPL consecutive features, element offset `off` into a buffer of type `dtype`.
@@ -93,8 +104,8 @@ __device__ __forceinline__ void store_frag(void* base, int dtype, int64_t off, b
 #pragma unroll
         for (int k = 0; k < FPL / 4; ++k) {
             uint2 t;
-            t.x = f32_to_bf16(v[4 * k + 0]) | (f32_to_bf16(v[4 * k + 1]) << 16);
-            t.y = f32_to_bf16(v[4 * k + 2]) | (f32_to_bf16(v[4 * k + 3]) << 16);
+            t.x = pack_bf16x2(v[4 * k + 0], v[4 * k + 1]);
+            t.y = pack_bf16x2(v[4 * k + 2], v[4 * k + 3]);
             p[k] = t;
         }
     }

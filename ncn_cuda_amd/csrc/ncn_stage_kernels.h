@@ -87,6 +87,8 @@ __device__ __forceinline__ float dot_frag(const float (&a)[F], const float (&b)[
 // forward (torch_ref/ncn_pytorch.py:74-94)
 //   s_i = <x_i,Wi> + <x_j,Wj>      T = alpha x_i + (1-alpha) s_i x_j      F = tanh T = 1 - 2r,
 //   r = 1/(1 + exp(2T))            a' = m a + (1-m) F                     x' = m x + (1-m) a'
+// The registers hold X = x / m^t and A = xa / m^t after t steps, which turns the two updates into
+//   A <- A + (1-m)/m^(t+1) F   and   X <- X + (1-m) A   (the powers of m come from a host-made table).
 // ---------------------------------------------------------------------------------------------
 template <int NC, int EC, int R, int F, int WPE = 1>
 __global__ void __launch_bounds__(kBlockThreads, WPE) stage_forward_kernel(const StageArgs A) {
@@ -97,9 +99,7 @@ __global__ void __launch_bounds__(kBlockThreads, WPE) stage_forward_kernel(const
     __shared__ float4 bcast_lds[T::LR == 1 ? 1 : kWavesPerBlock * (F / 4) * 64];
     float4* slots = bcast_lds + (T::LR == 1 ? 0 : wave * (F / 4) * 64);
     const int fl = lane % T::LF;
-    const float m = A.m, om = 1.0f - A.m;
-    const float ka = kTwoLog2e * A.alpha, kc = kTwoLog2e * (1.0f - A.alpha);
-    const float m2om = -2.0f * om;
+    const float om = 1.0f - A.m;
 
     float wi[F], wj[F];
     load_w<F>(A, head, EC, fl, wi, wj);
@@ -119,6 +119,10 @@ __global__ void __launch_bounds__(kBlockThreads, WPE) stage_forward_kernel(const
         for (int jo = 0; jo < T::LR; ++jo) {
 #pragma unroll
             for (int jr = 0; jr < R; ++jr) {
+                const int ts = jo * R + jr;            // steps done so far
+                const float lam = A.step[ts].flam;     // z = lam X_i + c_i Xj
+                const float kc = A.step[ts].fkc;       // c_i = kc S_i
+                const float kap = A.step[ts].fkap;     // A <- A + kap F
                 float xj[F];
                 row_lane_broadcast<T::LF, T::LR, F>(x[jr], xj, jo, lane, slots);
                 const float e = dot_frag<F>(xj, wj);
@@ -130,16 +134,22 @@ __global__ void __launch_bounds__(kBlockThreads, WPE) stage_forward_kernel(const
                     const float c = kc * s;
 #pragma unroll
                     for (int f = 0; f < F; ++f) {
-                        const float z = fmaf(c, xj[f], ka * x[rr][f]);
+                        const float z = fmaf(c, xj[f], lam * x[rr][f]);
                         const float r = __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(z) + 1.0f);
-                        a[rr][f] = fmaf(m2om, r, fmaf(m, a[rr][f], om));
-                        x[rr][f] = fmaf(om, a[rr][f], m * x[rr][f]);
+                        a[rr][f] = fmaf(-2.0f * kap, r, a[rr][f] + kap);
+                        x[rr][f] = fmaf(om, a[rr][f], x[rr][f]);
                     }
                 }
             }
         }
+        const float dn = A.m_pow_n;
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) {
+#pragma unroll
+            for (int f = 0; f < F; ++f) {
+                x[rr][f] *= dn;
+                a[rr][f] *= dn;
+            }
             store_frag<F>(A.out0, A.out_dtype, off[rr], valid, x[rr]);
             store_frag<F>(A.out1, A.out_dtype, off[rr], valid, a[rr]);
             if (A.aux0) {
@@ -153,6 +163,7 @@ __global__ void __launch_bounds__(kBlockThreads, WPE) stage_forward_kernel(const
 // ---------------------------------------------------------------------------------------------
 // inverse (torch_ref/ncn_pytorch_invertible.py:87-113), steps j = n_cache-1 .. 0
 //   x = (y - (1-m) b)/m       recompute r from x        a = (b - (1-m) F)/m
+// with the same m^t scaling of the registers as the backward kernel below (Y = m^t x, B = m^t xa).
 // ---------------------------------------------------------------------------------------------
 template <int NC, int EC, int R, int F, int WPE = 1>
 __global__ void __launch_bounds__(kBlockThreads, WPE) stage_inverse_kernel(const StageArgs A) {
@@ -163,9 +174,7 @@ __global__ void __launch_bounds__(kBlockThreads, WPE) stage_inverse_kernel(const
     __shared__ float4 bcast_lds[T::LR == 1 ? 1 : kWavesPerBlock * (F / 4) * 64];
     float4* slots = bcast_lds + (T::LR == 1 ? 0 : wave * (F / 4) * 64);
     const int fl = lane % T::LF;
-    const float om = 1.0f - A.m;
-    const float ka = kTwoLog2e * A.alpha, kc = kTwoLog2e * (1.0f - A.alpha);
-    const float inv_m = 1.0f / A.m, k_ba = om / A.m;
+    const float nom = A.m - 1.0f;
 
     float wi[F], wj[F];
     load_w<F>(A, head, EC, fl, wi, wj);
@@ -185,28 +194,36 @@ __global__ void __launch_bounds__(kBlockThreads, WPE) stage_inverse_kernel(const
         for (int jo = T::LR - 1; jo >= 0; --jo) {
 #pragma unroll
             for (int jr = R - 1; jr >= 0; --jr) {
+                const int ts = (T::LR - 1 - jo) * R + (R - 1 - jr);   // inversion steps done so far
+                const float lam = A.step[ts].lam, kc2 = A.step[ts].kc2, kap = A.step[ts].kap;
 #pragma unroll
                 for (int rr = 0; rr < R; ++rr)
 #pragma unroll
-                    for (int f = 0; f < F; ++f) y[rr][f] = fmaf(y[rr][f], inv_m, -k_ba * b[rr][f]);
+                    for (int f = 0; f < F; ++f) y[rr][f] = fmaf(nom, b[rr][f], y[rr][f]);
                 float xj[F];
                 row_lane_broadcast<T::LF, T::LR, F>(y[jr], xj, jo, lane, slots);
                 const float e = dot_frag<F>(xj, wj);
 #pragma unroll
                 for (int rr = 0; rr < R; ++rr) {
                     const float s = lane_sum<1, T::LF>(dot_frag<F>(y[rr], wi) + e);
-                    const float c = kc * s;
+                    const float c = kc2 * s;
 #pragma unroll
                     for (int f = 0; f < F; ++f) {
-                        const float z = fmaf(c, xj[f], ka * y[rr][f]);
+                        const float z = fmaf(c, xj[f], lam * y[rr][f]);
                         const float r = __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(z) + 1.0f);
-                        b[rr][f] = fmaf(2.0f * k_ba, r, fmaf(b[rr][f], inv_m, -k_ba));
+                        b[rr][f] = fmaf(2.0f * kap, r, b[rr][f] - kap);
                     }
                 }
             }
         }
+        const float up = A.inv_m_pow_n;
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) {
+#pragma unroll
+            for (int f = 0; f < F; ++f) {
+                y[rr][f] *= up;
+                b[rr][f] *= up;
+            }
             store_frag<F>(A.out0, A.out_dtype, off[rr], valid, y[rr]);
             store_frag<F>(A.out1, A.out_dtype, off[rr], valid, b[rr]);
         }
