@@ -47,6 +47,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--config", default="cfg3", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run one plain 1 GiB device copy, so that a rocprofv3 --pmc run has a kernel of known "
+                         "traffic to calibrate FETCH_SIZE / WRITE_SIZE against")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the layer shards over batch; "
@@ -99,6 +102,12 @@ def main():
                 events.append((e0, e1))
         return cx, cxa, dy, dya_, dWs
 
+    if args.copy_probe:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()

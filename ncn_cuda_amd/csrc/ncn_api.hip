@@ -52,6 +52,7 @@ struct Plan {
     int groups_per_tile;
     uint32_t groups, tiles_per_inst, total_tiles;
     int grid_x;
+    int partial_rows;  // rows of the dW partial buffer the backward launch writes
 };
 
 Plan make_plan(const ncn_shape* sh, int activation) {
@@ -62,9 +63,23 @@ Plan make_plan(const ncn_shape* sh, int activation) {
     p.groups = (uint32_t)(sh->N / sh->n_cache);
     p.tiles_per_inst = (p.groups + p.groups_per_tile - 1) / p.groups_per_tile;
     p.total_tiles = (uint32_t)(sh->batch * p.tiles_per_inst);
-    const int tiles_per_block = (p.path == 2) ? 4 : 1;
-    const int64_t blocks = ((int64_t)p.total_tiles + tiles_per_block - 1) / tiles_per_block;
-    p.grid_x = (int)(blocks < kMaxGridX ? blocks : kMaxGridX);
+    if (p.path == 2) {
+        // 4 waves per block, wave w works on head w % n_head: the grid holds a multiple of n_head waves and at
+        // most kMaxGridX partial rows (one per n_head consecutive waves)
+        const int C = sh->n_head;
+        const int g4 = (C % 4 == 0) ? 4 : (C % 2 == 0 ? 2 : 1);
+        const int64_t quantum = C / g4;                                   // blocks per multiple of n_head waves
+        const int64_t cap = (int64_t)kMaxGridX * C / 4 / quantum * quantum;  // rows = blocks * 4 / C <= kMaxGridX
+        int64_t blocks = ((int64_t)p.total_tiles * C + 3) / 4;
+        blocks = (blocks + quantum - 1) / quantum * quantum;
+        if (blocks > cap) blocks = cap;
+        if (blocks < quantum) blocks = quantum;
+        p.grid_x = (int)blocks;
+        p.partial_rows = (int)(blocks * 4 / C);
+    } else {
+        p.grid_x = (int)(p.total_tiles < (uint32_t)kMaxGridX ? p.total_tiles : (uint32_t)kMaxGridX);
+        p.partial_rows = p.grid_x;
+    }
     return p;
 }
 
@@ -78,6 +93,7 @@ void fill_common(StageArgs& a, const ncn_shape* sh, const Plan& p, int stage, fl
     a.groups_pow2 = (p.groups & (p.groups - 1)) == 0 ? 1u : 0u;
     a.n_cache = sh->n_cache;
     a.head_dim = (int)(sh->E / sh->n_head);
+    a.n_head = sh->n_head;
     a.activation = activation;
     a.alpha = alpha;
     a.m = m;
@@ -233,7 +249,7 @@ int ncn_backward(const void* y, const void* ya, int y_dtype, const void* dy, con
         hipError_t err = (p.path == 2) ? launch_fast_backward(a, shape->n_head, p.grid_x, s)
                                        : launch_generic(kBackward, a, shape->n_head, p.grid_x, s);
         if (err != hipSuccess) return (int)err;
-        err = launch_reduce_dw(a.dw_partials, p.grid_x, 2 * shape->E, a.dw_partials + (int64_t)kMaxGridX * 2 * shape->E,
+        err = launch_reduce_dw(a.dw_partials, p.partial_rows, 2 * shape->E, a.dw_partials + (int64_t)kMaxGridX * 2 * shape->E,
                                dW + (int64_t)k * 2 * shape->E, s);
         if (err != hipSuccess) return (int)err;
     }

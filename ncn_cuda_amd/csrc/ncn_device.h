@@ -22,14 +22,14 @@ struct StageArgs {
     float* aux0;
     float* aux1;
     const float* W;      // [2E] of this stage
-    float* dw_partials;  // backward: [gridDim.x][2E]
+    float* dw_partials;  // backward: [partial rows][2E]
     int64_t N, E;
     uint32_t total_tiles;     // batch * tiles_per_instance
     uint32_t tiles_per_inst;  // ceil(groups / groups-per-wave-tile)
     uint32_t groups;          // N / n_cache
     uint32_t stride;          // stride of this stage in blocks: 0, or 2^(stage-1) mod groups
     uint32_t groups_pow2;     // 1 when `groups` is a power of two
-    int32_t n_cache, head_dim;
+    int32_t n_cache, head_dim, n_head;
     int32_t in_dtype, g_dtype, out_dtype;
     int32_t activation;
     float alpha, m;

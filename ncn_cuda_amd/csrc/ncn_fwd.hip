@@ -6,7 +6,7 @@
 namespace ncn {
 
 hipError_t launch_fast_forward(Pass pass, const StageArgs& a, int n_head, int grid_x, hipStream_t s) {
-    const dim3 grid(grid_x, n_head), block(kBlockThreads);
+    const dim3 grid(grid_x), block(kBlockThreads);
 #define NCN_CASE(NC, EC, R, F)                                                                        \
     static_assert(fast_tile(NC, EC).r == R && fast_tile(NC, EC).f == F, "duplicate config entry");                \
     if (a.n_cache == NC && a.head_dim == EC) {                                                       \

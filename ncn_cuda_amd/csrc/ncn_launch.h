@@ -33,7 +33,7 @@ constexpr int kGenericMaxHeadDim = 64;
 constexpr int kGenericArrays = 7;
 
 // Upper bound on gridDim.x of a stage launch == rows of the dW partial buffer.
-constexpr int kMaxGridX = 2048;
+constexpr int kMaxGridX = 4096;
 // dW partial rows are summed in two levels: chunks of kReduceRowsPerBlock rows, then the chunk sums.
 constexpr int kReduceRowsPerBlock = 32;
 constexpr int kReduceLevel1Rows = kMaxGridX / kReduceRowsPerBlock;

@@ -14,11 +14,14 @@
 //   * <x_j,Wj> costs F FMAs per lane and step, i.e. 1/R per element.
 // The step loop runs over j/R at run time and is unrolled over j%R, so register rows are addressed
 // statically while the code stays R steps long.
-// A wave loops over wave tiles of one head (blockIdx.y), keeps that head's slices of Wi, Wj in
-// registers, and in backward accumulates dWi, dWj in registers over all its tiles; they are reduced
-// across lanes and waves once per block and leave as one [2*Ec] partial per block.
+// Wave w of the grid works on head w % n_head for its whole life (the grid holds a multiple of n_head
+// waves) and loops over the wave tiles w / n_head, + waves / n_head, ..: the waves of a block therefore
+// touch the n_head adjacent head slices of the same rows at about the same time, so a 128-byte line that
+// holds two bf16 head slices is fetched from HBM once, not once per head.  A wave keeps its head's slices
+// of Wi, Wj in registers, and in backward accumulates dWi, dWj in registers over all its tiles; they are
+// reduced across its lanes once and leave as this wave's [2*Ec] slice of a partial row.
 //
-// Memory: a lane reads and writes only its own F-feature fragments of its own R rows (16-byte vector
+// Memory: a lane reads and writes only its own F-feature fragments of its own R rows (8/16-byte vector
 // accesses; the LF lanes of a row cover its contiguous Ec-element head slice), each row exactly once
 // per stage.
 #pragma once
@@ -95,7 +98,10 @@ __global__ void __launch_bounds__(kBlockThreads, WPE) stage_forward_kernel(const
     using T = Tile<NC, EC, R, F>;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int head = blockIdx.y;
+    const uint32_t nwaves = gridDim.x * kWavesPerBlock;
+    const uint32_t gwave = blockIdx.x * kWavesPerBlock + wave;
+    const int head = gwave % A.n_head;
+    const uint32_t tile_step = nwaves / A.n_head;
     __shared__ float4 bcast_lds[T::LR == 1 ? 1 : kWavesPerBlock * (F / 4) * 64];
     float4* slots = bcast_lds + (T::LR == 1 ? 0 : wave * (F / 4) * 64);
     const int fl = lane % T::LF;
@@ -104,8 +110,7 @@ __global__ void __launch_bounds__(kBlockThreads, WPE) stage_forward_kernel(const
     float wi[F], wj[F];
     load_w<F>(A, head, EC, fl, wi, wj);
 
-    const uint32_t nwaves = gridDim.x * kWavesPerBlock;
-    for (uint32_t t = blockIdx.x * kWavesPerBlock + wave; t < A.total_tiles; t += nwaves) {
+    for (uint32_t t = gwave / A.n_head; t < A.total_tiles; t += tile_step) {
         int64_t off[R];
         const bool valid = tile_offsets<NC, EC, R, F>(A, t, lane, head, off);
         float x[R][F], a[R][F];
@@ -170,7 +175,10 @@ __global__ void __launch_bounds__(kBlockThreads, WPE) stage_inverse_kernel(const
     using T = Tile<NC, EC, R, F>;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int head = blockIdx.y;
+    const uint32_t nwaves = gridDim.x * kWavesPerBlock;
+    const uint32_t gwave = blockIdx.x * kWavesPerBlock + wave;
+    const int head = gwave % A.n_head;
+    const uint32_t tile_step = nwaves / A.n_head;
     __shared__ float4 bcast_lds[T::LR == 1 ? 1 : kWavesPerBlock * (F / 4) * 64];
     float4* slots = bcast_lds + (T::LR == 1 ? 0 : wave * (F / 4) * 64);
     const int fl = lane % T::LF;
@@ -179,8 +187,7 @@ __global__ void __launch_bounds__(kBlockThreads, WPE) stage_inverse_kernel(const
     float wi[F], wj[F];
     load_w<F>(A, head, EC, fl, wi, wj);
 
-    const uint32_t nwaves = gridDim.x * kWavesPerBlock;
-    for (uint32_t t = blockIdx.x * kWavesPerBlock + wave; t < A.total_tiles; t += nwaves) {
+    for (uint32_t t = gwave / A.n_head; t < A.total_tiles; t += tile_step) {
         int64_t off[R];
         const bool valid = tile_offsets<NC, EC, R, F>(A, t, lane, head, off);
         float y[R][F], b[R][F];
@@ -250,7 +257,10 @@ __global__ void __launch_bounds__(kBlockThreads, WPE) stage_backward_kernel(cons
     using T = Tile<NC, EC, R, F>;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int head = blockIdx.y;
+    const uint32_t nwaves = gridDim.x * kWavesPerBlock;
+    const uint32_t gwave = blockIdx.x * kWavesPerBlock + wave;
+    const int head = gwave % A.n_head;
+    const uint32_t tile_step = nwaves / A.n_head;
     __shared__ float4 bcast_lds[T::LR == 1 ? 1 : kWavesPerBlock * (F / 4) * 64];
     float4* slots = bcast_lds + (T::LR == 1 ? 0 : wave * (F / 4) * 64);
     const int fl = lane % T::LF;
@@ -265,8 +275,7 @@ __global__ void __launch_bounds__(kBlockThreads, WPE) stage_backward_kernel(cons
 #pragma unroll
     for (int f = 0; f < F; ++f) dwi[f] = dwj[f] = 0.f;
 
-    const uint32_t nwaves = gridDim.x * kWavesPerBlock;
-    for (uint32_t t = blockIdx.x * kWavesPerBlock + wave; t < A.total_tiles; t += nwaves) {
+    for (uint32_t t = gwave / A.n_head; t < A.total_tiles; t += tile_step) {
         int64_t off[R];
         const bool valid = tile_offsets<NC, EC, R, F>(A, t, lane, head, off);
         float Y[R][F], B[R][F], G[R][F], P[R][F];
@@ -359,27 +368,19 @@ __global__ void __launch_bounds__(kBlockThreads, WPE) stage_backward_kernel(cons
         }
     }
 
-    // dW: lanes holding the same feature chunk -> one value; then across the block's waves.
-    __shared__ float red[kWavesPerBlock][2][EC];
+    // dW: lanes holding the same feature chunk -> one value; this wave owns slot (gwave / n_head, head).
 #pragma unroll
     for (int f = 0; f < F; ++f) {
         dwi[f] = lane_sum<T::LF, 64>(dwi[f]);
         dwj[f] = lane_sum<T::LF, 64>(dwj[f]);
     }
     if (lane < T::LF) {
+        float* row = A.dw_partials + (int64_t)(gwave / A.n_head) * (2 * A.E) + (int64_t)head * EC + fl * F;
 #pragma unroll
         for (int f = 0; f < F; ++f) {
-            red[wave][0][fl * F + f] = dwi[f];
-            red[wave][1][fl * F + f] = dwj[f];
+            row[f] = dwi[f];
+            row[A.E + f] = dwj[f];
         }
-    }
-    __syncthreads();
-    for (int k = threadIdx.x; k < 2 * EC; k += kBlockThreads) {
-        const int half = k / EC, f = k - half * EC;
-        float sum = 0.f;
-#pragma unroll
-        for (int w = 0; w < kWavesPerBlock; ++w) sum += red[w][half][f];
-        A.dw_partials[(int64_t)blockIdx.x * (2 * A.E) + (int64_t)half * A.E + (int64_t)head * EC + f] = sum;
     }
 }
 
