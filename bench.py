@@ -36,6 +36,9 @@ VALU_PEAK_TFLOPS = 157.3   # MI355X FP32 vector peak (packed); 78.6 without pack
 # float32 operations per element and step of the kernels as written in ncn_stage_kernels.h (FMA = 2, exp2 and
 # rcp = 1 each), without the per-row and per-lane bookkeeping: forward 1 FMA (dot) + 2 (z) + 1 (t+1) + 2 FMA (xa)
 # + 2 (x) + exp2 + rcp = 13; backward 11 FMA + 4 mul/add + exp2 + rcp = 28.
+# HBM bytes of one backward-stage launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (calibrated on a
+# 1 GiB copy; see profiles/stage_kernels_cfg3.md).  Only the headline workload has been measured.
+MEASURED_BWD_TRAFFIC_BYTES = {"cfg3": 1.0824e9}
 FLOPS_FWD_PER_ELEM_STEP = 13.0
 FLOPS_BWD_PER_ELEM_STEP = 28.0
 
@@ -143,7 +146,7 @@ def main():
                                f"{C} heads of {E // C}, n_cache={n}, {L} stages, alpha=0.9, m=0.9, tanh, "
                                f"{cfg['dtype']} storage", "positions_per_s": batch * N / (ms_per_step * 1e-3)},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_BWD_TRAFFIC_BYTES.get(args.config),
                      "kernel": f"stage_backward_kernel<{n},{E // C}>", "avg_launch_ms": bwd_ms,
                      "algorithmic_bytes_per_launch": bytes_bwd_launch},
         "stack": {"algorithmic_bytes_fused": 10.0 * P * sbytes,

@@ -1,0 +1,137 @@
+"""The C-ABI library and the host-side argument checks, without a GPU: the shared object loads, exports every
+function include/ncn_hip.h declares, and rejects bad arguments before any GPU work."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from conftest import ROOT
+
+HEADER = os.path.join(ROOT, "include", "ncn_hip.h")
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from ncn_cuda_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        from ncn_cuda_amd import _build
+        _build.build()
+    return _lib
+
+
+def _declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ncn_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_header_functions_are_exported(lib):
+    names = _declared_functions()
+    assert {"ncn_forward", "ncn_backward", "ncn_inverse", "ncn_workspace_bytes", "ncn_kernel_path",
+            "ncn_check_shape", "ncn_error_string", "ncn_version"} <= set(names)
+    handle = lib.load()
+    for name in names:
+        assert getattr(handle, name) is not None, name
+    assert sorted(lib.EXPORTS) == names
+    assert re.fullmatch(r"\d+\.\d+", handle.ncn_version().decode())
+
+
+def _shape(lib, batch, N, E, C, n):
+    return lib.NcnShape(batch, N, E, C, n)
+
+
+def test_check_shape_codes(lib):
+    h = lib.load()
+    ok = _shape(lib, 2, 64, 32, 4, 4)
+    assert h.ncn_check_shape(ctypes.byref(ok), 0, 1, 0) == 0
+    assert h.ncn_check_shape(None, 0, 1, 0) == -1
+    assert h.ncn_check_shape(ctypes.byref(_shape(lib, 2, 65, 32, 4, 4)), 0, 1, 0) == -2   # N % n_cache
+    assert h.ncn_check_shape(ctypes.byref(_shape(lib, 2, 64, 30, 4, 4)), 0, 1, 0) == -2   # E % n_head
+    assert h.ncn_check_shape(ctypes.byref(_shape(lib, 0, 64, 32, 4, 4)), 0, 1, 0) == -2
+    assert h.ncn_check_shape(ctypes.byref(ok), -1, 1, 0) == -2
+    assert h.ncn_check_shape(ctypes.byref(ok), 0, 0, 0) == -2
+    assert h.ncn_check_shape(ctypes.byref(ok), 0, 1, 7) == -4                             # activation
+    assert h.ncn_check_shape(ctypes.byref(_shape(lib, 1, 256, 32, 4, 128)), 0, 1, 0) == -6  # n_cache > 64
+    assert h.ncn_check_shape(ctypes.byref(_shape(lib, 1, 64, 512, 4, 4)), 0, 1, 0) == -6    # head width 128
+    for code in (0, -1, -2, -3, -4, -5, -6, -7, -8):
+        assert len(h.ncn_error_string(code)) > 0
+
+
+def test_kernel_path_and_workspace(lib):
+    h = lib.load()
+    assert h.ncn_kernel_path(ctypes.byref(_shape(lib, 128, 4096, 128, 4, 16))) == 2   # headline shape: register kernels
+    assert h.ncn_kernel_path(ctypes.byref(_shape(lib, 1, 256, 32, 4, 2))) == 2        # config 1 (Ec = 8)
+    assert h.ncn_kernel_path(ctypes.byref(_shape(lib, 1, 24, 10, 2, 3))) == 1         # n = 3, Ec = 5: generic
+    assert h.ncn_kernel_path(ctypes.byref(_shape(lib, 1, 256, 32, 4, 128))) == 0
+    ws = h.ncn_workspace_bytes(ctypes.byref(_shape(lib, 128, 4096, 128, 4, 16)))
+    assert ws > 0 and ws % 16 == 0 and ws < (1 << 24)
+    assert h.ncn_workspace_bytes(ctypes.byref(_shape(lib, 1, 65, 32, 4, 4))) == 0
+
+
+def test_entry_points_reject_bad_arguments_before_touching_the_gpu(lib):
+    h = lib.load()
+    sh = _shape(lib, 2, 64, 32, 4, 4)
+    p = ctypes.c_void_p(4096)       # never dereferenced: every call below fails validation first
+    z = ctypes.c_void_p(0)
+    odd = ctypes.c_void_p(4100)
+    assert h.ncn_forward(z, p, 0, p, p, 0, z, z, p, ctypes.byref(sh), 0, 1, 0.9, 0.9, 0, z) == -1
+    assert h.ncn_forward(p, p, 5, p, p, 0, z, z, p, ctypes.byref(sh), 0, 1, 0.9, 0.9, 0, z) == -3
+    assert h.ncn_forward(odd, p, 0, p, p, 0, z, z, p, ctypes.byref(sh), 0, 1, 0.9, 0.9, 0, z) == -7
+    assert h.ncn_forward(p, p, 0, p, p, 0, p, z, p, ctypes.byref(sh), 0, 1, 0.9, 0.9, 0, z) == -1  # y32 without ya32
+    assert h.ncn_inverse(p, p, 0, z, p, 0, p, ctypes.byref(sh), 0, 1, 0.9, 0.9, 0, z) == -1
+    ws = h.ncn_workspace_bytes(ctypes.byref(sh))
+    args = [p, p, 0, p, p, 0, p, p, 0, z, z, p, p]
+    assert h.ncn_backward(*args, z, ctypes.c_size_t(0), ctypes.byref(sh), 0, 1, 0.9, 0.9, 0, z) == -5
+    assert h.ncn_backward(*args, p, ctypes.c_size_t(ws - 1), ctypes.byref(sh), 0, 1, 0.9, 0.9, 0, z) == -5
+    assert h.ncn_backward(*args, p, ctypes.c_size_t(ws), ctypes.byref(sh), 0, 2, 0.9, 0.9, 0, z) == -8  # needs x_rec
+
+
+def test_python_validation_mirrors_reference_asserts():
+    from ncn_cuda_amd import ncn_cuda_module as M
+    x = torch.randn(2, 32, 16)
+    W = torch.randn(32)
+    with pytest.raises(ValueError, match="block_size must divide N"):   # torch_ref/ncn_pytorch.py:25
+        M.forward(x, x, W, 0.9, 0, 5, 2, 0)
+    with pytest.raises(ValueError, match="n_head must divide E"):
+        M.forward(x, x, W, 0.9, 0, 4, 3, 0)
+    with pytest.raises(ValueError, match="2E"):
+        M.forward(x, x, W[:-1], 0.9, 0, 4, 2, 0)
+    with pytest.raises(ValueError, match="activation"):
+        M.forward(x, x, W, 0.9, 9, 4, 2, 0)
+    with pytest.raises(ValueError, match="same shape"):
+        M.forward(x, x[:, :16], W, 0.9, 0, 4, 2, 0)
+    with pytest.raises(TypeError):
+        M.forward(x.double(), x.double(), W, 0.9, 0, 4, 2, 0)
+    with pytest.raises(ValueError, match="unsupported"):
+        M.forward(torch.randn(1, 256, 16), torch.randn(1, 256, 16), W, 0.9, 0, 128, 2, 0)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):           # product path never runs on the CPU
+        M.forward(x, x, W, 0.9, 0, 4, 2, 0)
+
+
+def test_surface_matches_reference_names():
+    import inspect
+
+    import ncn_cuda_amd as pkg
+    assert list(inspect.signature(pkg.fused_ncn_cuda_v2).parameters) == [
+        "x", "xa", "W", "alpha", "activation", "n_cache", "n_head", "module_l"]
+    assert list(inspect.signature(pkg.NCNModuleCuda.__init__).parameters)[1:] == [
+        "alpha", "activation", "n_cache", "n_head", "module_nr", "embed_dim"]
+    assert list(inspect.signature(pkg.NCNNetCuda.__init__).parameters)[1:] == [
+        "alpha", "activation", "n_cache", "n_head", "num_modules", "embed_dim"]
+    assert list(inspect.signature(pkg.NCNNetTestCuda.__init__).parameters)[1:] == [
+        "alpha", "activation", "n_cache", "n_head", "num_modules", "weights"]
+    net = pkg.NCNNetCuda(0.9, "tanh", 4, 2, 3, 16)
+    assert sorted(net.state_dict()) == ["ncn_modules.0.weight", "ncn_modules.1.weight", "ncn_modules.2.weight"]
+    assert net.ncn_modules[1].weight.shape == (32,)
+    assert pkg.ACTIVATION_CODES == {"tanh": 0, "relu": 1, "sigmoid": 2, "linear": -1}
+
+
+def test_product_code_never_imports_the_oracle():
+    pkg_dir = os.path.join(ROOT, "ncn_cuda_amd")
+    for dirpath, _, files in os.walk(pkg_dir):
+        for f in files:
+            if f.endswith((".py", ".h", ".hip")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text.lower() or f == "never", (dirpath, f)

@@ -1,0 +1,158 @@
+"""Checks of the oracle that do not depend on any stored vector: closed forms, special cases and invariants
+chosen so that a dropped term, a wrong sign or a transposed index fails at least one of them."""
+import math
+
+import pytest
+import torch
+
+from oracle import ncn_oracle as O
+
+D = torch.float64
+
+
+def _rand(*shape, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return scale * torch.randn(*shape, generator=g, dtype=D)
+
+
+@pytest.mark.parametrize("N,n", [(256, 2), (1024, 4), (4096, 16), (8192, 2), (2048, 8), (48, 3), (64, 64)])
+def test_index_map_is_a_bijection_at_every_stage(N, n):
+    m = N // n
+    for stage in range(0, m.bit_length() + 3):
+        pos = O.stage_positions(N, n, stage)
+        assert sorted(pos.reshape(-1).tolist()) == list(range(N))
+        assert (pos % n == torch.arange(n)[None, :]).all()  # slot o always reads offset o of some block
+    assert torch.equal(O.stage_positions(N, n, 0).reshape(-1), torch.arange(N))  # stage 0: contiguous blocks
+
+
+def test_index_map_hand_values():
+    # N=256, n=2: stride 1, 2, 64 at stages 1, 2, 7
+    assert O.group_pos_to_index(256, 2, 1, 0, 1) == 3
+    assert O.group_pos_to_index(256, 2, 2, 0, 1) == 5
+    assert O.group_pos_to_index(256, 2, 7, 0, 1) == 129
+    assert O.group_pos_to_index(256, 2, 7, 5, 1) == 139
+    assert O.stage_stride(256, 2, 8) == 0  # 2^7 mod 128: the stride wraps to contiguous blocks again
+    assert O.stage_stride(48, 3, 5) == 0 and O.stage_stride(48, 3, 4) == 8  # groups = 16
+
+
+def test_single_row_group_by_hand():
+    """n = 1: one row, one step, s = <x, Wi + Wj>."""
+    E, C = 6, 2
+    x, xa, W = _rand(1, 1, E, seed=1), _rand(1, 1, E, seed=2), _rand(2 * E, seed=3, scale=0.5)
+    alpha, m = 0.7, 0.9
+    y, ya = O.stage_forward(x, xa, W, alpha, 1, C, 0, m)
+    for c in range(C):
+        sl = slice(c * 3, c * 3 + 3)
+        xv, av = x[0, 0, sl], xa[0, 0, sl]
+        s = torch.dot(xv, W[sl] + W[E + c * 3:E + c * 3 + 3])
+        F = torch.tanh(alpha * xv + (1 - alpha) * s * xv)
+        a2 = m * av + (1 - m) * F
+        assert torch.allclose(ya[0, 0, sl], a2, atol=1e-15)
+        assert torch.allclose(y[0, 0, sl], m * xv + (1 - m) * a2, atol=1e-15)
+
+
+def test_alpha_one_ignores_weights_and_grouping():
+    """alpha = 1: T = x, rows decouple, W drops out; n steps of a' = m a + (1-m) tanh x, x' = m x + (1-m) a'."""
+    x, xa = _rand(2, 16, 8, seed=4), _rand(2, 16, 8, seed=5)
+    W1, W2 = _rand(16, seed=6), _rand(16, seed=7)
+    n, C, m = 4, 2, 0.9
+    y1, ya1 = O.stage_forward(x, xa, W1, 1.0, n, C, 2, m)
+    y2, ya2 = O.stage_forward(x, xa, W2, 1.0, n, C, 0, m)
+    assert torch.allclose(y1, y2, atol=1e-14) and torch.allclose(ya1, ya2, atol=1e-14)
+    xe, ae = x.clone(), xa.clone()
+    for _ in range(n):
+        ae = m * ae + (1 - m) * torch.tanh(xe)
+        xe = m * xe + (1 - m) * ae
+    assert torch.allclose(y1, xe, atol=1e-14) and torch.allclose(ya1, ae, atol=1e-14)
+    # and dW vanishes
+    dy, dya = _rand(2, 16, 8, seed=8), _rand(2, 16, 8, seed=9)
+    *_, dW = O.stage_backward(y1, ya1, dy, dya, W1, 1.0, n, C, 2, m)
+    assert dW.abs().max().item() < 1e-15
+
+
+def test_zero_weights_decouple_rows():
+    x, xa = _rand(1, 8, 4, seed=10), _rand(1, 8, 4, seed=11)
+    alpha, m, n = 0.6, 0.9, 4
+    y, ya = O.stage_forward(x, xa, torch.zeros(8, dtype=D), alpha, n, 1, 1, m)
+    xe, ae = x.clone(), xa.clone()
+    for _ in range(n):
+        ae = m * ae + (1 - m) * torch.tanh(alpha * xe)
+        xe = m * xe + (1 - m) * ae
+    assert torch.allclose(y, xe, atol=1e-14) and torch.allclose(ya, ae, atol=1e-14)
+
+
+def test_pivot_row_uses_pre_step_value_and_step_order():
+    """Two rows, linear activation, by hand: step 0 pivots on row 0, step 1 on the UPDATED row 1."""
+    alpha, m = 0.5, 0.9
+    x = torch.tensor([[[1.0], [2.0]]], dtype=D)
+    xa = torch.zeros(1, 2, 1, dtype=D)
+    W = torch.tensor([0.3, -0.2], dtype=D)  # Wi = 0.3, Wj = -0.2
+    y, ya = O.stage_forward(x, xa, W, alpha, 2, 1, 0, m, activation="linear")
+    r = [1.0, 2.0]
+    a = [0.0, 0.0]
+    for j in range(2):
+        xj = r[j]
+        new_r, new_a = [], []
+        for i in range(2):
+            s = r[i] * 0.3 + xj * -0.2
+            T = alpha * r[i] + (1 - alpha) * s * xj
+            a2 = m * a[i] + (1 - m) * T
+            new_a.append(a2)
+            new_r.append(m * r[i] + (1 - m) * a2)
+        r, a = new_r, new_a
+    assert torch.allclose(y.reshape(-1), torch.tensor(r, dtype=D), atol=1e-15)
+    assert torch.allclose(ya.reshape(-1), torch.tensor(a, dtype=D), atol=1e-15)
+
+
+@pytest.mark.parametrize("act", ["tanh", "sigmoid", "linear"])
+def test_closed_form_backward_equals_autograd(act):
+    batch, N, E, C, n, L, alpha = 2, 24, 6, 2, 4, 4, 0.8
+    x, xa = _rand(batch, N, E, seed=12), _rand(batch, N, E, seed=13)
+    Ws = [_rand(2 * E, seed=20 + l, scale=0.4) for l in range(L)]
+    dy, dya = _rand(batch, N, E, seed=14), _rand(batch, N, E, seed=15)
+    yi, ya, dx, dxa, dWs = O.net_autograd(x, xa, Ws, dy, dya, alpha, n, C, activation=act)
+    xr, xar, dx2, dxa2, dWs2 = O.net_backward(yi, ya, dy, dya, Ws, alpha, n, C, activation=act)
+    assert O.rel_err(dx2, dx) < 1e-10 and O.rel_err(dxa2, dxa) < 1e-10
+    for l in range(L):
+        assert O.rel_err(dWs2[l], dWs[l]) < 1e-10
+    assert O.rel_err(xr, x) < 1e-11 and O.rel_err(xar, xa) < 1e-11
+    dx3, dxa3, dWs3 = O.net_backward_from_inputs(x, xa, dy, dya, Ws, alpha, n, C, activation=act)
+    assert O.rel_err(dx3, dx) < 1e-12 and O.rel_err(dWs3[0], dWs[0]) < 1e-12
+
+
+def test_inverse_round_trip_and_first_stage_offset():
+    batch, N, E, C, n, alpha = 2, 64, 8, 2, 8, 0.9
+    x, xa = _rand(batch, N, E, seed=30), _rand(batch, N, E, seed=31)
+    Ws = [_rand(2 * E, seed=40 + l, scale=0.1) for l in range(3)]
+    y, ya = O.net_forward(x, xa, Ws, alpha, n, C, first_stage=2)
+    xr, xar = O.net_inverse(y, ya, Ws, alpha, n, C, first_stage=2)
+    assert O.rel_err(xr, x) < 1e-11 and O.rel_err(xar, xa) < 1e-11
+    # stages 2,3,4 are not stages 0,1,2
+    y0, _ = O.net_forward(x, xa, Ws, alpha, n, C, first_stage=0)
+    assert O.rel_err(y0, y) > 1e-4
+
+
+def test_dw_is_additive_over_batch_shards():
+    batch, N, E, C, n, alpha = 4, 32, 8, 2, 4, 0.9
+    x, xa = _rand(batch, N, E, seed=50), _rand(batch, N, E, seed=51)
+    W = _rand(2 * E, seed=52, scale=0.4)
+    dy, dya = _rand(batch, N, E, seed=53), _rand(batch, N, E, seed=54)
+    y, ya = O.stage_forward(x, xa, W, alpha, n, C, 1)
+    *_, dW = O.stage_backward(y, ya, dy, dya, W, alpha, n, C, 1)
+    parts = [O.stage_backward(y[b:b + 2], ya[b:b + 2], dy[b:b + 2], dya[b:b + 2], W, alpha, n, C, 1)[-1]
+             for b in (0, 2)]
+    assert torch.allclose(parts[0] + parts[1], dW, atol=1e-13)
+
+
+def test_heads_use_disjoint_weight_slices():
+    """Changing head 1's slice of Wi / Wj must not move head 0's outputs, and vice versa."""
+    batch, N, E, C, n, alpha = 1, 16, 8, 2, 4, 0.8
+    x, xa = _rand(batch, N, E, seed=60), _rand(batch, N, E, seed=61)
+    W = _rand(2 * E, seed=62, scale=0.5)
+    y, _ = O.stage_forward(x, xa, W, alpha, n, C, 1)
+    W2 = W.clone()
+    W2[4:8] += 1.0          # Wi of head 1
+    W2[E + 4:E + 8] -= 1.0  # Wj of head 1
+    y2, _ = O.stage_forward(x, xa, W2, alpha, n, C, 1)
+    assert torch.equal(y[..., :4], y2[..., :4])
+    assert not torch.allclose(y[..., 4:], y2[..., 4:])
