@@ -83,6 +83,24 @@ Plan make_plan(const ncn_shape* sh, int activation) {
     return p;
 }
 
+void fill_step_table(StepTable& t, int n_cache, float alpha, float m) {
+    const double md = m, al = alpha, k2l = 2.8853900817779268;
+    t.alpha = alpha;
+    t.m = m;
+    t.m_pow_n = (float)std::pow(md, (double)n_cache);
+    t.inv_m_pow_n = (float)std::pow(md, -(double)n_cache);
+    for (int k = 0; k < 64; ++k) {
+        const double im = std::pow(md, -(double)(k + 1)), mt = std::pow(md, (double)k);
+        t.step[k].lam = (float)(k2l * al * im);
+        t.step[k].kc2 = (float)(k2l * (1.0 - al) * im * im);
+        t.step[k].kap = (float)((1.0 - md) * mt);
+        t.step[k].krho = (float)(4.0 * (1.0 - md) / md * (1.0 - al) * im);
+        t.step[k].flam = (float)(k2l * al * mt);
+        t.step[k].fkc = (float)(k2l * (1.0 - al) * mt * mt);
+        t.step[k].fkap = (float)((1.0 - md) * im);
+    }
+}
+
 void fill_common(StageArgs& a, const ncn_shape* sh, const Plan& p, int stage, float alpha, float m, int activation) {
     a.N = sh->N;
     a.E = sh->E;
@@ -95,22 +113,7 @@ void fill_common(StageArgs& a, const ncn_shape* sh, const Plan& p, int stage, fl
     a.head_dim = (int)(sh->E / sh->n_head);
     a.n_head = sh->n_head;
     a.activation = activation;
-    a.alpha = alpha;
-    a.m = m;
-    const double md = m, al = alpha, k2l = 2.8853900817779268;
-    a.m_pow_n = (float)std::pow(md, (double)sh->n_cache);
-    a.inv_m_pow_n = (float)std::pow(md, -(double)sh->n_cache);
-    for (int t = 0; t < 64; ++t) {
-        const double im = std::pow(md, -(double)(t + 1));
-        a.step[t].lam = (float)(k2l * al * im);
-        a.step[t].kc2 = (float)(k2l * (1.0 - al) * im * im);
-        a.step[t].kap = (float)((1.0 - md) * std::pow(md, (double)t));
-        a.step[t].krho = (float)(4.0 * (1.0 - md) / md * (1.0 - al) * im);
-        const double mt = std::pow(md, (double)t);
-        a.step[t].flam = (float)(k2l * al * mt);
-        a.step[t].fkc = (float)(k2l * (1.0 - al) * mt * mt);
-        a.step[t].fkap = (float)((1.0 - md) * im);
-    }
+    fill_step_table(a.tab, sh->n_cache, alpha, m);
 }
 
 }  // namespace

@@ -7,6 +7,22 @@
 
 namespace ncn {
 
+// Scalars of the recurrence, made on the host in double precision and read by the kernels through scalar loads.
+struct StepTable {
+    float alpha, m;
+    float m_pow_n, inv_m_pow_n;  // m^n_cache and its reciprocal
+    // Per-step scalars of the reversible backward / inverse, index t = number of inversion steps already done
+    // (t = 0 is the stage's last step):
+    //   im = m^-(t+1),  lam = 2 log2(e) alpha im,  kc2 = 2 log2(e) (1-alpha) im^2,
+    //   kap = (1-m) m^t,  krho = 4 (1-m)/m (1-alpha) im
+    // and of the forward, index t = number of steps already done:
+    //   flam = 2 log2(e) alpha m^t,  fkc = 2 log2(e) (1-alpha) m^2t,  fkap = (1-m) / m^(t+1)
+    struct StepScalars {
+        float lam, kc2, kap, krho;
+        float flam, fkc, fkap;
+    } step[64];
+};
+
 // Everything one stage launch needs.  Which pointer means what depends on the kernel:
 //   forward : in0,in1 = x,xa        out0,out1 = y,ya      aux0,aux1 = optional float32 copies of y,ya
 //   inverse : in0,in1 = y,ya        out0,out1 = x,xa
@@ -32,18 +48,7 @@ struct StageArgs {
     int32_t n_cache, head_dim, n_head;
     int32_t in_dtype, g_dtype, out_dtype;
     int32_t activation;
-    float alpha, m;
-    float m_pow_n, inv_m_pow_n;  // m^n_cache and its reciprocal
-    // Per-step scalars of the reversible backward, index t = number of inversion steps already done
-    // (t = 0 is the stage's last step).  Computed on the host in double precision:
-    //   im = m^-(t+1),  lam = 2 log2(e) alpha im,  kc2 = 2 log2(e) (1-alpha) im^2,
-    //   kap = (1-m) m^t,  krho = 4 (1-m)/m (1-alpha) im
-    // and of the forward, index t = number of steps already done:
-    //   flam = 2 log2(e) alpha m^t,  fkc = 2 log2(e) (1-alpha) m^2t,  fkap = (1-m) / m^(t+1)
-    struct StepScalars {
-        float lam, kc2, kap, krho;
-        float flam, fkc, fkap;
-    } step[64];
+    StepTable tab;
 };
 
 // ---------------------------------------------------------------------------------------------

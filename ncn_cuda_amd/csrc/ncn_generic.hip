@@ -42,7 +42,7 @@ __device__ __forceinline__ GenericLane generic_lane(const StageArgs& A, uint32_t
 __global__ void __launch_bounds__(64) generic_forward_kernel(const StageArgs A, const int inverse) {
     extern __shared__ float lds[];
     const int lane = threadIdx.x, head = blockIdx.y, ec = A.head_dim, n = A.n_cache;
-    const float alpha = A.alpha, m = A.m, om = 1.f - A.m, oa = 1.f - A.alpha;
+    const float alpha = A.tab.alpha, m = A.tab.m, om = 1.f - A.tab.m, oa = 1.f - A.tab.alpha;
     const float inv_m = 1.f / m, k_ba = om / m;
     const float* Wi = A.W + (int64_t)head * ec;
     const float* Wj = Wi + A.E;
@@ -100,7 +100,7 @@ __global__ void __launch_bounds__(64) generic_forward_kernel(const StageArgs A, 
 __global__ void __launch_bounds__(64) generic_backward_kernel(const StageArgs A) {
     extern __shared__ float lds[];
     const int lane = threadIdx.x, head = blockIdx.y, ec = A.head_dim, n = A.n_cache;
-    const float alpha = A.alpha, m = A.m, om = 1.f - A.m, oa = 1.f - A.alpha;
+    const float alpha = A.tab.alpha, m = A.tab.m, om = 1.f - A.tab.m, oa = 1.f - A.tab.alpha;
     const float inv_m = 1.f / m, k_ba = om / m, k1 = om * om, k2 = om, kh1 = m * om;
     const float* Wi = A.W + (int64_t)head * ec;
     const float* Wj = Wi + A.E;

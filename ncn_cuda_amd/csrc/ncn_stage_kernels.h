@@ -66,12 +66,13 @@ __device__ __forceinline__ bool tile_offsets(const StageArgs& A, uint32_t t, int
 }
 
 template <int F>
-__device__ __forceinline__ void load_w(const StageArgs& A, int head, int ec, int fl, float (&wi)[F], float (&wj)[F]) {
-    const float* w = A.W + (int64_t)head * ec + fl * F;
+__device__ __forceinline__ void load_w(const float* W, int64_t E, int head, int ec, int fl, float (&wi)[F],
+                                       float (&wj)[F]) {
+    const float* w = W + (int64_t)head * ec + fl * F;
 #pragma unroll
     for (int f = 0; f < F; ++f) {
         wi[f] = w[f];
-        wj[f] = w[A.E + f];
+        wj[f] = w[E + f];
     }
 }
 
@@ -87,154 +88,98 @@ __device__ __forceinline__ float dot_frag(const float (&a)[F], const float (&b)[
 }
 
 // ---------------------------------------------------------------------------------------------
-// forward (torch_ref/ncn_pytorch.py:74-94)
+// forward (torch_ref/ncn_pytorch.py:74-94), all n_cache steps on one register tile
 //   s_i = <x_i,Wi> + <x_j,Wj>      T = alpha x_i + (1-alpha) s_i x_j      F = tanh T = 1 - 2r,
 //   r = 1/(1 + exp(2T))            a' = m a + (1-m) F                     x' = m x + (1-m) a'
 // The registers hold X = x / m^t and A = xa / m^t after t steps, which turns the two updates into
 //   A <- A + (1-m)/m^(t+1) F   and   X <- X + (1-m) A   (the powers of m come from a host-made table).
 // ---------------------------------------------------------------------------------------------
-template <int NC, int EC, int R, int F, int WPE = 1>
-__global__ void __launch_bounds__(kBlockThreads, WPE) stage_forward_kernel(const StageArgs A) {
+template <int NC, int EC, int R, int F>
+__device__ __forceinline__ void forward_steps(float (&x)[R][F], float (&a)[R][F], const float (&wi)[F],
+                                              const float (&wj)[F], const StepTable& S, int lane, float4* slots) {
     using T = Tile<NC, EC, R, F>;
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const uint32_t nwaves = gridDim.x * kWavesPerBlock;
-    const uint32_t gwave = blockIdx.x * kWavesPerBlock + wave;
-    const int head = gwave % A.n_head;
-    const uint32_t tile_step = nwaves / A.n_head;
-    __shared__ float4 bcast_lds[T::LR == 1 ? 1 : kWavesPerBlock * (F / 4) * 64];
-    float4* slots = bcast_lds + (T::LR == 1 ? 0 : wave * (F / 4) * 64);
-    const int fl = lane % T::LF;
-    const float om = 1.0f - A.m;
-
-    float wi[F], wj[F];
-    load_w<F>(A, head, EC, fl, wi, wj);
-
-    for (uint32_t t = gwave / A.n_head; t < A.total_tiles; t += tile_step) {
-        int64_t off[R];
-        const bool valid = tile_offsets<NC, EC, R, F>(A, t, lane, head, off);
-        float x[R][F], a[R][F];
-#pragma unroll
-        for (int rr = 0; rr < R; ++rr) {
-            load_frag<F>(A.in0, A.in_dtype, off[rr], valid, x[rr]);
-            load_frag<F>(A.in1, A.in_dtype, off[rr], valid, a[rr]);
-        }
-
+    const float om = 1.0f - S.m;
 #pragma unroll 1
-        for (int jo = 0; jo < T::LR; ++jo) {
+    for (int jo = 0; jo < T::LR; ++jo) {
 #pragma unroll
-            for (int jr = 0; jr < R; ++jr) {
-                const int ts = jo * R + jr;            // steps done so far
-                const float lam = A.step[ts].flam;     // z = lam X_i + c_i Xj
-                const float kc = A.step[ts].fkc;       // c_i = kc S_i
-                const float kap = A.step[ts].fkap;     // A <- A + kap F
-                float xj[F];
-                row_lane_broadcast<T::LF, T::LR, F>(x[jr], xj, jo, lane, slots);
-                const float e = dot_frag<F>(xj, wj);
-                // pivot row last: its registers are the source of xj when LR == 1
+        for (int jr = 0; jr < R; ++jr) {
+            const int ts = jo * R + jr;            // steps done so far
+            const float lam = S.step[ts].flam;     // z = lam X_i + c_i Xj
+            const float kc = S.step[ts].fkc;       // c_i = kc S_i
+            const float kap = S.step[ts].fkap;     // A <- A + kap F
+            float xj[F];
+            row_lane_broadcast<T::LF, T::LR, F>(x[jr], xj, jo, lane, slots);
+            const float e = dot_frag<F>(xj, wj);
+            // pivot row last: its registers are the source of xj when LR == 1
 #pragma unroll
-                for (int k = 1; k <= R; ++k) {
-                    const int rr = (jr + k) % R;
-                    const float s = lane_sum<1, T::LF>(dot_frag<F>(x[rr], wi) + e);
-                    const float c = kc * s;
+            for (int k = 1; k <= R; ++k) {
+                const int rr = (jr + k) % R;
+                const float s = lane_sum<1, T::LF>(dot_frag<F>(x[rr], wi) + e);
+                const float c = kc * s;
 #pragma unroll
-                    for (int f = 0; f < F; ++f) {
-                        const float z = fmaf(c, xj[f], lam * x[rr][f]);
-                        const float r = __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(z) + 1.0f);
-                        a[rr][f] = fmaf(-2.0f * kap, r, a[rr][f] + kap);
-                        x[rr][f] = fmaf(om, a[rr][f], x[rr][f]);
-                    }
+                for (int f = 0; f < F; ++f) {
+                    const float z = fmaf(c, xj[f], lam * x[rr][f]);
+                    const float r = __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(z) + 1.0f);
+                    a[rr][f] = fmaf(-2.0f * kap, r, a[rr][f] + kap);
+                    x[rr][f] = fmaf(om, a[rr][f], x[rr][f]);
                 }
             }
         }
-        const float dn = A.m_pow_n;
-#pragma unroll
-        for (int rr = 0; rr < R; ++rr) {
-#pragma unroll
-            for (int f = 0; f < F; ++f) {
-                x[rr][f] *= dn;
-                a[rr][f] *= dn;
-            }
-            store_frag<F>(A.out0, A.out_dtype, off[rr], valid, x[rr]);
-            store_frag<F>(A.out1, A.out_dtype, off[rr], valid, a[rr]);
-            if (A.aux0) {
-                store_frag<F>(A.aux0, NCN_F32, off[rr], valid, x[rr]);
-                store_frag<F>(A.aux1, NCN_F32, off[rr], valid, a[rr]);
-            }
-        }
     }
+    const float dn = S.m_pow_n;
+#pragma unroll
+    for (int rr = 0; rr < R; ++rr)
+#pragma unroll
+        for (int f = 0; f < F; ++f) {
+            x[rr][f] *= dn;
+            a[rr][f] *= dn;
+        }
 }
 
 // ---------------------------------------------------------------------------------------------
 // inverse (torch_ref/ncn_pytorch_invertible.py:87-113), steps j = n_cache-1 .. 0
 //   x = (y - (1-m) b)/m       recompute r from x        a = (b - (1-m) F)/m
-// with the same m^t scaling of the registers as the backward kernel below (Y = m^t x, B = m^t xa).
+// with the same m^t scaling of the registers as the backward below (Y = m^t x, B = m^t xa).
 // ---------------------------------------------------------------------------------------------
-template <int NC, int EC, int R, int F, int WPE = 1>
-__global__ void __launch_bounds__(kBlockThreads, WPE) stage_inverse_kernel(const StageArgs A) {
+template <int NC, int EC, int R, int F>
+__device__ __forceinline__ void inverse_steps(float (&y)[R][F], float (&b)[R][F], const float (&wi)[F],
+                                              const float (&wj)[F], const StepTable& S, int lane, float4* slots) {
     using T = Tile<NC, EC, R, F>;
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const uint32_t nwaves = gridDim.x * kWavesPerBlock;
-    const uint32_t gwave = blockIdx.x * kWavesPerBlock + wave;
-    const int head = gwave % A.n_head;
-    const uint32_t tile_step = nwaves / A.n_head;
-    __shared__ float4 bcast_lds[T::LR == 1 ? 1 : kWavesPerBlock * (F / 4) * 64];
-    float4* slots = bcast_lds + (T::LR == 1 ? 0 : wave * (F / 4) * 64);
-    const int fl = lane % T::LF;
-    const float nom = A.m - 1.0f;
-
-    float wi[F], wj[F];
-    load_w<F>(A, head, EC, fl, wi, wj);
-
-    for (uint32_t t = gwave / A.n_head; t < A.total_tiles; t += tile_step) {
-        int64_t off[R];
-        const bool valid = tile_offsets<NC, EC, R, F>(A, t, lane, head, off);
-        float y[R][F], b[R][F];
-#pragma unroll
-        for (int rr = 0; rr < R; ++rr) {
-            load_frag<F>(A.in0, A.in_dtype, off[rr], valid, y[rr]);
-            load_frag<F>(A.in1, A.in_dtype, off[rr], valid, b[rr]);
-        }
-
+    const float nom = S.m - 1.0f;
 #pragma unroll 1
-        for (int jo = T::LR - 1; jo >= 0; --jo) {
+    for (int jo = T::LR - 1; jo >= 0; --jo) {
 #pragma unroll
-            for (int jr = R - 1; jr >= 0; --jr) {
-                const int ts = (T::LR - 1 - jo) * R + (R - 1 - jr);   // inversion steps done so far
-                const float lam = A.step[ts].lam, kc2 = A.step[ts].kc2, kap = A.step[ts].kap;
+        for (int jr = R - 1; jr >= 0; --jr) {
+            const int ts = (T::LR - 1 - jo) * R + (R - 1 - jr);   // inversion steps done so far
+            const float lam = S.step[ts].lam, kc2 = S.step[ts].kc2, kap = S.step[ts].kap;
 #pragma unroll
-                for (int rr = 0; rr < R; ++rr)
+            for (int rr = 0; rr < R; ++rr)
 #pragma unroll
-                    for (int f = 0; f < F; ++f) y[rr][f] = fmaf(nom, b[rr][f], y[rr][f]);
-                float xj[F];
-                row_lane_broadcast<T::LF, T::LR, F>(y[jr], xj, jo, lane, slots);
-                const float e = dot_frag<F>(xj, wj);
+                for (int f = 0; f < F; ++f) y[rr][f] = fmaf(nom, b[rr][f], y[rr][f]);
+            float xj[F];
+            row_lane_broadcast<T::LF, T::LR, F>(y[jr], xj, jo, lane, slots);
+            const float e = dot_frag<F>(xj, wj);
 #pragma unroll
-                for (int rr = 0; rr < R; ++rr) {
-                    const float s = lane_sum<1, T::LF>(dot_frag<F>(y[rr], wi) + e);
-                    const float c = kc2 * s;
+            for (int rr = 0; rr < R; ++rr) {
+                const float s = lane_sum<1, T::LF>(dot_frag<F>(y[rr], wi) + e);
+                const float c = kc2 * s;
 #pragma unroll
-                    for (int f = 0; f < F; ++f) {
-                        const float z = fmaf(c, xj[f], lam * y[rr][f]);
-                        const float r = __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(z) + 1.0f);
-                        b[rr][f] = fmaf(2.0f * kap, r, b[rr][f] - kap);
-                    }
+                for (int f = 0; f < F; ++f) {
+                    const float z = fmaf(c, xj[f], lam * y[rr][f]);
+                    const float r = __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(z) + 1.0f);
+                    b[rr][f] = fmaf(2.0f * kap, r, b[rr][f] - kap);
                 }
             }
         }
-        const float up = A.inv_m_pow_n;
-#pragma unroll
-        for (int rr = 0; rr < R; ++rr) {
-#pragma unroll
-            for (int f = 0; f < F; ++f) {
-                y[rr][f] *= up;
-                b[rr][f] *= up;
-            }
-            store_frag<F>(A.out0, A.out_dtype, off[rr], valid, y[rr]);
-            store_frag<F>(A.out1, A.out_dtype, off[rr], valid, b[rr]);
-        }
     }
+    const float up = S.inv_m_pow_n;
+#pragma unroll
+    for (int rr = 0; rr < R; ++rr)
+#pragma unroll
+        for (int f = 0; f < F; ++f) {
+            y[rr][f] *= up;
+            b[rr][f] *= up;
+        }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -250,27 +195,163 @@ __global__ void __launch_bounds__(kBlockThreads, WPE) stage_inverse_kernel(const
 // folded into per-step scalars: after t inversion steps the registers hold
 //   Y = m^t x,   B = m^t xa,   G = g / m^t,   P = p / m^t,
 // which turns  x <- (y - (1-m) b)/m  into  Y <- Y - (1-m) B,   g <- m g + ..  into  G <- G + ../m^(t+1)
-// and  p <- (1-m) g + m p  into  P <- P + (1-m) G  (one FMA each); the powers of m are kept in double.
+// and  p <- (1-m) g + m p  into  P <- P + (1-m) G  (one FMA each).
+//
+// On entry Y, B = stage outputs, G, H = their gradients; on exit G, H = gradients of the stage inputs and
+// Y, B = m^n_cache times the stage inputs (multiply by StepTable::inv_m_pow_n before storing them).
+// dwi, dwj accumulate this lane's share of dWi, dWj; with MASKED the share is weighted by `own` (1, or 0 for a
+// group whose dW another tile accounts for).
 // ---------------------------------------------------------------------------------------------
+template <int NC, int EC, int R, int F, bool MASKED>
+__device__ __forceinline__ void backward_steps(float (&Y)[R][F], float (&B)[R][F], float (&G)[R][F], float (&P)[R][F],
+                                               const float (&wi)[F], const float (&wj)[F], float (&dwi)[F],
+                                               float (&dwj)[F], float own, const StepTable& S, int lane,
+                                               float4* slots) {
+    using T = Tile<NC, EC, R, F>;
+    const int rl = (lane / T::LF) % T::LR;
+    const float om = 1.0f - S.m;
+    const float ku = 4.0f * om / S.m * S.alpha;  // G += ku * U        (U = P (r - r^2))
+    const float nom = -om;
+#pragma unroll
+    for (int rr = 0; rr < R; ++rr)
+#pragma unroll
+        for (int f = 0; f < F; ++f) P[rr][f] = fmaf(om, G[rr][f], P[rr][f]);  // h -> p
+
+#pragma unroll 1
+    for (int jo = T::LR - 1; jo >= 0; --jo) {
+        const float sel = (T::LR == 1 || rl == jo) ? 1.0f : 0.0f;  // this lane holds the pivot row
+#pragma unroll
+        for (int jr = R - 1; jr >= 0; --jr) {
+            const int ts = (T::LR - 1 - jo) * R + (R - 1 - jr);   // inversion steps done so far
+            const float lam = S.step[ts].lam;     // z = lam Y_i + chat_i Yj
+            const float kc2 = S.step[ts].kc2;     // chat_i = kc2 S_i
+            const float kap = S.step[ts].kap;     // B <- B - kap F
+            const float krho = S.step[ts].krho;   // rho_i = krho <U_i, Yj>
+#pragma unroll
+            for (int rr = 0; rr < R; ++rr)
+#pragma unroll
+                for (int f = 0; f < F; ++f) Y[rr][f] = fmaf(nom, B[rr][f], Y[rr][f]);  // m^(t+1) x of this step
+            float xj[F], v[F];
+            row_lane_broadcast<T::LF, T::LR, F>(Y[jr], xj, jo, lane, slots);
+#pragma unroll
+            for (int f = 0; f < F; ++f) v[f] = 0.f;
+            const float e = dot_frag<F>(xj, wj);
+            float rhosum = 0.f;
+#pragma unroll
+            for (int rr = 0; rr < R; ++rr) {
+                const float Ssum = lane_sum<1, T::LF>(dot_frag<F>(Y[rr], wi) + e);
+                const float chat = kc2 * Ssum;
+                float u[F];
+                float rh = 0.f;
+#pragma unroll
+                for (int f = 0; f < F; ++f) {
+                    const float z = fmaf(chat, xj[f], lam * Y[rr][f]);
+                    const float r = __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(z) + 1.0f);
+                    B[rr][f] = fmaf(2.0f * kap, r, B[rr][f] - kap);   // m^(t+1) xa of this step
+                    u[f] = P[rr][f] * fmaf(-r, r, r);
+                    rh = fmaf(u[f], xj[f], rh);
+                }
+                rh = lane_sum<1, T::LF>(rh);
+                const float rho = krho * rh;       // (1-alpha) r_i / m^(t+1)
+                const float c4 = krho * Ssum;      // (1-alpha) s_i u-scale / m^(t+1)
+                const float rho_w = MASKED ? rho * own : rho;
+                rhosum += rho;
+#pragma unroll
+                for (int f = 0; f < F; ++f) {
+                    dwi[f] = fmaf(rho_w, Y[rr][f], dwi[f]);
+                    v[f] = fmaf(c4, u[f], v[f]);
+                    G[rr][f] = fmaf(rho, wi[f], fmaf(ku, u[f], G[rr][f]));
+                    if (rr != jr) P[rr][f] = fmaf(om, G[rr][f], P[rr][f]);
+                }
+            }
+            const float rhosum_w = MASKED ? rhosum * own : rhosum;
+#pragma unroll
+            for (int f = 0; f < F; ++f) {
+                dwj[f] = fmaf(rhosum_w, xj[f], dwj[f]);
+                const float vt = lane_sum<T::LF, T::LPG>(fmaf(rhosum, wj[f], v[f]));  // over the group's row lanes
+                G[jr][f] = fmaf(sel, vt, G[jr][f]);
+                P[jr][f] = fmaf(om, G[jr][f], P[jr][f]);
+            }
+            __builtin_amdgcn_sched_barrier(0);  // keep steps apart: interleaving them only costs registers
+        }
+    }
+    // undo the scaling of the gradients: NC steps done
+    const float dn = S.m_pow_n;       // m^NC
+#pragma unroll
+    for (int rr = 0; rr < R; ++rr)
+#pragma unroll
+        for (int f = 0; f < F; ++f) {
+            G[rr][f] *= dn;
+            P[rr][f] = fmaf(P[rr][f], dn, nom * G[rr][f]);  // back to h = p - (1-m) g
+        }
+}
+
+// ---------------------------------------------------------------------------------------------
+// One-stage kernels: gather the register tile from HBM, run the steps, scatter.
+// ---------------------------------------------------------------------------------------------
+#define NCN_WAVE_PROLOGUE                                                                       \
+    using T = Tile<NC, EC, R, F>;                                                               \
+    const int lane = threadIdx.x & 63;                                                          \
+    const int wave = threadIdx.x >> 6;                                                          \
+    const uint32_t nwaves = gridDim.x * kWavesPerBlock;                                         \
+    const uint32_t gwave = blockIdx.x * kWavesPerBlock + wave;                                  \
+    const int head = gwave % A.n_head;                                                          \
+    const uint32_t tile_step = nwaves / A.n_head;                                               \
+    __shared__ float4 bcast_lds[T::LR == 1 ? 1 : kWavesPerBlock * (F / 4) * 64];                \
+    float4* slots = bcast_lds + (T::LR == 1 ? 0 : wave * (F / 4) * 64);                         \
+    const int fl = lane % T::LF;                                                                \
+    float wi[F], wj[F];                                                                         \
+    load_w<F>(A.W, A.E, head, EC, fl, wi, wj);
+
+template <int NC, int EC, int R, int F, int WPE = 1>
+__global__ void __launch_bounds__(kBlockThreads, WPE) stage_forward_kernel(const StageArgs A) {
+    NCN_WAVE_PROLOGUE
+    for (uint32_t t = gwave / A.n_head; t < A.total_tiles; t += tile_step) {
+        int64_t off[R];
+        const bool valid = tile_offsets<NC, EC, R, F>(A, t, lane, head, off);
+        float x[R][F], a[R][F];
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) {
+            load_frag<F>(A.in0, A.in_dtype, off[rr], valid, x[rr]);
+            load_frag<F>(A.in1, A.in_dtype, off[rr], valid, a[rr]);
+        }
+        forward_steps<NC, EC, R, F>(x, a, wi, wj, A.tab, lane, slots);
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) {
+            store_frag<F>(A.out0, A.out_dtype, off[rr], valid, x[rr]);
+            store_frag<F>(A.out1, A.out_dtype, off[rr], valid, a[rr]);
+            if (A.aux0) {
+                store_frag<F>(A.aux0, NCN_F32, off[rr], valid, x[rr]);
+                store_frag<F>(A.aux1, NCN_F32, off[rr], valid, a[rr]);
+            }
+        }
+    }
+}
+
+template <int NC, int EC, int R, int F, int WPE = 1>
+__global__ void __launch_bounds__(kBlockThreads, WPE) stage_inverse_kernel(const StageArgs A) {
+    NCN_WAVE_PROLOGUE
+    for (uint32_t t = gwave / A.n_head; t < A.total_tiles; t += tile_step) {
+        int64_t off[R];
+        const bool valid = tile_offsets<NC, EC, R, F>(A, t, lane, head, off);
+        float y[R][F], b[R][F];
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) {
+            load_frag<F>(A.in0, A.in_dtype, off[rr], valid, y[rr]);
+            load_frag<F>(A.in1, A.in_dtype, off[rr], valid, b[rr]);
+        }
+        inverse_steps<NC, EC, R, F>(y, b, wi, wj, A.tab, lane, slots);
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) {
+            store_frag<F>(A.out0, A.out_dtype, off[rr], valid, y[rr]);
+            store_frag<F>(A.out1, A.out_dtype, off[rr], valid, b[rr]);
+        }
+    }
+}
+
 template <int NC, int EC, int R, int F, int WPE = 1>
 __global__ void __launch_bounds__(kBlockThreads, WPE) stage_backward_kernel(const StageArgs A) {
-    using T = Tile<NC, EC, R, F>;
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const uint32_t nwaves = gridDim.x * kWavesPerBlock;
-    const uint32_t gwave = blockIdx.x * kWavesPerBlock + wave;
-    const int head = gwave % A.n_head;
-    const uint32_t tile_step = nwaves / A.n_head;
-    __shared__ float4 bcast_lds[T::LR == 1 ? 1 : kWavesPerBlock * (F / 4) * 64];
-    float4* slots = bcast_lds + (T::LR == 1 ? 0 : wave * (F / 4) * 64);
-    const int fl = lane % T::LF;
-    const int rl = (lane / T::LF) % T::LR;
-    const float alpha = A.alpha, om = 1.0f - A.m;
-    const float ku = 4.0f * om / A.m * alpha;  // G += ku * U        (U = P (r - r^2))
-    const float nom = -om;
-
-    float wi[F], wj[F];
-    load_w<F>(A, head, EC, fl, wi, wj);
+    NCN_WAVE_PROLOGUE
     float dwi[F], dwj[F];
 #pragma unroll
     for (int f = 0; f < F; ++f) dwi[f] = dwj[f] = 0.f;
@@ -278,89 +359,24 @@ __global__ void __launch_bounds__(kBlockThreads, WPE) stage_backward_kernel(cons
     for (uint32_t t = gwave / A.n_head; t < A.total_tiles; t += tile_step) {
         int64_t off[R];
         const bool valid = tile_offsets<NC, EC, R, F>(A, t, lane, head, off);
-        float Y[R][F], B[R][F], G[R][F], P[R][F];
+        float Y[R][F], B[R][F], G[R][F], H[R][F];
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) {
             load_frag<F>(A.in0, A.in_dtype, off[rr], valid, Y[rr]);
             load_frag<F>(A.in1, A.in_dtype, off[rr], valid, B[rr]);
             load_frag<F>(A.g0, A.g_dtype, off[rr], valid, G[rr]);
-            load_frag<F>(A.g1, A.g_dtype, off[rr], valid && A.g1 != nullptr, P[rr]);
-#pragma unroll
-            for (int f = 0; f < F; ++f) P[rr][f] = fmaf(om, G[rr][f], P[rr][f]);
+            load_frag<F>(A.g1, A.g_dtype, off[rr], valid && A.g1 != nullptr, H[rr]);
         }
-#pragma unroll 1
-        for (int jo = T::LR - 1; jo >= 0; --jo) {
-            const float sel = (T::LR == 1 || rl == jo) ? 1.0f : 0.0f;  // this lane holds the pivot row
-#pragma unroll
-            for (int jr = R - 1; jr >= 0; --jr) {
-                const int ts = (T::LR - 1 - jo) * R + (R - 1 - jr);   // inversion steps done so far
-                const float lam = A.step[ts].lam;     // z = lam Y_i + chat_i Yj
-                const float kc2 = A.step[ts].kc2;     // chat_i = kc2 S_i
-                const float kap = A.step[ts].kap;     // B <- B - kap F
-                const float krho = A.step[ts].krho;   // rho_i = krho <U_i, Yj>
-#pragma unroll
-                for (int rr = 0; rr < R; ++rr)
-#pragma unroll
-                    for (int f = 0; f < F; ++f) Y[rr][f] = fmaf(nom, B[rr][f], Y[rr][f]);  // m^(t+1) x of this step
-                float xj[F], v[F];
-                row_lane_broadcast<T::LF, T::LR, F>(Y[jr], xj, jo, lane, slots);
-#pragma unroll
-                for (int f = 0; f < F; ++f) v[f] = 0.f;
-                const float e = dot_frag<F>(xj, wj);
-                float rhosum = 0.f;
-#pragma unroll
-                for (int rr = 0; rr < R; ++rr) {
-                    const float S = lane_sum<1, T::LF>(dot_frag<F>(Y[rr], wi) + e);
-                    const float chat = kc2 * S;
-                    float u[F];
-                    float rh = 0.f;
-#pragma unroll
-                    for (int f = 0; f < F; ++f) {
-                        const float z = fmaf(chat, xj[f], lam * Y[rr][f]);
-                        const float r = __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(z) + 1.0f);
-                        B[rr][f] = fmaf(2.0f * kap, r, B[rr][f] - kap);   // m^(t+1) xa of this step
-                        u[f] = P[rr][f] * fmaf(-r, r, r);
-                        rh = fmaf(u[f], xj[f], rh);
-                    }
-                    rh = lane_sum<1, T::LF>(rh);
-                    const float rho = krho * rh;     // (1-alpha) r_i / m^(t+1)
-                    const float c4 = krho * S;       // (1-alpha) s_i u-scale / m^(t+1)
-                    rhosum += rho;
-#pragma unroll
-                    for (int f = 0; f < F; ++f) {
-                        dwi[f] = fmaf(rho, Y[rr][f], dwi[f]);
-                        v[f] = fmaf(c4, u[f], v[f]);
-                        G[rr][f] = fmaf(rho, wi[f], fmaf(ku, u[f], G[rr][f]));
-                        if (rr != jr) P[rr][f] = fmaf(om, G[rr][f], P[rr][f]);
-                    }
-                }
-#pragma unroll
-                for (int f = 0; f < F; ++f) {
-                    dwj[f] = fmaf(rhosum, xj[f], dwj[f]);
-                    const float vt = lane_sum<T::LF, T::LPG>(fmaf(rhosum, wj[f], v[f]));  // over the group's row lanes
-                    G[jr][f] = fmaf(sel, vt, G[jr][f]);
-                    P[jr][f] = fmaf(om, G[jr][f], P[jr][f]);
-                }
-                __builtin_amdgcn_sched_barrier(0);  // keep steps apart: interleaving them only costs registers
-            }
-        }
-        // undo the scalings: t = NC steps done
-        const float up = A.inv_m_pow_n;   // m^-NC
-        const float dn = A.m_pow_n;       // m^NC
+        backward_steps<NC, EC, R, F, false>(Y, B, G, H, wi, wj, dwi, dwj, 1.0f, A.tab, lane, slots);
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) {
-#pragma unroll
-            for (int f = 0; f < F; ++f) {
-                G[rr][f] *= dn;
-                P[rr][f] = fmaf(P[rr][f], dn, nom * G[rr][f]);  // back to h = p - (1-m) g
-            }
             store_frag<F>(A.out0, A.out_dtype, off[rr], valid, G[rr]);
-            store_frag<F>(A.out1, A.out_dtype, off[rr], valid, P[rr]);
+            store_frag<F>(A.out1, A.out_dtype, off[rr], valid, H[rr]);
             if (A.aux0) {
 #pragma unroll
                 for (int f = 0; f < F; ++f) {
-                    Y[rr][f] *= up;
-                    B[rr][f] *= up;
+                    Y[rr][f] *= A.tab.inv_m_pow_n;
+                    B[rr][f] *= A.tab.inv_m_pow_n;
                 }
                 store_frag<F>(A.aux0, NCN_F32, off[rr], valid, Y[rr]);
                 store_frag<F>(A.aux1, NCN_F32, off[rr], valid, B[rr]);
@@ -383,5 +399,6 @@ __global__ void __launch_bounds__(kBlockThreads, WPE) stage_backward_kernel(cons
         }
     }
 }
+#undef NCN_WAVE_PROLOGUE
 
 }  // namespace ncn
