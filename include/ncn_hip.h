@@ -78,11 +78,16 @@ typedef struct ncn_shape {
  * y32, ya32   out  optional (NULL to skip) float32 copies of the final y, ya: what a bf16 caller saves
  *                  for the reversible backward.
  * W           in   [n_stages, 2E] float32
+ * workspace        optional scratch (NULL, 0 to skip).  With n_stages > 1 and small groups the library keeps
+ *                  tiles of rows in LDS across several stages instead of launching stage by stage; when that
+ *                  takes more than one pass it needs ncn_workspace_bytes_stages(.., backward = 0) bytes here
+ *                  and float32 outputs, and silently falls back to one launch per stage without them.
  */
 int ncn_forward(const void* x, const void* xa, int in_dtype,
                 void* y, void* ya, int out_dtype,
                 float* y32, float* ya32,
                 const float* W,
+                void* workspace, size_t workspace_bytes,
                 const ncn_shape* shape, int first_stage, int n_stages,
                 float alpha, float m, int activation, void* stream);
 
@@ -102,7 +107,9 @@ int ncn_forward(const void* x, const void* xa, int in_dtype,
  *                  the four of x_rec, xa_rec, dx, dxa carry the state between stages in place.
  * W           in   [n_stages, 2E] float32
  * dW          out  [n_stages, 2E] float32, overwritten (summed over batch, groups and rows)
- * workspace        scratch of at least ncn_workspace_bytes(shape) bytes
+ * workspace        scratch of at least ncn_workspace_bytes(shape) bytes; with n_stages > 1,
+ *                  ncn_workspace_bytes_stages(.., backward = 1) bytes let the library use its multi-stage
+ *                  LDS-resident passes (it falls back to one launch per stage with less)
  */
 int ncn_backward(const void* y, const void* ya, int y_dtype,
                  const void* dy, const void* dya, int dy_dtype,
@@ -128,6 +135,11 @@ int ncn_inverse(const void* y, const void* ya, int in_dtype,
 /* Bytes of scratch ncn_backward needs for this shape (0 on an invalid shape).  No reference counterpart:
  * the reference allocates a [batch,N,2E] partial-dW tensor per call (ncn_bwd_cuda_kernel.cu:251). */
 size_t ncn_workspace_bytes(const ncn_shape* shape);
+
+/* Bytes of scratch that let ncn_forward (backward = 0) or ncn_backward (backward = 1) run stages
+ * first_stage .. first_stage+n_stages-1 with the multi-stage passes; never less than what the call needs anyway
+ * (0 for forward, ncn_workspace_bytes for backward).  No reference counterpart. */
+size_t ncn_workspace_bytes_stages(const ncn_shape* shape, int first_stage, int n_stages, int activation, int backward);
 
 /* 2: hand-tuned register kernel, 1: generic LDS kernel, 0: not supported (n_cache > 64, or the
  * head width does not fit the generic kernel's LDS).  No reference counterpart. */

@@ -11,7 +11,8 @@ LIB_PATH = os.path.join(PKG_DIR, "libncn_hip.so")
 NCN_F32, NCN_BF16 = 0, 1
 ACT_TANH, ACT_RELU, ACT_SIGMOID, ACT_LINEAR = 0, 1, 2, -1
 
-EXPORTS = ("ncn_forward", "ncn_backward", "ncn_inverse", "ncn_workspace_bytes", "ncn_kernel_path",
+EXPORTS = ("ncn_forward", "ncn_backward", "ncn_inverse", "ncn_workspace_bytes", "ncn_workspace_bytes_stages",
+           "ncn_kernel_path",
            "ncn_check_shape", "ncn_error_string", "ncn_version")
 
 
@@ -36,7 +37,7 @@ def load():
     vp, f32p, shp = ctypes.c_void_p, ctypes.c_void_p, ctypes.POINTER(NcnShape)
     i, fl = ctypes.c_int, ctypes.c_float
     lib.ncn_forward.restype = i
-    lib.ncn_forward.argtypes = [vp, vp, i, vp, vp, i, f32p, f32p, f32p, shp, i, i, fl, fl, i, vp]
+    lib.ncn_forward.argtypes = [vp, vp, i, vp, vp, i, f32p, f32p, f32p, vp, ctypes.c_size_t, shp, i, i, fl, fl, i, vp]
     lib.ncn_backward.restype = i
     lib.ncn_backward.argtypes = [vp, vp, i, vp, vp, i, vp, vp, i, f32p, f32p, f32p, f32p, vp, ctypes.c_size_t,
                                  shp, i, i, fl, fl, i, vp]
@@ -44,6 +45,8 @@ def load():
     lib.ncn_inverse.argtypes = [vp, vp, i, vp, vp, i, f32p, shp, i, i, fl, fl, i, vp]
     lib.ncn_workspace_bytes.restype = ctypes.c_size_t
     lib.ncn_workspace_bytes.argtypes = [shp]
+    lib.ncn_workspace_bytes_stages.restype = ctypes.c_size_t
+    lib.ncn_workspace_bytes_stages.argtypes = [shp, i, i, i, i]
     lib.ncn_kernel_path.restype = i
     lib.ncn_kernel_path.argtypes = [shp]
     lib.ncn_check_shape.restype = i

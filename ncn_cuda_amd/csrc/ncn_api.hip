@@ -4,6 +4,7 @@
 #include <cmath>
 
 #include "../../include/ncn_hip.h"
+#include "ncn_fused_kernels.h"
 #include "ncn_launch.h"
 
 namespace {
@@ -116,6 +117,26 @@ void fill_common(StageArgs& a, const ncn_shape* sh, const Plan& p, int stage, fl
     fill_step_table(a.tab, sh->n_cache, alpha, m);
 }
 
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+size_t base_workspace_bytes(const ncn_shape* sh) {
+    return align256((size_t)(kMaxGridX + kReduceLevel1Rows) * 2 * (size_t)sh->E * sizeof(float));
+}
+
+// the multi-stage plan of a stage range, or an empty vector when the one-stage loop should be used
+std::vector<FusedPass> multi_stage_plan(const ncn_shape* sh, int first_stage, int n_stages, int activation, bool backward) {
+    std::vector<FusedPass> none;
+    if (n_stages < 2 || kernel_path(sh, activation) != 2 || !fused_supported(sh, activation)) return none;
+    std::vector<FusedPass> passes = plan_fused(sh, first_stage, n_stages, backward);
+    bool any = false;
+    for (const FusedPass& p : passes) any = any || !p.single;
+    return any ? passes : none;
+}
+
+size_t temp_bytes(const ncn_shape* sh, bool backward) {
+    return align256((size_t)sh->batch * sh->N * sh->E * sizeof(float)) * (backward ? 4 : 2);
+}
+
 }  // namespace
 
 extern "C" {
@@ -152,22 +173,75 @@ int ncn_kernel_path(const ncn_shape* shape) {
 
 size_t ncn_workspace_bytes(const ncn_shape* shape) {
     if (check_shape(shape, 0, 1, NCN_ACT_TANH) != NCN_OK) return 0;
-    return (size_t)(kMaxGridX + kReduceLevel1Rows) * 2 * (size_t)shape->E * sizeof(float);
+    return base_workspace_bytes(shape);
+}
+
+size_t ncn_workspace_bytes_stages(const ncn_shape* shape, int first_stage, int n_stages, int activation, int backward) {
+    if (check_shape(shape, first_stage, n_stages, activation) != NCN_OK) return 0;
+    const size_t base = backward ? base_workspace_bytes(shape) : 0;
+    const std::vector<FusedPass> passes = multi_stage_plan(shape, first_stage, n_stages, activation, backward != 0);
+    return passes.size() >= 2 ? base + temp_bytes(shape, backward != 0) : base;
 }
 
 int ncn_forward(const void* x, const void* xa, int in_dtype, void* y, void* ya, int out_dtype, float* y32, float* ya32,
-                const float* W, const ncn_shape* shape, int first_stage, int n_stages, float alpha, float m,
-                int activation, void* stream) {
+                const float* W, void* workspace, size_t workspace_bytes, const ncn_shape* shape, int first_stage,
+                int n_stages, float alpha, float m, int activation, void* stream) {
     int rc = check_shape(shape, first_stage, n_stages, activation);
     if (rc != NCN_OK) return rc;
     if (!x || !xa || !y || !ya || !W) return NCN_ERR_NULL;
     if ((y32 == nullptr) != (ya32 == nullptr)) return NCN_ERR_NULL;
     if (!known_dtype(in_dtype) || !known_dtype(out_dtype)) return NCN_ERR_DTYPE;
     if (!aligned16(x) || !aligned16(xa) || !aligned16(y) || !aligned16(ya) || !aligned16(W) || !aligned16(y32) ||
-        !aligned16(ya32))
+        !aligned16(ya32) || !aligned16(workspace))
         return NCN_ERR_ALIGN;
     const Plan p = make_plan(shape, activation);
     hipStream_t s = static_cast<hipStream_t>(stream);
+    const int64_t wstride = 2 * shape->E;
+
+    // several stages: LDS-resident passes when the shape allows and the buffers permit the ping-pong
+    std::vector<FusedPass> passes = multi_stage_plan(shape, first_stage, n_stages, activation, false);
+    const size_t np = passes.size();
+    bool fused_ok = np > 0;
+    if (np >= 2 && (out_dtype != NCN_F32 || !workspace || workspace_bytes < temp_bytes(shape, false))) fused_ok = false;
+    if (np == 1 && !passes[0].closed && (x == y || xa == ya)) fused_ok = false;  // a halo pass cannot run in place
+    if (fused_ok) {
+        const size_t one = temp_bytes(shape, false) / 2;
+        void* t0 = workspace;
+        void* t1 = workspace ? static_cast<char*>(workspace) + one : nullptr;
+        const void* cur0 = x;
+        const void* cur1 = xa;
+        int cur_dtype = in_dtype;
+        for (size_t k = 0; k < np; ++k) {
+            const FusedPass& ps = passes[k];
+            const bool to_out = ((np - 1 - k) % 2) == 0;
+            const bool last = (k + 1 == np);
+            void* d0 = to_out ? y : t0;
+            void* d1 = to_out ? ya : t1;
+            const int d_dtype = to_out ? out_dtype : NCN_F32;
+            hipError_t err;
+            if (ps.single) {
+                StageArgs a{};
+                fill_common(a, shape, p, first_stage + ps.first, alpha, m, activation);
+                a.in0 = cur0; a.in1 = cur1; a.in_dtype = cur_dtype;
+                a.out0 = d0; a.out1 = d1; a.out_dtype = d_dtype;
+                a.aux0 = last ? y32 : nullptr; a.aux1 = last ? ya32 : nullptr;
+                a.W = W + ps.first * wstride;
+                err = launch_fast_forward(kForward, a, shape->n_head, p.grid_x, s);
+            } else {
+                FusedArgs a{};
+                a.in0 = cur0; a.in1 = cur1; a.in_dtype = cur_dtype;
+                a.out0 = d0; a.out1 = d1; a.out_dtype = d_dtype;
+                a.aux0 = last ? y32 : nullptr; a.aux1 = last ? ya32 : nullptr;
+                a.W = W + ps.first * wstride;
+                fill_step_table(a.tab, shape->n_cache, alpha, m);
+                err = launch_fused(false, a, shape, ps, s);
+            }
+            if (err != hipSuccess) return (int)err;
+            cur0 = d0; cur1 = d1; cur_dtype = d_dtype;
+        }
+        return NCN_OK;
+    }
+
     for (int k = 0; k < n_stages; ++k) {
         StageArgs a{};
         fill_common(a, shape, p, first_stage + k, alpha, m, activation);
@@ -180,7 +254,7 @@ int ncn_forward(const void* x, const void* xa, int in_dtype, void* y, void* ya, 
         const bool last = (k == n_stages - 1);
         a.aux0 = last ? y32 : nullptr;
         a.aux1 = last ? ya32 : nullptr;
-        a.W = W + (int64_t)k * 2 * shape->E;
+        a.W = W + k * wstride;
         hipError_t err = (p.path == 2) ? launch_fast_forward(kForward, a, shape->n_head, p.grid_x, s)
                                        : launch_generic(kForward, a, shape->n_head, p.grid_x, s);
         if (err != hipSuccess) return (int)err;
@@ -232,6 +306,68 @@ int ncn_backward(const void* y, const void* ya, int y_dtype, const void* dy, con
         return NCN_ERR_ALIGN;
     const Plan p = make_plan(shape, activation);
     hipStream_t s = static_cast<hipStream_t>(stream);
+    float* partials = static_cast<float*>(workspace);
+    float* level1 = partials + (int64_t)kMaxGridX * 2 * shape->E;
+    const int64_t wstride = 2 * shape->E;
+
+    // several stages: LDS-resident passes, last pass of the range first; the state ping-pongs between the
+    // output arrays and four float32 arrays behind the dW scratch
+    std::vector<FusedPass> passes = multi_stage_plan(shape, first_stage, n_stages, activation, true);
+    const size_t np = passes.size();
+    bool fused_ok = np > 0;
+    if (np >= 2 && workspace_bytes < base_workspace_bytes(shape) + temp_bytes(shape, true)) fused_ok = false;
+    if (np == 1 && !passes[0].closed && (y == x_rec || ya == xa_rec || dy == dx || (dya && dya == dxa))) fused_ok = false;
+    if (fused_ok) {
+        const size_t one = temp_bytes(shape, true) / 4;
+        char* tb = static_cast<char*>(workspace) + base_workspace_bytes(shape);
+        float* t[4] = {reinterpret_cast<float*>(tb), reinterpret_cast<float*>(tb + one),
+                       reinterpret_cast<float*>(tb + 2 * one), reinterpret_cast<float*>(tb + 3 * one)};
+        const void* cy = y; const void* cya = ya; int cy_dtype = y_dtype;
+        const void* cg = dy; const void* cga = dya; int cg_dtype = dy_dtype;
+        for (size_t e = 0; e < np; ++e) {
+            const FusedPass& ps = passes[np - 1 - e];
+            const bool to_out = ((np - 1 - e) % 2) == 0;
+            float* dxr = to_out ? x_rec : t[0];
+            float* dxar = to_out ? xa_rec : t[1];
+            void* ddx = to_out ? dx : static_cast<void*>(t[2]);
+            void* ddxa = to_out ? dxa : static_cast<void*>(t[3]);
+            const int d_dtype = to_out ? dx_dtype : NCN_F32;
+            hipError_t err;
+            if (ps.single) {
+                StageArgs a{};
+                fill_common(a, shape, p, first_stage + ps.first, alpha, m, activation);
+                a.in0 = cy; a.in1 = cya; a.in_dtype = cy_dtype;
+                a.g0 = cg; a.g1 = cga; a.g_dtype = cg_dtype;
+                a.out0 = ddx; a.out1 = ddxa; a.out_dtype = d_dtype;
+                a.aux0 = dxr; a.aux1 = dxar;
+                a.W = W + ps.first * wstride;
+                a.dw_partials = partials;
+                err = launch_fast_backward(a, shape->n_head, p.grid_x, s);
+                if (err != hipSuccess) return (int)err;
+                err = launch_reduce_dw(partials, p.partial_rows, wstride, wstride, level1, dW + ps.first * wstride, s);
+            } else {
+                FusedArgs a{};
+                a.in0 = cy; a.in1 = cya; a.in_dtype = cy_dtype;
+                a.g0 = cg; a.g1 = cga; a.g_dtype = cg_dtype;
+                a.out0 = ddx; a.out1 = ddxa; a.out_dtype = d_dtype;
+                a.aux0 = dxr; a.aux1 = dxar;
+                a.W = W + ps.first * wstride;
+                a.dw_partials = partials;
+                fill_step_table(a.tab, shape->n_cache, alpha, m);
+                err = launch_fused(true, a, shape, ps, s);
+                if (err != hipSuccess) return (int)err;
+                const int rows = fused_grid(shape, ps) / shape->n_head;
+                for (int k = 0; k < ps.count && err == hipSuccess; ++k)
+                    err = launch_reduce_dw(partials + k * wstride, rows, (int64_t)ps.count * wstride, wstride, level1,
+                                           dW + (ps.first + k) * wstride, s);
+            }
+            if (err != hipSuccess) return (int)err;
+            cy = dxr; cya = dxar; cy_dtype = NCN_F32;
+            cg = ddx; cga = ddxa; cg_dtype = d_dtype;
+        }
+        return NCN_OK;
+    }
+
     for (int k = n_stages - 1; k >= 0; --k) {
         StageArgs a{};
         fill_common(a, shape, p, first_stage + k, alpha, m, activation);
@@ -248,12 +384,11 @@ int ncn_backward(const void* y, const void* ya, int y_dtype, const void* dy, con
         a.aux0 = x_rec;
         a.aux1 = xa_rec;
         a.W = W + (int64_t)k * 2 * shape->E;
-        a.dw_partials = static_cast<float*>(workspace);
+        a.dw_partials = partials;
         hipError_t err = (p.path == 2) ? launch_fast_backward(a, shape->n_head, p.grid_x, s)
                                        : launch_generic(kBackward, a, shape->n_head, p.grid_x, s);
         if (err != hipSuccess) return (int)err;
-        err = launch_reduce_dw(a.dw_partials, p.partial_rows, 2 * shape->E, a.dw_partials + (int64_t)kMaxGridX * 2 * shape->E,
-                               dW + (int64_t)k * 2 * shape->E, s);
+        err = launch_reduce_dw(partials, p.partial_rows, wstride, wstride, level1, dW + k * wstride, s);
         if (err != hipSuccess) return (int)err;
     }
     return NCN_OK;

@@ -1,0 +1,188 @@
+// Planning and launching of the multi-stage (LDS-resident) passes; kernels in ncn_fused_kernels.h.
+#include <vector>
+
+#include "ncn_fused_kernels.h"
+#include "ncn_launch.h"
+
+namespace ncn {
+
+namespace {
+
+// shapes the multi-stage kernels are built for; tile shapes as in the one-stage table
+// (n_cache = 8 and up is bound by arithmetic even stage by stage: measured 10 % slower through LDS)
+#define NCN_FOR_EACH_FUSED_CONFIG(X) \
+    X(2, 16) X(4, 16) X(2, 32) X(4, 32)
+
+constexpr size_t kFusedStateBytes = 64 * 1024;  // LDS for the row arrays of one workgroup (2 forward, 4 backward)
+constexpr int kFusedMaxGrid = 512;              // two workgroups per CU
+
+size_t fused_lds_bytes(int nc, int ec, bool backward, uint32_t window, int n_stages) {
+    const TileShape t = fast_tile(nc, ec);
+    const int lr = nc / t.r;
+    size_t bytes = (size_t)(backward ? 4 : 2) * window * nc * ec * sizeof(float);
+    if (lr > 1) bytes += (size_t)kFusedWaves * t.f * 64 * sizeof(float);
+    if (backward) bytes += (size_t)kFusedWaves * n_stages * 2 * ec * sizeof(float);
+    return bytes;
+}
+
+uint32_t stage_stride_of(int stage, uint32_t groups) {
+    if (stage == 0) return 0;
+    uint64_t s = 1 % groups;
+    for (int k = 1; k < stage; ++k) s = (s * 2) % groups;
+    return (uint32_t)s;
+}
+
+uint32_t floor_pow2(uint32_t v) {
+    uint32_t p = 1;
+    while (p * 2 <= v) p *= 2;
+    return p;
+}
+
+}  // namespace
+
+bool fused_supported(const ncn_shape* sh, int activation) {
+    if (activation != NCN_ACT_TANH) return false;
+    const int64_t ec = sh->E / sh->n_head;
+    const uint32_t groups = (uint32_t)(sh->N / sh->n_cache);
+    if ((groups & (groups - 1)) != 0 || groups < 2) return false;
+#define NCN_MATCH(NC, EC) \
+    if (sh->n_cache == NC && ec == EC) return true;
+    NCN_FOR_EACH_FUSED_CONFIG(NCN_MATCH)
+#undef NCN_MATCH
+    return false;
+}
+
+// Cuts stages [first, first + count) into passes, ascending.  Window capacity in sub-blocks is a power of two.
+std::vector<FusedPass> plan_fused(const ncn_shape* sh, int first, int count, bool backward) {
+    std::vector<FusedPass> passes;
+    const int nc = sh->n_cache, ec = (int)(sh->E / sh->n_head);
+    const uint32_t groups = (uint32_t)(sh->N / nc);
+    const uint32_t cap_rows = (uint32_t)(kFusedStateBytes / ((backward ? 4 : 2) * ec * sizeof(float)));
+    uint32_t cap = floor_pow2(cap_rows / nc);
+    if (cap > groups) cap = groups;
+    if (cap < 4) return passes;
+    std::vector<uint32_t> s(count);
+    for (int k = 0; k < count; ++k) s[k] = stage_stride_of(first + k, groups);
+
+    // backward keeps a dW slot per wave and stage in LDS: 7 stages leave room for two workgroups per CU
+    const int max_stages = backward ? kFusedMaxStages - 1 : kFusedMaxStages;
+    // stages [a, b) as one pass; returns its cost in "full passes over the data" (read + write), or < 0 if impossible
+    auto make = [&](int a, int b, FusedPass& p) -> double {
+        if (b - a > max_stages || b - a < 2) return -1.0;
+        uint32_t s0 = 0;
+        for (int k = a; k < b; ++k)
+            if (s[k] && (!s0 || s[k] < s0)) s0 = s[k];
+        if (!s0) s0 = groups / cap;  // only contiguous-block stages: any class structure works, take full windows
+        p.first = a;
+        p.count = b - a;
+        p.single = 0;
+        p.class_stride = s0;
+        p.ring = groups / s0;
+        uint32_t sum = 0;
+        for (int k = a; k < b; ++k) {
+            if (s[k] % s0) return -1.0;
+            p.sub_stride[k - a] = s[k] / s0;
+            sum += s[k] / s0;
+        }
+        if (p.ring <= cap) {  // closed: cap / ring whole rings of adjacent classes per window
+            p.closed = 1;
+            p.window = cap;
+            p.halo = 0;
+            p.own = cap;
+            p.tiles_per_ring = 1;
+            p.class_groups = s0 / (cap / p.ring);
+            return 2.0;
+        }
+        p.closed = 0;
+        p.window = cap;
+        p.halo = (uint32_t)(nc - 1) * sum;
+        if (2 * p.halo >= cap) return -1.0;
+        p.own = cap - 2 * p.halo;
+        if (p.own * 4 < cap * 3) return -1.0;  // more than a third of the window would be redundant work
+        p.tiles_per_ring = (p.ring + p.own - 1) / p.own;
+        p.class_groups = s0;
+        return 1.0 + (double)cap / p.own;
+    };
+
+    // cheapest cut of the range into passes (a one-stage launch costs one read + one write = 2)
+    std::vector<double> best(count + 1, 1e30);
+    std::vector<int> from(count + 1, -1);
+    std::vector<FusedPass> how(count + 1);
+    best[0] = 0.0;
+    for (int b = 1; b <= count; ++b) {
+        if (best[b - 1] + 2.0 < best[b]) {
+            best[b] = best[b - 1] + 2.0;
+            from[b] = b - 1;
+            FusedPass p{};
+            p.first = b - 1;
+            p.count = 1;
+            p.single = 1;
+            how[b] = p;
+        }
+        for (int a = b - 2; a >= 0 && b - a <= max_stages; --a) {
+            FusedPass p{};
+            const double c = make(a, b, p);
+            if (c >= 0.0 && best[a] + c < best[b] - 1e-9) {
+                best[b] = best[a] + c;
+                from[b] = a;
+                how[b] = p;
+            }
+        }
+    }
+    for (int b = count; b > 0; b = from[b]) passes.insert(passes.begin(), how[b]);
+    return passes;
+}
+
+template <int NC, int EC>
+static hipError_t launch_fused_t(bool backward, const FusedArgs& a, int grid, size_t lds, hipStream_t s) {
+    constexpr TileShape t = fast_tile(NC, EC);
+    static_assert(t.r != 0, "multi-stage shapes must be one-stage shapes too");
+    hipError_t err;
+    if (backward) {
+        auto k = fused_backward_kernel<NC, EC, t.r, t.f>;
+        err = hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (err != hipSuccess) return err;
+        hipLaunchKernelGGL(k, dim3(grid), dim3(kFusedThreads), lds, s, a);
+    } else {
+        auto k = fused_forward_kernel<NC, EC, t.r, t.f>;
+        err = hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (err != hipSuccess) return err;
+        hipLaunchKernelGGL(k, dim3(grid), dim3(kFusedThreads), lds, s, a);
+    }
+    return hipGetLastError();
+}
+
+int fused_grid(const ncn_shape* sh, const FusedPass& p) {
+    const int64_t items = sh->batch * (int64_t)p.class_groups * p.tiles_per_ring * sh->n_head;
+    int64_t g = items < kFusedMaxGrid ? items : kFusedMaxGrid;
+    g = g / sh->n_head * sh->n_head;
+    if (g < sh->n_head) g = sh->n_head;
+    return (int)g;
+}
+
+hipError_t launch_fused(bool backward, FusedArgs& a, const ncn_shape* sh, const FusedPass& p, hipStream_t s) {
+    const int nc = sh->n_cache, ec = (int)(sh->E / sh->n_head);
+    a.N = sh->N;
+    a.E = sh->E;
+    a.n_head = sh->n_head;
+    a.n_stages = p.count;
+    a.class_stride = p.class_stride;
+    a.ring = p.ring;
+    a.window = p.window;
+    a.halo = p.halo;
+    a.own = p.own;
+    a.tiles_per_ring = p.tiles_per_ring;
+    a.closed = p.closed;
+    a.class_groups = p.class_groups;
+    a.total_items = (uint32_t)(sh->batch * (int64_t)p.class_groups * p.tiles_per_ring * sh->n_head);
+    for (int k = 0; k < kFusedMaxStages; ++k) a.sub_stride[k] = k < p.count ? p.sub_stride[k] : 0;
+    const int grid = fused_grid(sh, p);
+    const size_t lds = fused_lds_bytes(nc, ec, backward, p.window, p.count);
+#define NCN_CASE(NC, EC) \
+    if (nc == NC && ec == EC) return launch_fused_t<NC, EC>(backward, a, grid, lds, s);
+    NCN_FOR_EACH_FUSED_CONFIG(NCN_CASE)
+#undef NCN_CASE
+    return hipErrorInvalidConfiguration;
+}
+
+}  // namespace ncn

@@ -1,0 +1,308 @@
+// Multi-stage kernels: several consecutive stages on a tile of rows that stays in LDS.
+//
+// Why.  With small groups (n_cache 2..8) one stage does little arithmetic per byte and a one-stage launch runs
+// at HBM speed; every further stage that works on rows already in LDS saves one full read and write of the
+// activations (and, in backward, of the gradients).
+//
+// Which rows.  Stage l reads, for group b, slot o from block (b + o*s_l) mod groups (torch_ref/ncn_pytorch.py:38-40).
+// Take a run of stages whose non-zero strides are all multiples of S0 (powers of two here).  Then blocks of one
+// residue class r = b mod S0 only ever meet blocks of the same class, and inside a class, with the sub-block
+// index q = b div S0 on a ring of groups/S0 sub-blocks, the strides become s_l/S0.  A workgroup holds a window
+// of consecutive sub-blocks of one (batch, head, class):
+//   * closed pass: the window is one whole ring, or several whole rings of adjacent classes when a ring is
+//     smaller than the window (indices wrap inside each ring): nothing outside is ever needed;
+//   * halo pass:   the window is `own` sub-blocks plus `halo` = (n_cache-1) * sum(s_l/S0) on each side.  Every
+//     stage updates the groups that lie completely inside the window; rows near the window edge go stale, but
+//     by construction never reach an owned row.  Only owned rows are written back and only groups whose slot-0
+//     sub-block is owned count towards dW, so the redundant halo work is invisible outside.
+// A halo pass must not run in place (another workgroup still needs the old value of an owned row as its halo),
+// a closed pass may.  The host (ncn_fused.hip) cuts a stage range into passes and ping-pongs buffers.
+//
+// How.  Per stage each wave gathers R x F register tiles of whole groups from LDS (the tile shapes and the step
+// code are those of the one-stage kernels, ncn_stage_kernels.h), runs the n_cache steps and scatters the tile
+// back; one workgroup barrier separates stages.  Backward sums each wave's dW share of a stage into a per-wave LDS
+// slot (one writer per slot, fixed order: deterministic) and leaves one partial row per workgroup and stage.
+#pragma once
+#include "ncn_stage_kernels.h"
+
+namespace ncn {
+
+constexpr int kFusedMaxStages = 8;
+constexpr int kFusedWaves = 8;
+constexpr int kFusedThreads = 64 * kFusedWaves;
+
+struct FusedArgs {
+    const void* in0;   // forward: x    backward: y (outputs of the pass's last stage)
+    const void* in1;   //          xa             ya
+    const void* g0;    // backward: dy
+    const void* g1;    //           dya (may be null = zeros)
+    void* out0;        // forward: y    backward: dx
+    void* out1;        //          ya             dxa
+    float* aux0;       // forward: optional float32 copy of y     backward: x_rec (inputs of the pass's first stage)
+    float* aux1;       //          optional float32 copy of ya              xa_rec
+    const float* W;    // [n_stages][2E], first stage of the pass first
+    float* dw_partials;  // backward: [gridDim.x / n_head][n_stages][2E]
+    int64_t N, E;
+    int32_t n_head, n_stages;
+    int32_t in_dtype, g_dtype, out_dtype, aux_dtype_unused;
+    uint32_t class_stride;    // S0, in blocks
+    uint32_t ring;            // sub-blocks per class = groups / S0 (power of two)
+    uint32_t window;          // sub-blocks held in LDS
+    uint32_t halo;            // sub-blocks of halo on each side (0 for a closed pass)
+    uint32_t own;             // owned sub-blocks per window (= ring for a closed pass)
+    uint32_t tiles_per_ring;  // ceil(ring / own)
+    uint32_t closed;          // 1: the window holds window/ring whole rings (adjacent classes) and indices wrap
+    uint32_t class_groups;    // closed: S0 / (window / ring) windows per batch entry; halo: S0
+    uint32_t total_items;     // batch * class_groups * tiles_per_ring * n_head
+    uint32_t sub_stride[kFusedMaxStages];  // s_l / S0 per stage of the pass
+    StepTable tab;
+};
+
+struct FusedItem {
+    int head;
+    uint32_t cls, sub0, own_lo, own_cnt;
+    int64_t base;  // element offset of (batch, row 0, head slice)
+};
+
+template <int EC>
+__device__ __forceinline__ FusedItem fused_item(const FusedArgs& A, uint32_t item) {
+    FusedItem it;
+    it.head = item % A.n_head;
+    uint32_t t = item / A.n_head;
+    const uint32_t k = t % A.tiles_per_ring;
+    t /= A.tiles_per_ring;
+    const uint32_t cg = t % A.class_groups;
+    const uint32_t b = t / A.class_groups;
+    if (A.closed) {
+        it.cls = cg * (A.window / A.ring);   // first class of the window
+        it.sub0 = 0u;
+        it.own_lo = 0u;
+        it.own_cnt = A.window;
+    } else {
+        it.cls = cg;
+        it.sub0 = (k * A.own + A.ring - A.halo) & (A.ring - 1u);
+        it.own_lo = A.halo;
+        const uint32_t left = A.ring - k * A.own;
+        it.own_cnt = left < A.own ? left : A.own;
+    }
+    it.base = (int64_t)b * A.N * A.E + (int64_t)it.head * EC;
+    return it;
+}
+
+// element offset (without the feature) of local row `lr` = (window sub-block qi) * NC + slot
+template <int NC>
+__device__ __forceinline__ int64_t fused_row_offset(const FusedArgs& A, const FusedItem& it, uint32_t lr) {
+    const uint32_t qi = lr / NC, o = lr - qi * NC;
+    const uint32_t sub = (it.sub0 + qi) & (A.ring - 1u);
+    const uint32_t cls = A.closed ? it.cls + qi / A.ring : it.cls;
+    const uint32_t blk = sub * A.class_stride + cls;
+    return it.base + ((int64_t)blk * NC + o) * A.E;
+}
+
+// LDS row of slot i of the group whose slot-0 sub-block is window position qg
+template <int NC>
+__device__ __forceinline__ uint32_t fused_lds_row(const FusedArgs& A, uint32_t qg, uint32_t i, uint32_t sstride) {
+    uint32_t qi = qg + i * sstride;
+    if (A.closed) qi = (qg & ~(A.ring - 1u)) | (qi & (A.ring - 1u));  // wrap inside the group's own ring
+    return qi * NC + i;
+}
+
+template <int F>
+__device__ __forceinline__ void lds_load_frag(const float* row, float (&v)[F]) {
+#pragma unroll
+    for (int k = 0; k < F / 4; ++k) {
+        const float4 t = reinterpret_cast<const float4*>(row)[k];
+        v[4 * k] = t.x; v[4 * k + 1] = t.y; v[4 * k + 2] = t.z; v[4 * k + 3] = t.w;
+    }
+}
+template <int F>
+__device__ __forceinline__ void lds_store_frag(float* row, const float (&v)[F]) {
+#pragma unroll
+    for (int k = 0; k < F / 4; ++k)
+        reinterpret_cast<float4*>(row)[k] = make_float4(v[4 * k], v[4 * k + 1], v[4 * k + 2], v[4 * k + 3]);
+}
+
+// global -> LDS for every row of the window (4 features per thread and trip)
+template <int NC, int EC>
+__device__ __forceinline__ void fused_load_rows(const FusedArgs& A, const FusedItem& it, const void* src, int dtype,
+                                                float* dst, uint32_t rows) {
+    constexpr uint32_t CPR = EC / 4;
+    for (uint32_t c = threadIdx.x; c < rows * CPR; c += kFusedThreads) {
+        const uint32_t lr = c / CPR, c4 = c - lr * CPR;
+        float v[4];
+        if (src) load_frag<4>(src, dtype, fused_row_offset<NC>(A, it, lr) + c4 * 4, true, v);
+        else v[0] = v[1] = v[2] = v[3] = 0.f;
+        lds_store_frag<4>(dst + lr * EC + c4 * 4, v);
+    }
+}
+
+// LDS -> global for the owned rows
+template <int NC, int EC>
+__device__ __forceinline__ void fused_store_rows(const FusedArgs& A, const FusedItem& it, const float* src, void* dst,
+                                                 int dtype) {
+    constexpr uint32_t CPR = EC / 4;
+    const uint32_t r0 = it.own_lo * NC, rows = it.own_cnt * NC;
+    for (uint32_t c = threadIdx.x; c < rows * CPR; c += kFusedThreads) {
+        const uint32_t lr = r0 + c / CPR, c4 = c % CPR;
+        float v[4];
+        lds_load_frag<4>(src + lr * EC + c4 * 4, v);
+        store_frag<4>(dst, dtype, fused_row_offset<NC>(A, it, lr) + c4 * 4, true, v);
+    }
+}
+
+template <int NC, int EC, int R, int F>
+__global__ void __launch_bounds__(kFusedThreads) fused_forward_kernel(const FusedArgs A) {
+    using T = Tile<NC, EC, R, F>;
+    extern __shared__ float4 fused_lds4[];
+    float* lds = reinterpret_cast<float*>(fused_lds4);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int fl = lane % T::LF, rl = (lane / T::LF) % T::LR, gw = lane / T::LPG;
+    const uint32_t rows = A.window * NC;
+    float* xs = lds;
+    float* as = lds + rows * EC;
+    float4* slots = reinterpret_cast<float4*>(lds + 2 * rows * EC) + wave * (F / 4) * 64;
+
+    for (uint32_t item = blockIdx.x; item < A.total_items; item += gridDim.x) {
+        const FusedItem it = fused_item<EC>(A, item);
+        fused_load_rows<NC, EC>(A, it, A.in0, A.in_dtype, xs, rows);
+        fused_load_rows<NC, EC>(A, it, A.in1, A.in_dtype, as, rows);
+        __syncthreads();
+        for (int st = 0; st < A.n_stages; ++st) {
+            const uint32_t ss = A.sub_stride[st];
+            const uint32_t ngroups = A.closed ? A.window : A.window - (NC - 1) * ss;
+            float wi[F], wj[F];
+            load_w<F>(A.W + (int64_t)st * 2 * A.E, A.E, it.head, EC, fl, wi, wj);
+            for (uint32_t wt = wave; wt * T::GPW < ngroups; wt += kFusedWaves) {
+                const uint32_t qg = wt * T::GPW + gw;
+                const bool valid = qg < ngroups;
+                float x[R][F], a[R][F];
+                uint32_t row[R];
+#pragma unroll
+                for (int rr = 0; rr < R; ++rr) {
+                    row[rr] = fused_lds_row<NC>(A, valid ? qg : 0u, rl * R + rr, ss) * EC + fl * F;
+                    lds_load_frag<F>(xs + row[rr], x[rr]);
+                    lds_load_frag<F>(as + row[rr], a[rr]);
+                }
+                forward_steps<NC, EC, R, F>(x, a, wi, wj, A.tab, lane, slots);
+                if (valid) {
+#pragma unroll
+                    for (int rr = 0; rr < R; ++rr) {
+                        lds_store_frag<F>(xs + row[rr], x[rr]);
+                        lds_store_frag<F>(as + row[rr], a[rr]);
+                    }
+                }
+            }
+            __syncthreads();
+        }
+        fused_store_rows<NC, EC>(A, it, xs, A.out0, A.out_dtype);
+        fused_store_rows<NC, EC>(A, it, as, A.out1, A.out_dtype);
+        if (A.aux0) {
+            fused_store_rows<NC, EC>(A, it, xs, A.aux0, NCN_F32);
+            fused_store_rows<NC, EC>(A, it, as, A.aux1, NCN_F32);
+        }
+        __syncthreads();
+    }
+}
+
+template <int NC, int EC, int R, int F>
+__global__ void __launch_bounds__(kFusedThreads) fused_backward_kernel(const FusedArgs A) {
+    using T = Tile<NC, EC, R, F>;
+    extern __shared__ float4 fused_lds4[];
+    float* lds = reinterpret_cast<float*>(fused_lds4);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int fl = lane % T::LF, rl = (lane / T::LF) % T::LR, gw = lane / T::LPG;
+    const uint32_t rows = A.window * NC;
+    float* ys = lds;
+    float* bs = ys + rows * EC;
+    float* gs = bs + rows * EC;
+    float* hs = gs + rows * EC;
+    float* after = hs + rows * EC;
+    float4* slots = reinterpret_cast<float4*>(after) + wave * (F / 4) * 64;
+    float* dw_all = after + (T::LR == 1 ? 0 : kFusedWaves * F * 64);   // [wave][stage][2][EC]
+    const int dw_wave_stride = A.n_stages * 2 * EC;
+    float* dw_mine = dw_all + wave * dw_wave_stride;
+    for (int k = lane; k < dw_wave_stride; k += 64) dw_mine[k] = 0.f;
+
+    for (uint32_t item = blockIdx.x; item < A.total_items; item += gridDim.x) {
+        const FusedItem it = fused_item<EC>(A, item);
+        fused_load_rows<NC, EC>(A, it, A.in0, A.in_dtype, ys, rows);
+        fused_load_rows<NC, EC>(A, it, A.in1, A.in_dtype, bs, rows);
+        fused_load_rows<NC, EC>(A, it, A.g0, A.g_dtype, gs, rows);
+        fused_load_rows<NC, EC>(A, it, A.g1, A.g_dtype, hs, rows);
+        __syncthreads();
+        for (int st = A.n_stages - 1; st >= 0; --st) {
+            const uint32_t ss = A.sub_stride[st];
+            const uint32_t ngroups = A.closed ? A.window : A.window - (NC - 1) * ss;
+            float wi[F], wj[F], dwi[F], dwj[F];
+            load_w<F>(A.W + (int64_t)st * 2 * A.E, A.E, it.head, EC, fl, wi, wj);
+#pragma unroll
+            for (int f = 0; f < F; ++f) dwi[f] = dwj[f] = 0.f;
+            for (uint32_t wt = wave; wt * T::GPW < ngroups; wt += kFusedWaves) {
+                const uint32_t qg = wt * T::GPW + gw;
+                const bool valid = qg < ngroups;
+                const float own = (valid && qg - it.own_lo < it.own_cnt) ? 1.0f : 0.0f;  // unsigned compare: lo <= qg < lo+cnt
+                float Y[R][F], B[R][F], G[R][F], H[R][F];
+                uint32_t row[R];
+#pragma unroll
+                for (int rr = 0; rr < R; ++rr) {
+                    row[rr] = fused_lds_row<NC>(A, valid ? qg : 0u, rl * R + rr, ss) * EC + fl * F;
+                    lds_load_frag<F>(ys + row[rr], Y[rr]);
+                    lds_load_frag<F>(bs + row[rr], B[rr]);
+                    lds_load_frag<F>(gs + row[rr], G[rr]);
+                    lds_load_frag<F>(hs + row[rr], H[rr]);
+                }
+                backward_steps<NC, EC, R, F, true>(Y, B, G, H, wi, wj, dwi, dwj, own, A.tab, lane, slots);
+                if (valid) {
+                    const float up = A.tab.inv_m_pow_n;
+#pragma unroll
+                    for (int rr = 0; rr < R; ++rr) {
+#pragma unroll
+                        for (int f = 0; f < F; ++f) {
+                            Y[rr][f] *= up;
+                            B[rr][f] *= up;
+                        }
+                        lds_store_frag<F>(ys + row[rr], Y[rr]);
+                        lds_store_frag<F>(bs + row[rr], B[rr]);
+                        lds_store_frag<F>(gs + row[rr], G[rr]);
+                        lds_store_frag<F>(hs + row[rr], H[rr]);
+                    }
+                }
+            }
+            // this wave's dW share of the stage: sum the lanes that hold the same features, add to the wave's slot
+#pragma unroll
+            for (int f = 0; f < F; ++f) {
+                dwi[f] = lane_sum<T::LF, 64>(dwi[f]);
+                dwj[f] = lane_sum<T::LF, 64>(dwj[f]);
+            }
+            if (lane < T::LF) {
+                float* d = dw_mine + st * (2 * EC) + fl * F;
+#pragma unroll
+                for (int f = 0; f < F; ++f) {
+                    d[f] += dwi[f];
+                    d[EC + f] += dwj[f];
+                }
+            }
+            __syncthreads();
+        }
+        fused_store_rows<NC, EC>(A, it, gs, A.out0, A.out_dtype);
+        fused_store_rows<NC, EC>(A, it, hs, A.out1, A.out_dtype);
+        if (A.aux0) {
+            fused_store_rows<NC, EC>(A, it, ys, A.aux0, NCN_F32);
+            fused_store_rows<NC, EC>(A, it, bs, A.aux1, NCN_F32);
+        }
+        __syncthreads();
+    }
+    __syncthreads();
+    // one partial row per workgroup and stage; workgroup b owns slot (b / n_head, head b % n_head)
+    const int head = blockIdx.x % A.n_head;   // == head of every item of this workgroup (gridDim.x % n_head == 0)
+    float* prow = A.dw_partials + (int64_t)(blockIdx.x / A.n_head) * A.n_stages * (2 * A.E);
+    for (int k = threadIdx.x; k < A.n_stages * 2 * EC; k += kFusedThreads) {
+        const int st = k / (2 * EC), rem = k - st * 2 * EC, half = rem / EC, f = rem - half * EC;
+        float sum = 0.f;
+#pragma unroll
+        for (int w = 0; w < kFusedWaves; ++w) sum += dw_all[w * dw_wave_stride + st * 2 * EC + rem];
+        prow[(int64_t)st * (2 * A.E) + (int64_t)half * A.E + (int64_t)head * EC + f] = sum;
+    }
+}
+
+}  // namespace ncn

@@ -175,8 +175,8 @@ __global__ void __launch_bounds__(64) generic_backward_kernel(const StageArgs A)
 // out[blockIdx.y][col] = sum of rows [blockIdx.y * rows_per_block, +rows_per_block) of in[row][col].
 // 64 columns x 4 row lanes per block; launched twice (many blocks over row chunks, then one row of blocks) so
 // that the first level has enough loads in flight to run at memory speed.  The order of additions is fixed.
-__global__ void __launch_bounds__(256) reduce_rows_kernel(const float* __restrict__ in, int rows, int64_t cols,
-                                                          int rows_per_block, float* __restrict__ out) {
+__global__ void __launch_bounds__(256) reduce_rows_kernel(const float* __restrict__ in, int rows, int64_t row_stride,
+                                                          int64_t cols, int rows_per_block, float* __restrict__ out) {
     __shared__ float red[4][64];
     const int cx = threadIdx.x & 63, ry = threadIdx.x >> 6;
     const int64_t col = (int64_t)blockIdx.x * 64 + cx;
@@ -185,7 +185,7 @@ __global__ void __launch_bounds__(256) reduce_rows_kernel(const float* __restric
     float sum = 0.f;
     if (col < cols) {
 #pragma unroll 4
-        for (int r = r0 + ry; r < r1; r += 4) sum += in[(int64_t)r * cols + col];
+        for (int r = r0 + ry; r < r1; r += 4) sum += in[(int64_t)r * row_stride + col];
     }
     red[ry][cx] = sum;
     __syncthreads();
@@ -213,14 +213,15 @@ hipError_t launch_generic(Pass pass, const StageArgs& a, int n_head, int grid_x,
     return hipGetLastError();
 }
 
-hipError_t launch_reduce_dw(const float* partials, int rows, int64_t cols, float* level1, float* dW, hipStream_t s) {
+hipError_t launch_reduce_dw(const float* partials, int rows, int64_t row_stride, int64_t cols, float* level1, float* dW,
+                            hipStream_t s) {
     const unsigned col_blocks = (unsigned)((cols + 63) / 64);
     const int chunks = (rows + kReduceRowsPerBlock - 1) / kReduceRowsPerBlock;  // <= kReduceLevel1Rows
-    hipLaunchKernelGGL(reduce_rows_kernel, dim3(col_blocks, chunks), dim3(256), 0, s, partials, rows, cols,
+    hipLaunchKernelGGL(reduce_rows_kernel, dim3(col_blocks, chunks), dim3(256), 0, s, partials, rows, row_stride, cols,
                        kReduceRowsPerBlock, level1);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess) return err;
-    hipLaunchKernelGGL(reduce_rows_kernel, dim3(col_blocks, 1), dim3(256), 0, s, level1, chunks, cols, chunks, dW);
+    hipLaunchKernelGGL(reduce_rows_kernel, dim3(col_blocks, 1), dim3(256), 0, s, level1, chunks, cols, cols, chunks, dW);
     return hipGetLastError();
 }
 

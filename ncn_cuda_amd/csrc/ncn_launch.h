@@ -2,6 +2,8 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include <vector>
+
 #include "ncn_configs.h"
 #include "ncn_device.h"
 
@@ -41,6 +43,21 @@ constexpr int kReduceLevel1Rows = kMaxGridX / kReduceRowsPerBlock;
 hipError_t launch_fast_forward(Pass pass, const StageArgs& a, int n_head, int grid_x, hipStream_t s);
 hipError_t launch_fast_backward(const StageArgs& a, int n_head, int grid_x, hipStream_t s);
 hipError_t launch_generic(Pass pass, const StageArgs& a, int n_head, int grid_x, hipStream_t s);
-hipError_t launch_reduce_dw(const float* partials, int rows, int64_t cols, float* level1, float* dW, hipStream_t s);
+// dW[col] = sum over `rows` rows of partials[row * row_stride + col]; level1 is scratch of kReduceLevel1Rows * cols floats.
+hipError_t launch_reduce_dw(const float* partials, int rows, int64_t row_stride, int64_t cols, float* level1, float* dW,
+                            hipStream_t s);
+
+// ---- multi-stage (LDS-resident) passes, ncn_fused.hip --------------------------------------------------------
+struct FusedArgs;
+struct FusedPass {
+    int first, count;  // stages [first, first + count) relative to the range that was planned
+    int single;        // 1: not worth fusing, run `first` with the one-stage kernel
+    uint32_t class_stride, ring, window, halo, own, tiles_per_ring, closed, class_groups;
+    uint32_t sub_stride[8];
+};
+bool fused_supported(const ncn_shape* sh, int activation);
+std::vector<FusedPass> plan_fused(const ncn_shape* sh, int first, int count, bool backward);
+int fused_grid(const ncn_shape* sh, const FusedPass& p);
+hipError_t launch_fused(bool backward, FusedArgs& a, const ncn_shape* sh, const FusedPass& p, hipStream_t s);
 
 }  // namespace ncn

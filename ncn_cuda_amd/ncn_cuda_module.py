@@ -117,11 +117,16 @@ def forward_stages(x, xa, W, alpha, activation, cache_dim, nhead, first_stage, n
             y32 = torch.empty(x.shape, dtype=torch.float32, device=dev)
             ya32 = torch.empty(x.shape, dtype=torch.float32, device=dev)
     aux = (y32, ya32) if (save_fp32 and out_dtype != torch.float32) else (None, None)
+    lib = _lib.load()
+    ws, ws_bytes = None, 0
+    if n_stages > 1:
+        ws_bytes = lib.ncn_workspace_bytes_stages(ctypes.byref(shape), int(first_stage), int(n_stages), int(activation), 0)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
     with torch.cuda.device(dev):
-        rc = _lib.load().ncn_forward(_ptr(x), _ptr(xa), _DTYPES[x.dtype], _ptr(y), _ptr(ya), _DTYPES[out_dtype],
-                                     _ptr(aux[0]), _ptr(aux[1]), _ptr(w), ctypes.byref(shape),
-                                     int(first_stage), int(n_stages), float(alpha), float(m), int(activation),
-                                     _stream(dev))
+        rc = lib.ncn_forward(_ptr(x), _ptr(xa), _DTYPES[x.dtype], _ptr(y), _ptr(ya), _DTYPES[out_dtype],
+                             _ptr(aux[0]), _ptr(aux[1]), _ptr(w), _ptr(ws), ctypes.c_size_t(ws_bytes),
+                             ctypes.byref(shape), int(first_stage), int(n_stages), float(alpha), float(m),
+                             int(activation), _stream(dev))
     _lib.check(rc, "ncn_forward")
     return (y, ya, y32, ya32) if save_fp32 else (y, ya)
 
@@ -150,7 +155,7 @@ def backward_stages(y, ya, dy, dya, W, alpha, activation, cache_dim, nhead, firs
     E = y.shape[2]
     dW = torch.empty(n_stages, 2 * E, dtype=torch.float32, device=dev)
     lib = _lib.load()
-    ws_bytes = lib.ncn_workspace_bytes(ctypes.byref(shape))
+    ws_bytes = lib.ncn_workspace_bytes_stages(ctypes.byref(shape), int(first_stage), int(n_stages), int(activation), 1)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
         rc = lib.ncn_backward(_ptr(y), _ptr(ya), _DTYPES[y.dtype], _ptr(dy), _ptr(dya), _DTYPES[dy.dtype],

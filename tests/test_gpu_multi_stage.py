@@ -1,0 +1,88 @@
+"""Multi-stage calls (n_stages > 1): the LDS-resident passes must reproduce the one-launch-per-stage path and the
+oracle, for closed passes, halo passes, wrapped strides, stage ranges that do not start at 0, and dya = NULL."""
+import pytest
+import torch
+
+from oracle import ncn_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def M():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from ncn_cuda_amd import ncn_cuda_module
+    return ncn_cuda_module
+
+
+# (batch, N, E, C, n, first_stage, L)
+CASES = [
+    (3, 1024, 64, 2, 2, 0, 11),    # groups 512: halo passes, a closed pass, and strides that wrap to 0 at the end
+    (2, 8192, 128, 4, 2, 0, 13),   # the deep small-group configuration at its real N (batch cut down)
+    (2, 1024, 128, 4, 4, 0, 5),    # n = 4, 5 stages (groups 256)
+    (2, 512, 32, 2, 8, 0, 4),      # n = 8: no LDS passes, the call loops over one-stage launches
+    (2, 512, 32, 2, 4, 1, 5),      # n = 4, head width 16
+    (2, 2048, 64, 2, 2, 3, 6),     # range that starts at stage 3 (stride 4)
+    (1, 256, 32, 1, 2, 0, 8),      # one head; whole ring fits the window from the start
+    (5, 64, 128, 4, 4, 0, 3),      # tiny ring (16 groups)
+]
+
+
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "b%d_N%d_E%d_C%d_n%d_s%d_L%d" % c)
+def test_multi_stage_matches_single_stage_and_oracle(M, case):
+    batch, N, E, C, n, first, L = case
+    alpha = 0.9
+    x, xa, Ws, dyi, dya = O.make_inputs(batch, N, E, L, n, seed=17, xa_zero=False)
+    gx, gxa, gdy, gdya = x.cuda(), xa.cuda(), dyi.cuda(), dya.cuda()
+    gWs = [w.cuda() for w in Ws]
+    Wst = torch.stack(gWs)
+    # one launch per stage
+    outs = []
+    cx, cxa = gx, gxa
+    for l in range(L):
+        cx, cxa = M.forward(cx, cxa, gWs[l], alpha, 0, n, C, first + l)
+        outs.append((cx, cxa))
+    # one call for all stages
+    y, ya = M.forward_stages(gx, gxa, Wst, alpha, 0, n, C, first, L)
+    assert torch.equal(y, outs[-1][0]) and torch.equal(ya, outs[-1][1])  # same arithmetic, float32 between stages
+
+    d = torch.float64
+    ref = O.net_autograd(x.to(d), xa.to(d), [w.to(d) for w in Ws], dyi.to(d), dya.to(d), alpha, n, C, first_stage=first)
+    assert O.rel_err(y, ref[0]) < 1e-5 and O.rel_err(ya, ref[1]) < 1e-5
+
+    xr, xar, dx, dxa, dW = M.backward_stages(y, ya, gdy, gdya, Wst, alpha, 0, n, C, first, L)
+    # whole-range reversal: float32 rounding grows like (1/m)^(n L)
+    amp = (1 / 0.9) ** (n * L)
+    tol = max(1e-5, 5e-7 * amp)
+    assert O.rel_err(dx, ref[2]) < tol
+    assert O.rel_err(dxa, ref[3]) < tol
+    for l in range(L):
+        assert O.rel_err(dW[l], ref[4][l]) < tol, f"dW{l}"
+    assert O.rel_err(xr, x) < tol
+    assert O.rel_err(xar, xa) < tol
+
+    # the same reversal done stage by stage through single-stage calls agrees to rounding
+    cy, cya, cg, cga = y, ya, gdy, gdya
+    for l in range(L - 1, -1, -1):
+        cy, cya, cg, cga, dWl = M.backward_stages(cy, cya, cg, cga, gWs[l], alpha, 0, n, C, first + l, 1)
+        assert O.rel_err(dW[l], dWl[0]) < 1e-5
+    assert O.rel_err(dx, cg) < 1e-6 and O.rel_err(dxa, cga) < 1e-6
+
+
+def test_multi_stage_dya_none_and_bf16_input(M):
+    batch, N, E, C, n, L = 2, 1024, 128, 4, 2, 10
+    x, xa, Ws, dyi, _ = O.make_inputs(batch, N, E, L, n, seed=23, xa_zero=True, dtype=torch.bfloat16)
+    gx, gxa, gdy = x.cuda(), xa.cuda(), dyi.cuda()
+    Wst = torch.stack([w.cuda() for w in Ws])
+    y, ya = M.forward_stages(gx, gxa, Wst, 0.9, 0, n, C, 0, L, out_dtype=torch.float32)
+    f = torch.float32
+    ref = O.net_autograd(x.to(f), xa.to(f), [w.to(f) for w in Ws], dyi.to(f), torch.zeros_like(dyi, dtype=f), 0.9, n, C)
+    assert O.rel_err(y, ref[0]) < 2e-5 and O.rel_err(ya, ref[1]) < 2e-5
+    a = M.backward_stages(y, ya, gdy, None, Wst, 0.9, 0, n, C, 0, L, grad_dtype=torch.float32)
+    b = M.backward_stages(y, ya, gdy, torch.zeros_like(gdy), Wst, 0.9, 0, n, C, 0, L, grad_dtype=torch.float32)
+    for u, v in zip(a, b):
+        assert torch.equal(u, v)
+    assert O.rel_err(a[2], ref[2]) < 1e-4
+    for l in range(L):
+        assert O.rel_err(a[4][l], ref[4][l]) < 1e-4

@@ -29,7 +29,8 @@ def _declared_functions():
 
 def test_header_functions_are_exported(lib):
     names = _declared_functions()
-    assert {"ncn_forward", "ncn_backward", "ncn_inverse", "ncn_workspace_bytes", "ncn_kernel_path",
+    assert {"ncn_forward", "ncn_backward", "ncn_inverse", "ncn_workspace_bytes", "ncn_workspace_bytes_stages",
+            "ncn_kernel_path",
             "ncn_check_shape", "ncn_error_string", "ncn_version"} <= set(names)
     handle = lib.load()
     for name in names:
@@ -68,6 +69,14 @@ def test_kernel_path_and_workspace(lib):
     ws = h.ncn_workspace_bytes(ctypes.byref(_shape(lib, 128, 4096, 128, 4, 16)))
     assert ws > 0 and ws % 16 == 0 and ws < (1 << 24)
     assert h.ncn_workspace_bytes(ctypes.byref(_shape(lib, 1, 65, 32, 4, 4))) == 0
+    # multi-stage passes: deep small-group stacks ask for ping-pong arrays, the headline shape (n_cache = 16) does not
+    deep = _shape(lib, 128, 8192, 128, 4, 2)
+    P4 = 128 * 8192 * 128 * 4
+    assert h.ncn_workspace_bytes_stages(ctypes.byref(deep), 0, 13, 0, 0) == 2 * P4
+    assert h.ncn_workspace_bytes_stages(ctypes.byref(deep), 0, 13, 0, 1) == h.ncn_workspace_bytes(ctypes.byref(deep)) + 4 * P4
+    assert h.ncn_workspace_bytes_stages(ctypes.byref(deep), 0, 1, 0, 0) == 0
+    head = _shape(lib, 128, 4096, 128, 4, 16)
+    assert h.ncn_workspace_bytes_stages(ctypes.byref(head), 0, 3, 0, 1) == h.ncn_workspace_bytes(ctypes.byref(head))
 
 
 def test_entry_points_reject_bad_arguments_before_touching_the_gpu(lib):
@@ -76,10 +85,11 @@ def test_entry_points_reject_bad_arguments_before_touching_the_gpu(lib):
     p = ctypes.c_void_p(4096)       # never dereferenced: every call below fails validation first
     z = ctypes.c_void_p(0)
     odd = ctypes.c_void_p(4100)
-    assert h.ncn_forward(z, p, 0, p, p, 0, z, z, p, ctypes.byref(sh), 0, 1, 0.9, 0.9, 0, z) == -1
-    assert h.ncn_forward(p, p, 5, p, p, 0, z, z, p, ctypes.byref(sh), 0, 1, 0.9, 0.9, 0, z) == -3
-    assert h.ncn_forward(odd, p, 0, p, p, 0, z, z, p, ctypes.byref(sh), 0, 1, 0.9, 0.9, 0, z) == -7
-    assert h.ncn_forward(p, p, 0, p, p, 0, p, z, p, ctypes.byref(sh), 0, 1, 0.9, 0.9, 0, z) == -1  # y32 without ya32
+    nows = (z, ctypes.c_size_t(0))
+    assert h.ncn_forward(z, p, 0, p, p, 0, z, z, p, *nows, ctypes.byref(sh), 0, 1, 0.9, 0.9, 0, z) == -1
+    assert h.ncn_forward(p, p, 5, p, p, 0, z, z, p, *nows, ctypes.byref(sh), 0, 1, 0.9, 0.9, 0, z) == -3
+    assert h.ncn_forward(odd, p, 0, p, p, 0, z, z, p, *nows, ctypes.byref(sh), 0, 1, 0.9, 0.9, 0, z) == -7
+    assert h.ncn_forward(p, p, 0, p, p, 0, p, z, p, *nows, ctypes.byref(sh), 0, 1, 0.9, 0.9, 0, z) == -1  # y32 without ya32
     assert h.ncn_inverse(p, p, 0, z, p, 0, p, ctypes.byref(sh), 0, 1, 0.9, 0.9, 0, z) == -1
     ws = h.ncn_workspace_bytes(ctypes.byref(sh))
     args = [p, p, 0, p, p, 0, p, p, 0, z, z, p, p]
