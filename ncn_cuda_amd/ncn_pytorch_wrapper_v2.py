@@ -53,6 +53,56 @@ class NCNFunction(torch.autograd.Function):
         return dx, dxa, sum_dW, None, None, None, None, None
 
 
+def default_save_every(n_cache: int) -> int:
+    """Stages per saved checkpoint of the whole-net node: the reversible backward amplifies float32 rounding by
+    (1/m)^(n_cache * stages) between checkpoints; 26 steps keep that below 16x at m = 0.9."""
+    return max(1, 26 // max(1, int(n_cache)))
+
+
+class NCNNetFunction(torch.autograd.Function):
+    """The whole stage stack as ONE autograd node (no counterpart in the reference, which chains one NCNFunction
+    per stage, ncn_pytorch_wrapper_v2.py:107-117).  Stages run `save_every` at a time through the library's
+    multi-stage calls; only the float32 outputs of every `save_every`-th stage are kept for backward, which
+    reverses each segment from its outputs.  Inter-stage activations stay float32 whatever the I/O dtype."""
+
+    @staticmethod
+    def forward(ctx, x, xa, alpha, activation, n_cache, n_head, first_stage, save_every, *weights):
+        L = len(weights)
+        save_every = default_save_every(n_cache) if not save_every else int(save_every)
+        W = torch.stack([w.detach().reshape(-1).to(torch.float32) for w in weights])
+        saved = []
+        cx, cxa = x, xa
+        segs = [(a, min(save_every, L - a)) for a in range(0, L, save_every)]
+        for a, cnt in segs:
+            cx, cxa = ncn_cuda_module.forward_stages(cx, cxa, W[a:a + cnt], alpha, activation, n_cache, n_head,
+                                                     first_stage + a, cnt, out_dtype=torch.float32)
+            saved.extend([cx, cxa])
+        ctx.save_for_backward(W, *saved)
+        ctx.cfg = (alpha, activation, n_cache, n_head, first_stage, segs, x.dtype, [w.dtype for w in weights],
+                   [w.shape for w in weights])
+        return cx.to(x.dtype), cxa.to(x.dtype)
+
+    @staticmethod
+    def backward(ctx, dyi, dya):
+        W, *saved = ctx.saved_tensors
+        alpha, activation, n_cache, n_head, first_stage, segs, io_dtype, w_dtypes, w_shapes = ctx.cfg
+        dWs = [None] * W.shape[0]
+        g, ga = dyi, dya
+        for k in range(len(segs) - 1, -1, -1):
+            a, cnt = segs[k]
+            _, _, g, ga, dW = ncn_cuda_module.backward_stages(
+                saved[2 * k], saved[2 * k + 1], g, ga, W[a:a + cnt], alpha, activation, n_cache, n_head,
+                first_stage + a, cnt, grad_dtype=torch.float32, want_inputs=cnt > 1)
+            for j in range(cnt):
+                dWs[a + j] = dW[j].reshape(w_shapes[a + j]).to(w_dtypes[a + j])
+        return (g.to(io_dtype), ga.to(io_dtype), None, None, None, None, None, None, *dWs)
+
+
+def fused_ncn_net(x, xa, weights, alpha, activation, n_cache, n_head, first_stage=0, save_every=None):
+    """Stages first_stage .. first_stage+len(weights)-1 as one autograd node; activation is the int code."""
+    return NCNNetFunction.apply(x, xa, alpha, activation, n_cache, n_head, first_stage, save_every, *weights)
+
+
 def fused_ncn_cuda_v2(
     x: torch.Tensor,
     xa: torch.Tensor,
@@ -90,22 +140,34 @@ class NCNModuleCuda(nn.Module):
 
 
 class NCNNetCuda(nn.Module):
-    def __init__(self, alpha, activation, n_cache, n_head, num_modules, embed_dim):
+    """Same constructor as the reference.  `fuse_stages=True` (keyword only, not in the reference) runs the stack as
+    one NCNNetFunction node instead of one node per module; parameters and state_dict are the same either way."""
+
+    def __init__(self, alpha, activation, n_cache, n_head, num_modules, embed_dim, *, fuse_stages=False,
+                 save_every=None):
         super().__init__()
         self.num_modules = num_modules
-        activation_nr = ACTIVATION_CODES[activation]
+        self.alpha = alpha
+        self.activation_nr = ACTIVATION_CODES[activation]
+        self.n_cache = n_cache
+        self.n_head = n_head
+        self.fuse_stages = fuse_stages
+        self.save_every = save_every
         self.ncn_modules = nn.ModuleList(
-            [NCNModuleCuda(alpha, activation_nr, n_cache, n_head, module_nr, embed_dim)
+            [NCNModuleCuda(alpha, self.activation_nr, n_cache, n_head, module_nr, embed_dim)
              for module_nr in range(num_modules)])
 
     def forward(self, x, xa):
+        if self.fuse_stages:
+            return fused_ncn_net(x, xa, [m.weight for m in self.ncn_modules], self.alpha, self.activation_nr,
+                                 self.n_cache, self.n_head, 0, self.save_every)
         for module_nr in range(self.num_modules):
             x, xa = self.ncn_modules[module_nr](x, xa)
         return x, xa
 
 
 class NCNNetTestCuda(nn.Module):
-    def __init__(self, alpha, activation, n_cache, n_head, num_modules, weights):
+    def __init__(self, alpha, activation, n_cache, n_head, num_modules, weights, *, fuse_stages=False, save_every=None):
         super().__init__()
         self.num_modules = num_modules
         self.alpha = alpha
@@ -113,8 +175,13 @@ class NCNNetTestCuda(nn.Module):
         self.n_cache = n_cache
         self.n_head = n_head
         self.weights = weights
+        self.fuse_stages = fuse_stages
+        self.save_every = save_every
 
     def forward(self, x, xa):
+        if self.fuse_stages:
+            return fused_ncn_net(x, xa, list(self.weights[:self.num_modules]), self.alpha, self.activation_nr,
+                                 self.n_cache, self.n_head, 0, self.save_every)
         for module_nr in range(self.num_modules):
             x, xa = fused_ncn_cuda_v2(x, xa, self.weights[module_nr], self.alpha, self.activation_nr,
                                       self.n_cache, self.n_head, module_nr)

@@ -85,3 +85,57 @@ def test_bf16_autograd(pkg):
     for l in range(L):
         assert gWs[l].grad.dtype == torch.bfloat16
         assert O.rel_err(gWs[l].grad, ref_dWs[l]) < 2e-2
+
+
+@pytest.mark.parametrize("cfg", [(2, 1024, 128, 4, 2, 9, torch.float32), (2, 512, 128, 4, 4, 7, torch.float32),
+                                 (2, 256, 128, 4, 16, 3, torch.bfloat16), (2, 512, 64, 2, 2, 6, torch.bfloat16)],
+                         ids=["n2_L9_f32", "n4_L7_f32", "n16_L3_bf16", "n2_L6_bf16"])
+def test_whole_net_node_matches_oracle_and_per_stage_nodes(pkg, cfg):
+    """NCNNetFunction (one node for the stack, checkpoints every save_every stages) against the oracle and against
+    the reference-style chain of per-stage nodes."""
+    batch, N, E, C, n, L, dtype = cfg
+    alpha = 0.9
+    x, xa, Ws, dyi, dya = O.make_inputs(batch, N, E, L, n, seed=31, xa_zero=False, dtype=dtype)
+    f = torch.float64 if dtype == torch.float32 else torch.float32
+    ref = O.net_autograd(x.to(f), xa.to(f), [w.to(f) for w in Ws], dyi.to(f), dya.to(f), alpha, n, C)
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+
+    def run(fuse):
+        gx, gxa = x.cuda().requires_grad_(), xa.cuda().requires_grad_()
+        gWs = [w.cuda().requires_grad_() for w in Ws]
+        net = pkg.NCNNetTestCuda(alpha, "tanh", n, C, L, gWs, fuse_stages=fuse)
+        yi, ya = net(gx, gxa)
+        assert yi.dtype == dtype
+        torch.autograd.backward([yi, ya], [dyi.cuda(), dya.cuda()])
+        return yi, ya, gx.grad, gxa.grad, [w.grad for w in gWs]
+
+    fused, chain = run(True), run(False)
+    for got in (fused, chain):
+        assert O.rel_err(got[0], ref[0]) < tol and O.rel_err(got[1], ref[1]) < tol
+        assert O.rel_err(got[2], ref[2]) < tol and O.rel_err(got[3], ref[3]) < tol
+        for l in range(L):
+            assert got[4][l].dtype == dtype
+            assert O.rel_err(got[4][l], ref[4][l]) < tol, f"dW{l}"
+    assert pkg.default_save_every(2) == 13 and pkg.default_save_every(16) == 1
+
+
+def test_net_cuda_fuse_stages_flag_keeps_parameters(pkg):
+    torch.manual_seed(1)
+    a = pkg.NCNNetCuda(0.9, "tanh", 2, 4, 6, 128).cuda()
+    b = pkg.NCNNetCuda(0.9, "tanh", 2, 4, 6, 128, fuse_stages=True).cuda()
+    with torch.no_grad():
+        for m in a.ncn_modules:
+            m.weight.normal_(0, 0.5)
+    b.load_state_dict(a.state_dict())
+    x = torch.randn(2, 256, 128, device="cuda")
+    xa = torch.randn(2, 256, 128, device="cuda")
+    xs = [x.clone().requires_grad_() for _ in range(2)]
+    outs = []
+    for net, xi in zip((a, b), xs):
+        yi, ya = net(xi, xa)
+        (yi.square().sum() + ya.sum()).backward()
+        outs.append((yi, xi.grad, [m.weight.grad for m in net.ncn_modules]))
+    assert O.rel_err(outs[1][0], outs[0][0]) < 1e-6
+    assert O.rel_err(outs[1][1], outs[0][1]) < 1e-5
+    for ga, gb in zip(outs[0][2], outs[1][2]):
+        assert O.rel_err(gb, ga) < 1e-5
