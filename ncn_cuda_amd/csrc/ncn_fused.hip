@@ -1,4 +1,5 @@
 // Planning and launching of the multi-stage (LDS-resident) passes; kernels in ncn_fused_kernels.h.
+#include <cmath>
 #include <vector>
 
 #include "ncn_fused_kernels.h"
@@ -20,6 +21,7 @@ size_t fused_lds_bytes(int nc, int ec, bool backward, uint32_t window, int n_sta
     const TileShape t = fast_tile(nc, ec);
     const int lr = nc / t.r;
     size_t bytes = (size_t)(backward ? 4 : 2) * window * nc * ec * sizeof(float);
+    bytes += (size_t)kFusedMaxStages * 2 * ec * sizeof(float);  // the pass's weights
     if (lr > 1) bytes += (size_t)kFusedWaves * t.f * 64 * sizeof(float);
     if (backward) bytes += (size_t)kFusedWaves * n_stages * 2 * ec * sizeof(float);
     return bytes;
@@ -176,6 +178,8 @@ hipError_t launch_fused(bool backward, FusedArgs& a, const ncn_shape* sh, const 
     a.class_groups = p.class_groups;
     a.total_items = (uint32_t)(sh->batch * (int64_t)p.class_groups * p.tiles_per_ring * sh->n_head);
     for (int k = 0; k < kFusedMaxStages; ++k) a.sub_stride[k] = k < p.count ? p.sub_stride[k] : 0;
+    a.scale_dn = (float)std::pow((double)a.tab.m, (double)(nc * p.count));
+    a.scale_up = (float)std::pow((double)a.tab.m, -(double)(nc * p.count));
     const int grid = fused_grid(sh, p);
     const size_t lds = fused_lds_bytes(nc, ec, backward, p.window, p.count);
 #define NCN_CASE(NC, EC) \

@@ -20,7 +20,9 @@
 //
 // How.  Per stage each wave gathers R x F register tiles of whole groups from LDS (the tile shapes and the step
 // code are those of the one-stage kernels, ncn_stage_kernels.h), runs the n_cache steps and scatters the tile
-// back; one workgroup barrier separates stages.  Backward sums each wave's dW share of a stage into a per-wave LDS
+// back; one workgroup barrier separates stages.  The rows stay in the m-power-scaled form of the step code for the
+// whole pass (the step counter just keeps counting across stages; backward keeps p = (1-m) g + h in place of h),
+// so true values exist only in HBM.  The pass's weights sit in LDS.  Backward sums each wave's dW share of a stage into a per-wave LDS
 // slot (one writer per slot, fixed order: deterministic) and leaves one partial row per workgroup and stage.
 #pragma once
 #include "ncn_stage_kernels.h"
@@ -55,6 +57,7 @@ struct FusedArgs {
     uint32_t class_groups;    // closed: S0 / (window / ring) windows per batch entry; halo: S0
     uint32_t total_items;     // batch * class_groups * tiles_per_ring * n_head
     uint32_t sub_stride[kFusedMaxStages];  // s_l / S0 per stage of the pass
+    float scale_dn, scale_up;              // m^(n_cache * n_stages) and its reciprocal
     StepTable tab;
 };
 
@@ -150,6 +153,33 @@ __device__ __forceinline__ void fused_store_rows(const FusedArgs& A, const Fused
     }
 }
 
+// LDS -> global for the owned rows, each value times `scale`
+template <int NC, int EC>
+__device__ __forceinline__ void fused_store_rows_scaled(const FusedArgs& A, const FusedItem& it, const float* src,
+                                                        float scale, void* dst, int dtype, float* copy32) {
+    constexpr uint32_t CPR = EC / 4;
+    const uint32_t r0 = it.own_lo * NC, rows = it.own_cnt * NC;
+    for (uint32_t c = threadIdx.x; c < rows * CPR; c += kFusedThreads) {
+        const uint32_t lr = r0 + c / CPR, c4 = c % CPR;
+        float v[4];
+        lds_load_frag<4>(src + lr * EC + c4 * 4, v);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) v[k] *= scale;
+        const int64_t off = fused_row_offset<NC>(A, it, lr) + c4 * 4;
+        store_frag<4>(dst, dtype, off, true, v);
+        if (copy32) store_frag<4>(copy32, NCN_F32, off, true, v);
+    }
+}
+
+// the pass's weights, [stage][Wi | Wj][EC] of this workgroup's head, into LDS
+template <int EC>
+__device__ __forceinline__ void fused_load_weights(const FusedArgs& A, int head, float* w_lds) {
+    for (int k = threadIdx.x; k < A.n_stages * 2 * EC; k += kFusedThreads) {
+        const int st = k / (2 * EC), rem = k - st * 2 * EC, half = rem / EC, f = rem - half * EC;
+        w_lds[k] = A.W[(int64_t)st * 2 * A.E + (int64_t)half * A.E + (int64_t)head * EC + f];
+    }
+}
+
 template <int NC, int EC, int R, int F>
 __global__ void __launch_bounds__(kFusedThreads) fused_forward_kernel(const FusedArgs A) {
     using T = Tile<NC, EC, R, F>;
@@ -160,7 +190,9 @@ __global__ void __launch_bounds__(kFusedThreads) fused_forward_kernel(const Fuse
     const uint32_t rows = A.window * NC;
     float* xs = lds;
     float* as = lds + rows * EC;
-    float4* slots = reinterpret_cast<float4*>(lds + 2 * rows * EC) + wave * (F / 4) * 64;
+    float* w_lds = as + rows * EC;                              // [kFusedMaxStages][2][EC]
+    float4* slots = reinterpret_cast<float4*>(w_lds + kFusedMaxStages * 2 * EC) + wave * (F / 4) * 64;
+    fused_load_weights<EC>(A, blockIdx.x % A.n_head, w_lds);   // every item of this workgroup has this head
 
     for (uint32_t item = blockIdx.x; item < A.total_items; item += gridDim.x) {
         const FusedItem it = fused_item<EC>(A, item);
@@ -171,7 +203,8 @@ __global__ void __launch_bounds__(kFusedThreads) fused_forward_kernel(const Fuse
             const uint32_t ss = A.sub_stride[st];
             const uint32_t ngroups = A.closed ? A.window : A.window - (NC - 1) * ss;
             float wi[F], wj[F];
-            load_w<F>(A.W + (int64_t)st * 2 * A.E, A.E, it.head, EC, fl, wi, wj);
+            lds_load_frag<F>(w_lds + st * 2 * EC + fl * F, wi);
+            lds_load_frag<F>(w_lds + st * 2 * EC + EC + fl * F, wj);
             for (uint32_t wt = wave; wt * T::GPW < ngroups; wt += kFusedWaves) {
                 const uint32_t qg = wt * T::GPW + gw;
                 const bool valid = qg < ngroups;
@@ -183,7 +216,7 @@ __global__ void __launch_bounds__(kFusedThreads) fused_forward_kernel(const Fuse
                     lds_load_frag<F>(xs + row[rr], x[rr]);
                     lds_load_frag<F>(as + row[rr], a[rr]);
                 }
-                forward_steps<NC, EC, R, F>(x, a, wi, wj, A.tab, lane, slots);
+                forward_core<NC, EC, R, F>(x, a, wi, wj, A.tab, st * NC, lane, slots);
                 if (valid) {
 #pragma unroll
                     for (int rr = 0; rr < R; ++rr) {
@@ -194,12 +227,8 @@ __global__ void __launch_bounds__(kFusedThreads) fused_forward_kernel(const Fuse
             }
             __syncthreads();
         }
-        fused_store_rows<NC, EC>(A, it, xs, A.out0, A.out_dtype);
-        fused_store_rows<NC, EC>(A, it, as, A.out1, A.out_dtype);
-        if (A.aux0) {
-            fused_store_rows<NC, EC>(A, it, xs, A.aux0, NCN_F32);
-            fused_store_rows<NC, EC>(A, it, as, A.aux1, NCN_F32);
-        }
+        fused_store_rows_scaled<NC, EC>(A, it, xs, A.scale_dn, A.out0, A.out_dtype, A.aux0);
+        fused_store_rows_scaled<NC, EC>(A, it, as, A.scale_dn, A.out1, A.out_dtype, A.aux1);
         __syncthreads();
     }
 }
@@ -212,36 +241,53 @@ __global__ void __launch_bounds__(kFusedThreads) fused_backward_kernel(const Fus
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int fl = lane % T::LF, rl = (lane / T::LF) % T::LR, gw = lane / T::LPG;
     const uint32_t rows = A.window * NC;
+    const float om = 1.0f - A.tab.m;
     float* ys = lds;
     float* bs = ys + rows * EC;
     float* gs = bs + rows * EC;
-    float* hs = gs + rows * EC;
-    float* after = hs + rows * EC;
+    float* ps = gs + rows * EC;                                  // p = (1-m) g + h
+    float* w_lds = ps + rows * EC;                               // [kFusedMaxStages][2][EC]
+    float* after = w_lds + kFusedMaxStages * 2 * EC;
     float4* slots = reinterpret_cast<float4*>(after) + wave * (F / 4) * 64;
     float* dw_all = after + (T::LR == 1 ? 0 : kFusedWaves * F * 64);   // [wave][stage][2][EC]
     const int dw_wave_stride = A.n_stages * 2 * EC;
     float* dw_mine = dw_all + wave * dw_wave_stride;
     for (int k = lane; k < dw_wave_stride; k += 64) dw_mine[k] = 0.f;
+    const int head = blockIdx.x % A.n_head;   // == head of every item of this workgroup (gridDim.x % n_head == 0)
+    fused_load_weights<EC>(A, head, w_lds);
 
     for (uint32_t item = blockIdx.x; item < A.total_items; item += gridDim.x) {
         const FusedItem it = fused_item<EC>(A, item);
         fused_load_rows<NC, EC>(A, it, A.in0, A.in_dtype, ys, rows);
         fused_load_rows<NC, EC>(A, it, A.in1, A.in_dtype, bs, rows);
-        fused_load_rows<NC, EC>(A, it, A.g0, A.g_dtype, gs, rows);
-        fused_load_rows<NC, EC>(A, it, A.g1, A.g_dtype, hs, rows);
+        {   // g and p = (1-m) g + h
+            constexpr uint32_t CPR = EC / 4;
+            for (uint32_t c = threadIdx.x; c < rows * CPR; c += kFusedThreads) {
+                const uint32_t lr = c / CPR, c4 = c - lr * CPR;
+                const int64_t off = fused_row_offset<NC>(A, it, lr) + c4 * 4;
+                float g[4], h[4];
+                load_frag<4>(A.g0, A.g_dtype, off, true, g);
+                load_frag<4>(A.g1, A.g_dtype, off, A.g1 != nullptr, h);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) h[k] = fmaf(om, g[k], h[k]);
+                lds_store_frag<4>(gs + lr * EC + c4 * 4, g);
+                lds_store_frag<4>(ps + lr * EC + c4 * 4, h);
+            }
+        }
         __syncthreads();
         for (int st = A.n_stages - 1; st >= 0; --st) {
             const uint32_t ss = A.sub_stride[st];
             const uint32_t ngroups = A.closed ? A.window : A.window - (NC - 1) * ss;
             float wi[F], wj[F], dwi[F], dwj[F];
-            load_w<F>(A.W + (int64_t)st * 2 * A.E, A.E, it.head, EC, fl, wi, wj);
+            lds_load_frag<F>(w_lds + st * 2 * EC + fl * F, wi);
+            lds_load_frag<F>(w_lds + st * 2 * EC + EC + fl * F, wj);
 #pragma unroll
             for (int f = 0; f < F; ++f) dwi[f] = dwj[f] = 0.f;
             for (uint32_t wt = wave; wt * T::GPW < ngroups; wt += kFusedWaves) {
                 const uint32_t qg = wt * T::GPW + gw;
                 const bool valid = qg < ngroups;
-                const float own = (valid && qg - it.own_lo < it.own_cnt) ? 1.0f : 0.0f;  // unsigned compare: lo <= qg < lo+cnt
-                float Y[R][F], B[R][F], G[R][F], H[R][F];
+                const float own = (valid && qg - it.own_lo < it.own_cnt) ? 1.0f : 0.0f;  // unsigned: lo <= qg < lo+cnt
+                float Y[R][F], B[R][F], G[R][F], P[R][F];
                 uint32_t row[R];
 #pragma unroll
                 for (int rr = 0; rr < R; ++rr) {
@@ -249,22 +295,17 @@ __global__ void __launch_bounds__(kFusedThreads) fused_backward_kernel(const Fus
                     lds_load_frag<F>(ys + row[rr], Y[rr]);
                     lds_load_frag<F>(bs + row[rr], B[rr]);
                     lds_load_frag<F>(gs + row[rr], G[rr]);
-                    lds_load_frag<F>(hs + row[rr], H[rr]);
+                    lds_load_frag<F>(ps + row[rr], P[rr]);
                 }
-                backward_steps<NC, EC, R, F, true>(Y, B, G, H, wi, wj, dwi, dwj, own, A.tab, lane, slots);
+                backward_core<NC, EC, R, F, true>(Y, B, G, P, wi, wj, dwi, dwj, own, A.tab, (A.n_stages - 1 - st) * NC,
+                                                  lane, slots);
                 if (valid) {
-                    const float up = A.tab.inv_m_pow_n;
 #pragma unroll
                     for (int rr = 0; rr < R; ++rr) {
-#pragma unroll
-                        for (int f = 0; f < F; ++f) {
-                            Y[rr][f] *= up;
-                            B[rr][f] *= up;
-                        }
                         lds_store_frag<F>(ys + row[rr], Y[rr]);
                         lds_store_frag<F>(bs + row[rr], B[rr]);
                         lds_store_frag<F>(gs + row[rr], G[rr]);
-                        lds_store_frag<F>(hs + row[rr], H[rr]);
+                        lds_store_frag<F>(ps + row[rr], P[rr]);
                     }
                 }
             }
@@ -284,17 +325,32 @@ __global__ void __launch_bounds__(kFusedThreads) fused_backward_kernel(const Fus
             }
             __syncthreads();
         }
-        fused_store_rows<NC, EC>(A, it, gs, A.out0, A.out_dtype);
-        fused_store_rows<NC, EC>(A, it, hs, A.out1, A.out_dtype);
+        {   // owned rows back to true values: g = G m^T, h = P m^T - (1-m) g, x = Y / m^T, xa = B / m^T
+            constexpr uint32_t CPR = EC / 4;
+            const uint32_t r0 = it.own_lo * NC, nrows = it.own_cnt * NC;
+            for (uint32_t c = threadIdx.x; c < nrows * CPR; c += kFusedThreads) {
+                const uint32_t lr = r0 + c / CPR, c4 = c % CPR;
+                const int64_t off = fused_row_offset<NC>(A, it, lr) + c4 * 4;
+                float g[4], h[4];
+                lds_load_frag<4>(gs + lr * EC + c4 * 4, g);
+                lds_load_frag<4>(ps + lr * EC + c4 * 4, h);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    g[k] *= A.scale_dn;
+                    h[k] = fmaf(h[k], A.scale_dn, -om * g[k]);
+                }
+                store_frag<4>(A.out0, A.out_dtype, off, true, g);
+                store_frag<4>(A.out1, A.out_dtype, off, true, h);
+            }
+        }
         if (A.aux0) {
-            fused_store_rows<NC, EC>(A, it, ys, A.aux0, NCN_F32);
-            fused_store_rows<NC, EC>(A, it, bs, A.aux1, NCN_F32);
+            fused_store_rows_scaled<NC, EC>(A, it, ys, A.scale_up, A.aux0, NCN_F32, nullptr);
+            fused_store_rows_scaled<NC, EC>(A, it, bs, A.scale_up, A.aux1, NCN_F32, nullptr);
         }
         __syncthreads();
     }
     __syncthreads();
     // one partial row per workgroup and stage; workgroup b owns slot (b / n_head, head b % n_head)
-    const int head = blockIdx.x % A.n_head;   // == head of every item of this workgroup (gridDim.x % n_head == 0)
     float* prow = A.dw_partials + (int64_t)(blockIdx.x / A.n_head) * A.n_stages * (2 * A.E);
     for (int k = threadIdx.x; k < A.n_stages * 2 * EC; k += kFusedThreads) {
         const int st = k / (2 * EC), rem = k - st * 2 * EC, half = rem / EC, f = rem - half * EC;

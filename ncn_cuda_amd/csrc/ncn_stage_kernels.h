@@ -94,16 +94,19 @@ __device__ __forceinline__ float dot_frag(const float (&a)[F], const float (&b)[
 // The registers hold X = x / m^t and A = xa / m^t after t steps, which turns the two updates into
 //   A <- A + (1-m)/m^(t+1) F   and   X <- X + (1-m) A   (the powers of m come from a host-made table).
 // ---------------------------------------------------------------------------------------------
+// forward_core runs the n_cache steps of one stage on registers that already hold x / m^t0, xa / m^t0 with
+// t0 = step_base steps done before (several stages in a row just keep counting) and leaves them scaled.
 template <int NC, int EC, int R, int F>
-__device__ __forceinline__ void forward_steps(float (&x)[R][F], float (&a)[R][F], const float (&wi)[F],
-                                              const float (&wj)[F], const StepTable& S, int lane, float4* slots) {
+__device__ __forceinline__ void forward_core(float (&x)[R][F], float (&a)[R][F], const float (&wi)[F],
+                                             const float (&wj)[F], const StepTable& S, int step_base, int lane,
+                                             float4* slots) {
     using T = Tile<NC, EC, R, F>;
     const float om = 1.0f - S.m;
 #pragma unroll 1
     for (int jo = 0; jo < T::LR; ++jo) {
 #pragma unroll
         for (int jr = 0; jr < R; ++jr) {
-            const int ts = jo * R + jr;            // steps done so far
+            const int ts = step_base + jo * R + jr;   // steps done so far
             const float lam = S.step[ts].flam;     // z = lam X_i + c_i Xj
             const float kc = S.step[ts].fkc;       // c_i = kc S_i
             const float kap = S.step[ts].fkap;     // A <- A + kap F
@@ -126,6 +129,13 @@ __device__ __forceinline__ void forward_steps(float (&x)[R][F], float (&a)[R][F]
             }
         }
     }
+}
+
+// one stage from true values to true values
+template <int NC, int EC, int R, int F>
+__device__ __forceinline__ void forward_steps(float (&x)[R][F], float (&a)[R][F], const float (&wi)[F],
+                                              const float (&wj)[F], const StepTable& S, int lane, float4* slots) {
+    forward_core<NC, EC, R, F>(x, a, wi, wj, S, 0, lane, slots);
     const float dn = S.m_pow_n;
 #pragma unroll
     for (int rr = 0; rr < R; ++rr)
@@ -202,27 +212,24 @@ __device__ __forceinline__ void inverse_steps(float (&y)[R][F], float (&b)[R][F]
 // dwi, dwj accumulate this lane's share of dWi, dWj; with MASKED the share is weighted by `own` (1, or 0 for a
 // group whose dW another tile accounts for).
 // ---------------------------------------------------------------------------------------------
+// backward_core: the n_cache steps of one stage on registers in the scaled form above with t0 = step_base
+// inversion steps done before (P holds p / m^t0, not h); leaves them scaled by t0 + n_cache steps.
 template <int NC, int EC, int R, int F, bool MASKED>
-__device__ __forceinline__ void backward_steps(float (&Y)[R][F], float (&B)[R][F], float (&G)[R][F], float (&P)[R][F],
-                                               const float (&wi)[F], const float (&wj)[F], float (&dwi)[F],
-                                               float (&dwj)[F], float own, const StepTable& S, int lane,
-                                               float4* slots) {
+__device__ __forceinline__ void backward_core(float (&Y)[R][F], float (&B)[R][F], float (&G)[R][F], float (&P)[R][F],
+                                              const float (&wi)[F], const float (&wj)[F], float (&dwi)[F],
+                                              float (&dwj)[F], float own, const StepTable& S, int step_base, int lane,
+                                              float4* slots) {
     using T = Tile<NC, EC, R, F>;
     const int rl = (lane / T::LF) % T::LR;
     const float om = 1.0f - S.m;
     const float ku = 4.0f * om / S.m * S.alpha;  // G += ku * U        (U = P (r - r^2))
     const float nom = -om;
-#pragma unroll
-    for (int rr = 0; rr < R; ++rr)
-#pragma unroll
-        for (int f = 0; f < F; ++f) P[rr][f] = fmaf(om, G[rr][f], P[rr][f]);  // h -> p
-
 #pragma unroll 1
     for (int jo = T::LR - 1; jo >= 0; --jo) {
         const float sel = (T::LR == 1 || rl == jo) ? 1.0f : 0.0f;  // this lane holds the pivot row
 #pragma unroll
         for (int jr = R - 1; jr >= 0; --jr) {
-            const int ts = (T::LR - 1 - jo) * R + (R - 1 - jr);   // inversion steps done so far
+            const int ts = step_base + (T::LR - 1 - jo) * R + (R - 1 - jr);   // inversion steps done so far
             const float lam = S.step[ts].lam;     // z = lam Y_i + chat_i Yj
             const float kc2 = S.step[ts].kc2;     // chat_i = kc2 S_i
             const float kap = S.step[ts].kap;     // B <- B - kap F
@@ -275,6 +282,21 @@ __device__ __forceinline__ void backward_steps(float (&Y)[R][F], float (&B)[R][F
             __builtin_amdgcn_sched_barrier(0);  // keep steps apart: interleaving them only costs registers
         }
     }
+}
+
+// one stage: G, H true gradients in and out; Y, B true outputs in, m^n_cache times the stage inputs out
+template <int NC, int EC, int R, int F, bool MASKED>
+__device__ __forceinline__ void backward_steps(float (&Y)[R][F], float (&B)[R][F], float (&G)[R][F], float (&P)[R][F],
+                                               const float (&wi)[F], const float (&wj)[F], float (&dwi)[F],
+                                               float (&dwj)[F], float own, const StepTable& S, int lane,
+                                               float4* slots) {
+    const float om = 1.0f - S.m;
+    const float nom = -om;
+#pragma unroll
+    for (int rr = 0; rr < R; ++rr)
+#pragma unroll
+        for (int f = 0; f < F; ++f) P[rr][f] = fmaf(om, G[rr][f], P[rr][f]);  // h -> p
+    backward_core<NC, EC, R, F, MASKED>(Y, B, G, P, wi, wj, dwi, dwj, own, S, 0, lane, slots);
     // undo the scaling of the gradients: NC steps done
     const float dn = S.m_pow_n;       // m^NC
 #pragma unroll

@@ -45,7 +45,8 @@ def test_multi_stage_matches_single_stage_and_oracle(M, case):
         outs.append((cx, cxa))
     # one call for all stages
     y, ya = M.forward_stages(gx, gxa, Wst, alpha, 0, n, C, first, L)
-    assert torch.equal(y, outs[-1][0]) and torch.equal(ya, outs[-1][1])  # same arithmetic, float32 between stages
+    # same arithmetic up to where the powers of m are folded in (per stage vs per pass): rounding-level agreement
+    assert O.rel_err(y, outs[-1][0]) < 2e-6 and O.rel_err(ya, outs[-1][1]) < 2e-6
 
     d = torch.float64
     ref = O.net_autograd(x.to(d), xa.to(d), [w.to(d) for w in Ws], dyi.to(d), dya.to(d), alpha, n, C, first_stage=first)
@@ -67,7 +68,7 @@ def test_multi_stage_matches_single_stage_and_oracle(M, case):
     for l in range(L - 1, -1, -1):
         cy, cya, cg, cga, dWl = M.backward_stages(cy, cya, cg, cga, gWs[l], alpha, 0, n, C, first + l, 1)
         assert O.rel_err(dW[l], dWl[0]) < 1e-5
-    assert O.rel_err(dx, cg) < 1e-6 and O.rel_err(dxa, cga) < 1e-6
+    assert O.rel_err(dx, cg) < tol and O.rel_err(dxa, cga) < tol
 
 
 def test_multi_stage_dya_none_and_bf16_input(M):
