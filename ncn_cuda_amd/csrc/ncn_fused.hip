@@ -22,8 +22,9 @@ size_t fused_lds_bytes(int nc, int ec, bool backward, uint32_t window, int n_sta
     const int lr = nc / t.r;
     size_t bytes = (size_t)(backward ? 4 : 2) * window * nc * ec * sizeof(float);
     bytes += (size_t)kFusedMaxStages * 2 * ec * sizeof(float);  // the pass's weights
-    if (lr > 1) bytes += (size_t)kFusedWaves * t.f * 64 * sizeof(float);
-    if (backward) bytes += (size_t)kFusedWaves * n_stages * 2 * ec * sizeof(float);
+    const int nw = backward ? kFusedWavesBwd : kFusedWavesFwd;
+    if (lr > 1) bytes += (size_t)nw * t.f * 64 * sizeof(float);
+    if (backward) bytes += (size_t)nw * n_stages * 2 * ec * sizeof(float);
     return bytes;
 }
 
@@ -144,12 +145,12 @@ static hipError_t launch_fused_t(bool backward, const FusedArgs& a, int grid, si
         auto k = fused_backward_kernel<NC, EC, t.r, t.f>;
         err = hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (err != hipSuccess) return err;
-        hipLaunchKernelGGL(k, dim3(grid), dim3(kFusedThreads), lds, s, a);
+        hipLaunchKernelGGL(k, dim3(grid), dim3(64 * kFusedWavesBwd), lds, s, a);
     } else {
         auto k = fused_forward_kernel<NC, EC, t.r, t.f>;
         err = hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (err != hipSuccess) return err;
-        hipLaunchKernelGGL(k, dim3(grid), dim3(kFusedThreads), lds, s, a);
+        hipLaunchKernelGGL(k, dim3(grid), dim3(64 * kFusedWavesFwd), lds, s, a);
     }
     return hipGetLastError();
 }

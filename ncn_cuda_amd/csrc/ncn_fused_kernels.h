@@ -30,8 +30,8 @@
 namespace ncn {
 
 constexpr int kFusedMaxStages = 8;
-constexpr int kFusedWaves = 8;
-constexpr int kFusedThreads = 64 * kFusedWaves;
+constexpr int kFusedWavesFwd = 8;   // (16 waves per workgroup measured slower: all waves of a workgroup share its phases)
+constexpr int kFusedWavesBwd = 8;   // backward runs at 128 VGPRs: 4 waves per SIMD in all
 
 struct FusedArgs {
     const void* in0;   // forward: x    backward: y (outputs of the pass's last stage)
@@ -126,11 +126,11 @@ __device__ __forceinline__ void lds_store_frag(float* row, const float (&v)[F]) 
 }
 
 // global -> LDS for every row of the window (4 features per thread and trip)
-template <int NC, int EC>
+template <int NC, int EC, int NW>
 __device__ __forceinline__ void fused_load_rows(const FusedArgs& A, const FusedItem& it, const void* src, int dtype,
                                                 float* dst, uint32_t rows) {
     constexpr uint32_t CPR = EC / 4;
-    for (uint32_t c = threadIdx.x; c < rows * CPR; c += kFusedThreads) {
+    for (uint32_t c = threadIdx.x; c < rows * CPR; c += 64 * NW) {
         const uint32_t lr = c / CPR, c4 = c - lr * CPR;
         float v[4];
         if (src) load_frag<4>(src, dtype, fused_row_offset<NC>(A, it, lr) + c4 * 4, true, v);
@@ -140,12 +140,12 @@ __device__ __forceinline__ void fused_load_rows(const FusedArgs& A, const FusedI
 }
 
 // LDS -> global for the owned rows
-template <int NC, int EC>
+template <int NC, int EC, int NW>
 __device__ __forceinline__ void fused_store_rows(const FusedArgs& A, const FusedItem& it, const float* src, void* dst,
                                                  int dtype) {
     constexpr uint32_t CPR = EC / 4;
     const uint32_t r0 = it.own_lo * NC, rows = it.own_cnt * NC;
-    for (uint32_t c = threadIdx.x; c < rows * CPR; c += kFusedThreads) {
+    for (uint32_t c = threadIdx.x; c < rows * CPR; c += 64 * NW) {
         const uint32_t lr = r0 + c / CPR, c4 = c % CPR;
         float v[4];
         lds_load_frag<4>(src + lr * EC + c4 * 4, v);
@@ -154,12 +154,12 @@ __device__ __forceinline__ void fused_store_rows(const FusedArgs& A, const Fused
 }
 
 // LDS -> global for the owned rows, each value times `scale`
-template <int NC, int EC>
+template <int NC, int EC, int NW>
 __device__ __forceinline__ void fused_store_rows_scaled(const FusedArgs& A, const FusedItem& it, const float* src,
                                                         float scale, void* dst, int dtype, float* copy32) {
     constexpr uint32_t CPR = EC / 4;
     const uint32_t r0 = it.own_lo * NC, rows = it.own_cnt * NC;
-    for (uint32_t c = threadIdx.x; c < rows * CPR; c += kFusedThreads) {
+    for (uint32_t c = threadIdx.x; c < rows * CPR; c += 64 * NW) {
         const uint32_t lr = r0 + c / CPR, c4 = c % CPR;
         float v[4];
         lds_load_frag<4>(src + lr * EC + c4 * 4, v);
@@ -172,16 +172,17 @@ __device__ __forceinline__ void fused_store_rows_scaled(const FusedArgs& A, cons
 }
 
 // the pass's weights, [stage][Wi | Wj][EC] of this workgroup's head, into LDS
-template <int EC>
+template <int EC, int NW>
 __device__ __forceinline__ void fused_load_weights(const FusedArgs& A, int head, float* w_lds) {
-    for (int k = threadIdx.x; k < A.n_stages * 2 * EC; k += kFusedThreads) {
+    for (int k = threadIdx.x; k < A.n_stages * 2 * EC; k += 64 * NW) {
         const int st = k / (2 * EC), rem = k - st * 2 * EC, half = rem / EC, f = rem - half * EC;
         w_lds[k] = A.W[(int64_t)st * 2 * A.E + (int64_t)half * A.E + (int64_t)head * EC + f];
     }
 }
 
 template <int NC, int EC, int R, int F>
-__global__ void __launch_bounds__(kFusedThreads) fused_forward_kernel(const FusedArgs A) {
+__global__ void __launch_bounds__(64 * kFusedWavesFwd) fused_forward_kernel(const FusedArgs A) {
+    constexpr int NW = kFusedWavesFwd;
     using T = Tile<NC, EC, R, F>;
     extern __shared__ float4 fused_lds4[];
     float* lds = reinterpret_cast<float*>(fused_lds4);
@@ -192,12 +193,12 @@ __global__ void __launch_bounds__(kFusedThreads) fused_forward_kernel(const Fuse
     float* as = lds + rows * EC;
     float* w_lds = as + rows * EC;                              // [kFusedMaxStages][2][EC]
     float4* slots = reinterpret_cast<float4*>(w_lds + kFusedMaxStages * 2 * EC) + wave * (F / 4) * 64;
-    fused_load_weights<EC>(A, blockIdx.x % A.n_head, w_lds);   // every item of this workgroup has this head
+    fused_load_weights<EC, NW>(A, blockIdx.x % A.n_head, w_lds);   // every item of this workgroup has this head
 
     for (uint32_t item = blockIdx.x; item < A.total_items; item += gridDim.x) {
         const FusedItem it = fused_item<EC>(A, item);
-        fused_load_rows<NC, EC>(A, it, A.in0, A.in_dtype, xs, rows);
-        fused_load_rows<NC, EC>(A, it, A.in1, A.in_dtype, as, rows);
+        fused_load_rows<NC, EC, NW>(A, it, A.in0, A.in_dtype, xs, rows);
+        fused_load_rows<NC, EC, NW>(A, it, A.in1, A.in_dtype, as, rows);
         __syncthreads();
         for (int st = 0; st < A.n_stages; ++st) {
             const uint32_t ss = A.sub_stride[st];
@@ -205,7 +206,7 @@ __global__ void __launch_bounds__(kFusedThreads) fused_forward_kernel(const Fuse
             float wi[F], wj[F];
             lds_load_frag<F>(w_lds + st * 2 * EC + fl * F, wi);
             lds_load_frag<F>(w_lds + st * 2 * EC + EC + fl * F, wj);
-            for (uint32_t wt = wave; wt * T::GPW < ngroups; wt += kFusedWaves) {
+            for (uint32_t wt = wave; wt * T::GPW < ngroups; wt += NW) {
                 const uint32_t qg = wt * T::GPW + gw;
                 const bool valid = qg < ngroups;
                 float x[R][F], a[R][F];
@@ -227,14 +228,15 @@ __global__ void __launch_bounds__(kFusedThreads) fused_forward_kernel(const Fuse
             }
             __syncthreads();
         }
-        fused_store_rows_scaled<NC, EC>(A, it, xs, A.scale_dn, A.out0, A.out_dtype, A.aux0);
-        fused_store_rows_scaled<NC, EC>(A, it, as, A.scale_dn, A.out1, A.out_dtype, A.aux1);
+        fused_store_rows_scaled<NC, EC, NW>(A, it, xs, A.scale_dn, A.out0, A.out_dtype, A.aux0);
+        fused_store_rows_scaled<NC, EC, NW>(A, it, as, A.scale_dn, A.out1, A.out_dtype, A.aux1);
         __syncthreads();
     }
 }
 
 template <int NC, int EC, int R, int F>
-__global__ void __launch_bounds__(kFusedThreads) fused_backward_kernel(const FusedArgs A) {
+__global__ void __launch_bounds__(64 * kFusedWavesBwd) fused_backward_kernel(const FusedArgs A) {
+    constexpr int NW = kFusedWavesBwd;
     using T = Tile<NC, EC, R, F>;
     extern __shared__ float4 fused_lds4[];
     float* lds = reinterpret_cast<float*>(fused_lds4);
@@ -249,20 +251,20 @@ __global__ void __launch_bounds__(kFusedThreads) fused_backward_kernel(const Fus
     float* w_lds = ps + rows * EC;                               // [kFusedMaxStages][2][EC]
     float* after = w_lds + kFusedMaxStages * 2 * EC;
     float4* slots = reinterpret_cast<float4*>(after) + wave * (F / 4) * 64;
-    float* dw_all = after + (T::LR == 1 ? 0 : kFusedWaves * F * 64);   // [wave][stage][2][EC]
+    float* dw_all = after + (T::LR == 1 ? 0 : NW * F * 64);   // [wave][stage][2][EC]
     const int dw_wave_stride = A.n_stages * 2 * EC;
     float* dw_mine = dw_all + wave * dw_wave_stride;
     for (int k = lane; k < dw_wave_stride; k += 64) dw_mine[k] = 0.f;
     const int head = blockIdx.x % A.n_head;   // == head of every item of this workgroup (gridDim.x % n_head == 0)
-    fused_load_weights<EC>(A, head, w_lds);
+    fused_load_weights<EC, NW>(A, head, w_lds);
 
     for (uint32_t item = blockIdx.x; item < A.total_items; item += gridDim.x) {
         const FusedItem it = fused_item<EC>(A, item);
-        fused_load_rows<NC, EC>(A, it, A.in0, A.in_dtype, ys, rows);
-        fused_load_rows<NC, EC>(A, it, A.in1, A.in_dtype, bs, rows);
+        fused_load_rows<NC, EC, NW>(A, it, A.in0, A.in_dtype, ys, rows);
+        fused_load_rows<NC, EC, NW>(A, it, A.in1, A.in_dtype, bs, rows);
         {   // g and p = (1-m) g + h
             constexpr uint32_t CPR = EC / 4;
-            for (uint32_t c = threadIdx.x; c < rows * CPR; c += kFusedThreads) {
+            for (uint32_t c = threadIdx.x; c < rows * CPR; c += 64 * NW) {
                 const uint32_t lr = c / CPR, c4 = c - lr * CPR;
                 const int64_t off = fused_row_offset<NC>(A, it, lr) + c4 * 4;
                 float g[4], h[4];
@@ -283,7 +285,7 @@ __global__ void __launch_bounds__(kFusedThreads) fused_backward_kernel(const Fus
             lds_load_frag<F>(w_lds + st * 2 * EC + EC + fl * F, wj);
 #pragma unroll
             for (int f = 0; f < F; ++f) dwi[f] = dwj[f] = 0.f;
-            for (uint32_t wt = wave; wt * T::GPW < ngroups; wt += kFusedWaves) {
+            for (uint32_t wt = wave; wt * T::GPW < ngroups; wt += NW) {
                 const uint32_t qg = wt * T::GPW + gw;
                 const bool valid = qg < ngroups;
                 const float own = (valid && qg - it.own_lo < it.own_cnt) ? 1.0f : 0.0f;  // unsigned: lo <= qg < lo+cnt
@@ -328,7 +330,7 @@ __global__ void __launch_bounds__(kFusedThreads) fused_backward_kernel(const Fus
         {   // owned rows back to true values: g = G m^T, h = P m^T - (1-m) g, x = Y / m^T, xa = B / m^T
             constexpr uint32_t CPR = EC / 4;
             const uint32_t r0 = it.own_lo * NC, nrows = it.own_cnt * NC;
-            for (uint32_t c = threadIdx.x; c < nrows * CPR; c += kFusedThreads) {
+            for (uint32_t c = threadIdx.x; c < nrows * CPR; c += 64 * NW) {
                 const uint32_t lr = r0 + c / CPR, c4 = c % CPR;
                 const int64_t off = fused_row_offset<NC>(A, it, lr) + c4 * 4;
                 float g[4], h[4];
@@ -344,19 +346,19 @@ __global__ void __launch_bounds__(kFusedThreads) fused_backward_kernel(const Fus
             }
         }
         if (A.aux0) {
-            fused_store_rows_scaled<NC, EC>(A, it, ys, A.scale_up, A.aux0, NCN_F32, nullptr);
-            fused_store_rows_scaled<NC, EC>(A, it, bs, A.scale_up, A.aux1, NCN_F32, nullptr);
+            fused_store_rows_scaled<NC, EC, NW>(A, it, ys, A.scale_up, A.aux0, NCN_F32, nullptr);
+            fused_store_rows_scaled<NC, EC, NW>(A, it, bs, A.scale_up, A.aux1, NCN_F32, nullptr);
         }
         __syncthreads();
     }
     __syncthreads();
     // one partial row per workgroup and stage; workgroup b owns slot (b / n_head, head b % n_head)
     float* prow = A.dw_partials + (int64_t)(blockIdx.x / A.n_head) * A.n_stages * (2 * A.E);
-    for (int k = threadIdx.x; k < A.n_stages * 2 * EC; k += kFusedThreads) {
+    for (int k = threadIdx.x; k < A.n_stages * 2 * EC; k += 64 * NW) {
         const int st = k / (2 * EC), rem = k - st * 2 * EC, half = rem / EC, f = rem - half * EC;
         float sum = 0.f;
 #pragma unroll
-        for (int w = 0; w < kFusedWaves; ++w) sum += dw_all[w * dw_wave_stride + st * 2 * EC + rem];
+        for (int w = 0; w < NW; ++w) sum += dw_all[w * dw_wave_stride + st * 2 * EC + rem];
         prow[(int64_t)st * (2 * A.E) + (int64_t)half * A.E + (int64_t)head * EC + f] = sum;
     }
 }
