@@ -141,6 +141,17 @@ size_t ncn_workspace_bytes(const ncn_shape* shape);
  * (0 for forward, ncn_workspace_bytes for backward).  No reference counterpart. */
 size_t ncn_workspace_bytes_stages(const ncn_shape* shape, int first_stage, int n_stages, int activation, int backward);
 
+/* How ncn_forward / ncn_backward would cut stages first_stage .. first_stage+n_stages-1 into passes, for
+ * inspection and tests.  Returns the number of passes (0: one launch per stage), or a negative error code;
+ * writes up to max_passes records of 8 int32 into `out` (may be NULL):
+ *   [0] first stage of the pass relative to first_stage   [1] stages in the pass
+ *   [2] kind: 0 one-stage launch, 1 halo window, 2 closed rings
+ *   [3] class stride S0 in blocks   [4] window   [5] halo   [6] owned sub-blocks per window
+ *   [7] windows per batch entry and ring tile (classes, or groups of classes for closed rings)
+ * No reference counterpart. */
+int ncn_plan_passes(const ncn_shape* shape, int first_stage, int n_stages, int activation, int backward, int32_t* out,
+                    int max_passes);
+
 /* 2: hand-tuned register kernel, 1: generic LDS kernel, 0: not supported (n_cache > 64, or the
  * head width does not fit the generic kernel's LDS).  No reference counterpart. */
 int ncn_kernel_path(const ncn_shape* shape);

@@ -12,7 +12,7 @@ NCN_F32, NCN_BF16 = 0, 1
 ACT_TANH, ACT_RELU, ACT_SIGMOID, ACT_LINEAR = 0, 1, 2, -1
 
 EXPORTS = ("ncn_forward", "ncn_backward", "ncn_inverse", "ncn_workspace_bytes", "ncn_workspace_bytes_stages",
-           "ncn_kernel_path",
+           "ncn_plan_passes", "ncn_kernel_path",
            "ncn_check_shape", "ncn_error_string", "ncn_version")
 
 
@@ -47,6 +47,8 @@ def load():
     lib.ncn_workspace_bytes.argtypes = [shp]
     lib.ncn_workspace_bytes_stages.restype = ctypes.c_size_t
     lib.ncn_workspace_bytes_stages.argtypes = [shp, i, i, i, i]
+    lib.ncn_plan_passes.restype = i
+    lib.ncn_plan_passes.argtypes = [shp, i, i, i, i, ctypes.POINTER(ctypes.c_int32), i]
     lib.ncn_kernel_path.restype = i
     lib.ncn_kernel_path.argtypes = [shp]
     lib.ncn_check_shape.restype = i

@@ -141,7 +141,25 @@ size_t temp_bytes(const ncn_shape* sh, bool backward) {
 
 extern "C" {
 
-const char* ncn_version(void) { return "0.1"; }
+const char* ncn_version(void) { return "0.2"; }
+
+int ncn_plan_passes(const ncn_shape* shape, int first_stage, int n_stages, int activation, int backward, int32_t* out,
+                    int max_passes) {
+    int rc = check_shape(shape, first_stage, n_stages, activation);
+    if (rc != NCN_OK) return rc;
+    const std::vector<FusedPass> passes = multi_stage_plan(shape, first_stage, n_stages, activation, backward != 0);
+    int k = 0;
+    for (const FusedPass& p : passes) {
+        if (out && k < max_passes) {
+            int32_t* o = out + 8 * k;
+            o[0] = p.first; o[1] = p.count; o[2] = p.single ? 0 : (p.closed ? 2 : 1);
+            o[3] = (int32_t)p.class_stride; o[4] = (int32_t)p.window; o[5] = (int32_t)p.halo; o[6] = (int32_t)p.own;
+            o[7] = (int32_t)p.class_groups;
+        }
+        ++k;
+    }
+    return k;
+}
 
 const char* ncn_error_string(int code) {
     switch (code) {
@@ -203,7 +221,9 @@ int ncn_forward(const void* x, const void* xa, int in_dtype, void* y, void* ya, 
     const size_t np = passes.size();
     bool fused_ok = np > 0;
     if (np >= 2 && (out_dtype != NCN_F32 || !workspace || workspace_bytes < temp_bytes(shape, false))) fused_ok = false;
-    if (np == 1 && !passes[0].closed && (x == y || xa == ya)) fused_ok = false;  // a halo pass cannot run in place
+    // a halo pass (or a one-stage launch feeding one) must not write where another workgroup still reads its halo:
+    // refuse the in-place case when the first pass would write straight into x, xa
+    if (np >= 1 && (x == y || xa == ya) && ((np - 1) % 2) == 0 && !passes[0].closed && !passes[0].single) fused_ok = false;
     if (fused_ok) {
         const size_t one = temp_bytes(shape, false) / 2;
         void* t0 = workspace;
@@ -316,7 +336,9 @@ int ncn_backward(const void* y, const void* ya, int y_dtype, const void* dy, con
     const size_t np = passes.size();
     bool fused_ok = np > 0;
     if (np >= 2 && workspace_bytes < base_workspace_bytes(shape) + temp_bytes(shape, true)) fused_ok = false;
-    if (np == 1 && !passes[0].closed && (y == x_rec || ya == xa_rec || dy == dx || (dya && dya == dxa))) fused_ok = false;
+    if (np >= 1 && ((np - 1) % 2) == 0 && !passes[np - 1].closed && !passes[np - 1].single &&
+        (y == x_rec || ya == xa_rec || dy == dx || (dya && dya == dxa)))
+        fused_ok = false;  // the first pass to run is a halo pass and would write into its own input
     if (fused_ok) {
         const size_t one = temp_bytes(shape, true) / 4;
         char* tb = static_cast<char*>(workspace) + base_workspace_bytes(shape);

@@ -30,7 +30,7 @@ def _declared_functions():
 def test_header_functions_are_exported(lib):
     names = _declared_functions()
     assert {"ncn_forward", "ncn_backward", "ncn_inverse", "ncn_workspace_bytes", "ncn_workspace_bytes_stages",
-            "ncn_kernel_path",
+            "ncn_plan_passes", "ncn_kernel_path",
             "ncn_check_shape", "ncn_error_string", "ncn_version"} <= set(names)
     handle = lib.load()
     for name in names:
@@ -124,13 +124,16 @@ def test_surface_matches_reference_names():
     import inspect
 
     import ncn_cuda_amd as pkg
+    def positional(fn):  # keyword-only extras (fuse_stages, save_every) are additions, not part of the reference
+        return [n for n, q in inspect.signature(fn).parameters.items() if q.kind != q.KEYWORD_ONLY]
+
     assert list(inspect.signature(pkg.fused_ncn_cuda_v2).parameters) == [
         "x", "xa", "W", "alpha", "activation", "n_cache", "n_head", "module_l"]
-    assert list(inspect.signature(pkg.NCNModuleCuda.__init__).parameters)[1:] == [
+    assert positional(pkg.NCNModuleCuda.__init__)[1:] == [
         "alpha", "activation", "n_cache", "n_head", "module_nr", "embed_dim"]
-    assert list(inspect.signature(pkg.NCNNetCuda.__init__).parameters)[1:] == [
+    assert positional(pkg.NCNNetCuda.__init__)[1:] == [
         "alpha", "activation", "n_cache", "n_head", "num_modules", "embed_dim"]
-    assert list(inspect.signature(pkg.NCNNetTestCuda.__init__).parameters)[1:] == [
+    assert positional(pkg.NCNNetTestCuda.__init__)[1:] == [
         "alpha", "activation", "n_cache", "n_head", "num_modules", "weights"]
     net = pkg.NCNNetCuda(0.9, "tanh", 4, 2, 3, 16)
     assert sorted(net.state_dict()) == ["ncn_modules.0.weight", "ncn_modules.1.weight", "ncn_modules.2.weight"]
@@ -145,3 +148,54 @@ def test_product_code_never_imports_the_oracle():
             if f.endswith((".py", ".h", ".hip")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text.lower() or f == "never", (dirpath, f)
+
+
+def _passes(lib, shape, first, count, backward):
+    buf = (ctypes.c_int32 * (8 * 32))()
+    k = lib.load().ncn_plan_passes(ctypes.byref(shape), first, count, 0, int(backward), buf, 32)
+    assert 0 <= k <= 32
+    return [tuple(buf[8 * j:8 * j + 8]) for j in range(k)]
+
+
+@pytest.mark.parametrize("backward", [False, True])
+@pytest.mark.parametrize("dims", [(128, 8192, 128, 4, 2, 0, 13), (32, 1024, 128, 4, 4, 0, 5), (3, 1024, 64, 2, 2, 0, 11),
+                                  (2, 2048, 64, 2, 2, 3, 6), (5, 64, 128, 4, 4, 0, 3), (1, 1 << 16, 32, 1, 2, 0, 20)])
+def test_multi_stage_plan_invariants(lib, dims, backward):
+    """The pass planner (host logic): passes tile the stage range in order; a halo window owns what its halo leaves,
+    and the halo is (n_cache - 1) * sum of the pass's strides in sub-blocks; closed passes own their whole window."""
+    batch, N, E, C, n, first, count = dims
+    shape = _shape(lib, batch, N, E, C, n)
+    groups = N // n
+    passes = _passes(lib, shape, first, count, backward)
+    assert passes, "these shapes are eligible for multi-stage passes"
+    nxt = 0
+    for (p_first, p_count, kind, s0, window, halo, own, cgroups) in passes:
+        assert p_first == nxt and p_count >= 1
+        nxt += p_count
+        strides = [(0 if (first + p_first + k) == 0 else (1 << (first + p_first + k - 1)) % groups) for k in range(p_count)]
+        if kind == 0:
+            assert p_count == 1
+            continue
+        assert p_count >= 2 and p_count <= 8
+        assert window & (window - 1) == 0 and window <= groups
+        nz = [s for s in strides if s]
+        assert all(s % s0 == 0 for s in nz)
+        ring = groups // s0
+        rows_bytes = window * n * (E // C) * 4 * (4 if backward else 2)
+        assert rows_bytes <= 64 * 1024
+        if kind == 2:
+            assert ring <= window and halo == 0 and own == window and cgroups * (window // ring) == s0
+        else:
+            assert ring > window and cgroups == s0
+            assert halo == (n - 1) * sum(s // s0 for s in strides)
+            assert own == window - 2 * halo and 4 * own >= 3 * window
+    assert nxt == count
+
+
+def test_multi_stage_plan_declines_ineligible_shapes(lib):
+    assert _passes(lib, _shape(lib, 128, 4096, 128, 4, 16), 0, 3, False) == []   # n_cache = 16: arithmetic-bound
+    assert _passes(lib, _shape(lib, 2, 96, 32, 4, 4), 0, 3, False) == []         # 24 groups: not a power of two
+    assert _passes(lib, _shape(lib, 2, 1024, 128, 4, 2), 0, 1, False) == []      # a single stage
+    # the deep configuration: three passes forward, four at most backward, closed rings last
+    fwd = _passes(lib, _shape(lib, 128, 8192, 128, 4, 2), 0, 13, False)
+    assert [p[2] for p in fwd][-1] == 2 and len(fwd) <= 4
