@@ -1,6 +1,6 @@
 """MI355X (gfx950) implementation of the NCN layer behind the reference's Python surface."""
 from . import ncn_cuda_module
-from .ncn_pytorch_wrapper_v2 import (ACTIVATION_CODES, NCNFunction, NCNModuleCuda, NCNNetCuda, NCNNetFunction,
+from .modules import (ACTIVATION_CODES, NCNFunction, NCNModuleCuda, NCNNetCuda, NCNNetFunction,
                                      NCNNetTestCuda, default_save_every, fused_ncn_cuda_v2, fused_ncn_net, ncn_inverse)
 
 __all__ = ["ncn_cuda_module", "ACTIVATION_CODES", "NCNFunction", "NCNModuleCuda", "NCNNetCuda", "NCNNetTestCuda",

@@ -21,7 +21,7 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 int kernel_path(const ncn_shape* sh, int activation) {
     if (sh->n_cache < 1 || sh->n_cache > 64) return 0;
     const int64_t ec = sh->E / sh->n_head;
-    if (activation == NCN_ACT_TANH && ec <= 64 && fast_tile(sh->n_cache, (int)ec).r != 0) return 2;
+    if (activation == NCN_ACT_TANH && ec <= 128 && fast_tile(sh->n_cache, (int)ec).r != 0) return 2;
     if (ec <= kGenericMaxHeadDim) return 1;
     return 0;
 }
@@ -169,7 +169,7 @@ const char* ncn_error_string(int code) {
         case NCN_ERR_DTYPE: return "unknown element type (0 = float32, 1 = bfloat16)";
         case NCN_ERR_ACTIVATION: return "unknown activation code (0 tanh, 1 relu, 2 sigmoid, -1 linear)";
         case NCN_ERR_WORKSPACE: return "workspace is NULL or smaller than ncn_workspace_bytes()";
-        case NCN_ERR_UNSUPPORTED: return "unsupported shape: n_cache must be <= 64 and the head width <= 64";
+        case NCN_ERR_UNSUPPORTED: return "unsupported shape: n_cache must be <= 64 and the head width <= 64 (128 for power-of-two n_cache <= 16 with tanh)";
         case NCN_ERR_ALIGN: return "a pointer is not 16-byte aligned";
         case NCN_ERR_ALIAS: return "n_stages > 1 needs float32 x_rec, xa_rec, dx, dxa to carry the state";
         default: break;

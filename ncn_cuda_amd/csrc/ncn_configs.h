@@ -8,4 +8,5 @@
     X(2, 8, 2, 4) X(4, 8, 2, 4) X(8, 8, 4, 4) X(16, 8, 4, 4) X(32, 8, 4, 4) X(64, 8, 4, 4) \
     X(2, 16, 2, 4) X(4, 16, 2, 4) X(8, 16, 4, 4) X(16, 16, 4, 4) X(32, 16, 4, 4) X(64, 16, 4, 4) \
     X(2, 32, 2, 4) X(4, 32, 2, 4) X(8, 32, 4, 4) X(16, 32, 4, 4) X(32, 32, 4, 4) X(64, 32, 4, 8) \
-    X(2, 64, 2, 8) X(4, 64, 2, 8) X(8, 64, 4, 8) X(16, 64, 4, 8) X(32, 64, 4, 8)
+    X(2, 64, 2, 8) X(4, 64, 2, 8) X(8, 64, 4, 8) X(16, 64, 4, 8) X(32, 64, 4, 8) \
+    X(2, 128, 2, 8) X(4, 128, 2, 8) X(8, 128, 4, 8) X(16, 128, 4, 8)

@@ -1,194 +1,4 @@
-"""autograd.Function / nn.Module surface of the reference's ncn_cuda/ncn_pytorch_wrapper_v2.py.
-
-Same class and function names, same constructor and call signatures, same state_dict keys
-(`weight`, `ncn_modules.{l}.weight`), so a model written against the reference imports these
-instead and changes nothing else.  Behavioural differences:
-  * NCNModuleCuda.forward passes (n_cache, n_head) in the order fused_ncn_cuda_v2 expects; the
-    reference swaps them (ncn_pytorch_wrapper_v2.py:93-102 vs :53-62), which only works when both
-    are equal;
-  * reset_parameters uses the stored embed_dim (the reference reads an attribute it never sets,
-    ncn_pytorch_wrapper_v2.py:87-90);
-  * bfloat16 inputs are supported: the node then saves float32 copies of its outputs, because the
-    reversible backward divides by m at every step and would amplify bf16 rounding past 2e-2.
-"""
-import math
-from typing import Tuple
-
-import torch
-from torch import nn
-
-from . import ncn_cuda_module
-
-ACTIVATION_CODES = {"tanh": 0, "relu": 1, "sigmoid": 2, "linear": -1}  # ncn_pytorch_wrapper_v2.py:111
-
-
-class NCNFunction(torch.autograd.Function):
-    """One stage.  forward saves (yi, ya, W) and inverts them in backward, like the reference node
-    (ncn_pytorch_wrapper_v2.py:9-50)."""
-
-    @staticmethod
-    def forward(ctx, x, xa, W, alpha, activation, n_cache, n_head, module_l):
-        if x.dtype == torch.float32:
-            yi, ya = ncn_cuda_module.forward_stages(x, xa, W, alpha, activation, n_cache, n_head, module_l, 1)
-            ctx.save_for_backward(yi, ya, W)
-        else:
-            yi, ya, y32, ya32 = ncn_cuda_module.forward_stages(x, xa, W, alpha, activation, n_cache, n_head,
-                                                               module_l, 1, save_fp32=True)
-            ctx.save_for_backward(y32, ya32, W)
-        ctx.alpha = alpha
-        ctx.activation = activation
-        ctx.n_cache = n_cache
-        ctx.n_head = n_head
-        ctx.module_l = module_l
-        ctx.io_dtype = x.dtype
-        return yi, ya
-
-    @staticmethod
-    def backward(ctx, dyi, dya):
-        (yi, ya, W) = ctx.saved_tensors
-        _, _, dx, dxa, dW = ncn_cuda_module.backward_stages(
-            yi, ya, dyi, dya, W, ctx.alpha, ctx.activation, ctx.n_cache, ctx.n_head, ctx.module_l, 1,
-            grad_dtype=ctx.io_dtype, want_inputs=False)
-        sum_dW = dW.reshape(W.shape).to(W.dtype)
-        return dx, dxa, sum_dW, None, None, None, None, None
-
-
-def default_save_every(n_cache: int) -> int:
-    """Stages per saved checkpoint of the whole-net node: the reversible backward amplifies float32 rounding by
-    (1/m)^(n_cache * stages) between checkpoints; 26 steps keep that below 16x at m = 0.9."""
-    return max(1, 26 // max(1, int(n_cache)))
-
-
-class NCNNetFunction(torch.autograd.Function):
-    """The whole stage stack as ONE autograd node (no counterpart in the reference, which chains one NCNFunction
-    per stage, ncn_pytorch_wrapper_v2.py:107-117).  Stages run `save_every` at a time through the library's
-    multi-stage calls; only the float32 outputs of every `save_every`-th stage are kept for backward, which
-    reverses each segment from its outputs.  Inter-stage activations stay float32 whatever the I/O dtype."""
-
-    @staticmethod
-    def forward(ctx, x, xa, alpha, activation, n_cache, n_head, first_stage, save_every, *weights):
-        L = len(weights)
-        save_every = default_save_every(n_cache) if not save_every else int(save_every)
-        W = torch.stack([w.detach().reshape(-1).to(torch.float32) for w in weights])
-        saved = []
-        cx, cxa = x, xa
-        segs = [(a, min(save_every, L - a)) for a in range(0, L, save_every)]
-        for a, cnt in segs:
-            cx, cxa = ncn_cuda_module.forward_stages(cx, cxa, W[a:a + cnt], alpha, activation, n_cache, n_head,
-                                                     first_stage + a, cnt, out_dtype=torch.float32)
-            saved.extend([cx, cxa])
-        ctx.save_for_backward(W, *saved)
-        ctx.cfg = (alpha, activation, n_cache, n_head, first_stage, segs, x.dtype, [w.dtype for w in weights],
-                   [w.shape for w in weights])
-        return cx.to(x.dtype), cxa.to(x.dtype)
-
-    @staticmethod
-    def backward(ctx, dyi, dya):
-        W, *saved = ctx.saved_tensors
-        alpha, activation, n_cache, n_head, first_stage, segs, io_dtype, w_dtypes, w_shapes = ctx.cfg
-        dWs = [None] * W.shape[0]
-        g, ga = dyi, dya
-        for k in range(len(segs) - 1, -1, -1):
-            a, cnt = segs[k]
-            _, _, g, ga, dW = ncn_cuda_module.backward_stages(
-                saved[2 * k], saved[2 * k + 1], g, ga, W[a:a + cnt], alpha, activation, n_cache, n_head,
-                first_stage + a, cnt, grad_dtype=torch.float32, want_inputs=cnt > 1)
-            for j in range(cnt):
-                dWs[a + j] = dW[j].reshape(w_shapes[a + j]).to(w_dtypes[a + j])
-        return (g.to(io_dtype), ga.to(io_dtype), None, None, None, None, None, None, *dWs)
-
-
-def fused_ncn_net(x, xa, weights, alpha, activation, n_cache, n_head, first_stage=0, save_every=None):
-    """Stages first_stage .. first_stage+len(weights)-1 as one autograd node; activation is the int code."""
-    return NCNNetFunction.apply(x, xa, alpha, activation, n_cache, n_head, first_stage, save_every, *weights)
-
-
-def fused_ncn_cuda_v2(
-    x: torch.Tensor,
-    xa: torch.Tensor,
-    W: torch.Tensor,
-    alpha: float,
-    activation: int,
-    n_cache: int,
-    n_head: int,
-    module_l: int,
-) -> Tuple[torch.Tensor, torch.Tensor]:
-    yi, ya = NCNFunction.apply(x, xa, W, alpha, activation, n_cache, n_head, module_l)
-    return yi, ya
-
-
-class NCNModuleCuda(nn.Module):
-    def __init__(self, alpha, activation, n_cache, n_head, module_nr, embed_dim):
-        super().__init__()
-        self.alpha = alpha
-        self.activation = activation
-        self.n_cache = n_cache
-        self.n_head = n_head
-        self.module_nr = module_nr
-        self.embed_dim = embed_dim
-        self.weight = nn.Parameter(torch.ones(2 * embed_dim).normal_(mean=0.0, std=1 / (2.0 * embed_dim)),
-                                   requires_grad=True)
-
-    def reset_parameters(self):
-        stdv = 1.0 / math.sqrt(self.embed_dim)
-        for weight in self.parameters():
-            weight.data.uniform_(-stdv, +stdv)
-
-    def forward(self, x, xa):
-        return fused_ncn_cuda_v2(x, xa, self.weight, self.alpha, self.activation, self.n_cache, self.n_head,
-                                 self.module_nr)
-
-
-class NCNNetCuda(nn.Module):
-    """Same constructor as the reference.  `fuse_stages=True` (keyword only, not in the reference) runs the stack as
-    one NCNNetFunction node instead of one node per module; parameters and state_dict are the same either way."""
-
-    def __init__(self, alpha, activation, n_cache, n_head, num_modules, embed_dim, *, fuse_stages=False,
-                 save_every=None):
-        super().__init__()
-        self.num_modules = num_modules
-        self.alpha = alpha
-        self.activation_nr = ACTIVATION_CODES[activation]
-        self.n_cache = n_cache
-        self.n_head = n_head
-        self.fuse_stages = fuse_stages
-        self.save_every = save_every
-        self.ncn_modules = nn.ModuleList(
-            [NCNModuleCuda(alpha, self.activation_nr, n_cache, n_head, module_nr, embed_dim)
-             for module_nr in range(num_modules)])
-
-    def forward(self, x, xa):
-        if self.fuse_stages:
-            return fused_ncn_net(x, xa, [m.weight for m in self.ncn_modules], self.alpha, self.activation_nr,
-                                 self.n_cache, self.n_head, 0, self.save_every)
-        for module_nr in range(self.num_modules):
-            x, xa = self.ncn_modules[module_nr](x, xa)
-        return x, xa
-
-
-class NCNNetTestCuda(nn.Module):
-    def __init__(self, alpha, activation, n_cache, n_head, num_modules, weights, *, fuse_stages=False, save_every=None):
-        super().__init__()
-        self.num_modules = num_modules
-        self.alpha = alpha
-        self.activation_nr = ACTIVATION_CODES[activation]
-        self.n_cache = n_cache
-        self.n_head = n_head
-        self.weights = weights
-        self.fuse_stages = fuse_stages
-        self.save_every = save_every
-
-    def forward(self, x, xa):
-        if self.fuse_stages:
-            return fused_ncn_net(x, xa, list(self.weights[:self.num_modules]), self.alpha, self.activation_nr,
-                                 self.n_cache, self.n_head, 0, self.save_every)
-        for module_nr in range(self.num_modules):
-            x, xa = fused_ncn_cuda_v2(x, xa, self.weights[module_nr], self.alpha, self.activation_nr,
-                                      self.n_cache, self.n_head, module_nr)
-        return x, xa
-
-
-def ncn_inverse(y, ya, W, alpha, activation, n_cache, n_head, module_l):
-    """Inputs of one stage from its outputs (no autograd)."""
-    x, xa = ncn_cuda_module.inverse_stages(y, ya, W, alpha, activation, n_cache, n_head, module_l, 1)
-    return x, xa
+"""Import alias: `from ncn_cuda_amd.ncn_pytorch_wrapper_v2 import NCNNetCuda` works like the reference's module path
+(ncn_cuda/ncn_pytorch_wrapper_v2.py); the classes live in ncn_cuda_amd/modules.py."""
+from .modules import *  # noqa: F401,F403
+from .modules import __all__  # noqa: F401

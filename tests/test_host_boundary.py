@@ -55,7 +55,9 @@ def test_check_shape_codes(lib):
     assert h.ncn_check_shape(ctypes.byref(ok), 0, 0, 0) == -2
     assert h.ncn_check_shape(ctypes.byref(ok), 0, 1, 7) == -4                             # activation
     assert h.ncn_check_shape(ctypes.byref(_shape(lib, 1, 256, 32, 4, 128)), 0, 1, 0) == -6  # n_cache > 64
-    assert h.ncn_check_shape(ctypes.byref(_shape(lib, 1, 64, 512, 4, 4)), 0, 1, 0) == -6    # head width 128
+    assert h.ncn_check_shape(ctypes.byref(_shape(lib, 1, 64, 512, 4, 4)), 0, 1, 0) == 0     # head width 128: register kernel
+    assert h.ncn_check_shape(ctypes.byref(_shape(lib, 1, 64, 512, 4, 4)), 0, 1, 1) == -6    # .. but not with relu
+    assert h.ncn_check_shape(ctypes.byref(_shape(lib, 1, 64, 1024, 4, 4)), 0, 1, 0) == -6   # head width 256
     for code in (0, -1, -2, -3, -4, -5, -6, -7, -8):
         assert len(h.ncn_error_string(code)) > 0
 
@@ -199,3 +201,12 @@ def test_multi_stage_plan_declines_ineligible_shapes(lib):
     # the deep configuration: three passes forward, four at most backward, closed rings last
     fwd = _passes(lib, _shape(lib, 128, 8192, 128, 4, 2), 0, 13, False)
     assert [p[2] for p in fwd][-1] == 2 and len(fwd) <= 4
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    """No fallback: if libncn_hip.so is absent the binding raises instead of computing something else."""
+    from ncn_cuda_amd import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libncn_hip.so"))
+    with pytest.raises(RuntimeError, match="no CPU or PyTorch fallback"):
+        _lib.load()
