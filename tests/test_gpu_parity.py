@@ -74,6 +74,8 @@ SHAPES = [
     (2, 256, 128, 4, 16, 3),   # Ec=32, n=16: the headline tile
     (1, 256, 128, 4, 32, 3),   # the reference script's shape family (n_cache == Ec == 32)
     (2, 64, 128, 2, 4, 4),     # Ec=64
+    (2, 128, 128, 1, 16, 3),   # Ec=128 (one head)
+    (2, 64, 256, 2, 2, 3),     # Ec=128, n=2
     (5, 40, 32, 1, 2, 3),      # Ec=32, one head, 20 groups: partial wave tile
     (2, 64, 64, 4, 16, 6),     # stride wraps to 0 again (L > log2(groups)+1)
     (2, 36, 20, 2, 3, 3),      # generic kernel: n=3, Ec=10
