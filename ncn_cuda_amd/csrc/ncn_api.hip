@@ -21,7 +21,7 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 int kernel_path(const ncn_shape* sh, int activation) {
     if (sh->n_cache < 1 || sh->n_cache > 64) return 0;
     const int64_t ec = sh->E / sh->n_head;
-    if (activation == NCN_ACT_TANH && ec <= 128 && fast_tile(sh->n_cache, (int)ec).r != 0) return 2;
+    if (ec <= 128 && fast_tile(sh->n_cache, (int)ec).r != 0) return 2;
     if (ec <= kGenericMaxHeadDim) return 1;
     return 0;
 }
@@ -84,10 +84,12 @@ Plan make_plan(const ncn_shape* sh, int activation) {
     return p;
 }
 
-void fill_step_table(StepTable& t, int n_cache, float alpha, float m) {
+void fill_step_table(StepTable& t, int n_cache, float alpha, float m, int activation = NCN_ACT_TANH) {
     const double md = m, al = alpha, k2l = 2.8853900817779268;
     t.alpha = alpha;
     t.m = m;
+    t.activation = activation;
+    t.reserved = 0;
     t.m_pow_n = (float)std::pow(md, (double)n_cache);
     t.inv_m_pow_n = (float)std::pow(md, -(double)n_cache);
     for (int k = 0; k < 64; ++k) {
@@ -114,7 +116,7 @@ void fill_common(StageArgs& a, const ncn_shape* sh, const Plan& p, int stage, fl
     a.head_dim = (int)(sh->E / sh->n_head);
     a.n_head = sh->n_head;
     a.activation = activation;
-    fill_step_table(a.tab, sh->n_cache, alpha, m);
+    fill_step_table(a.tab, sh->n_cache, alpha, m, activation);
 }
 
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
@@ -169,7 +171,7 @@ const char* ncn_error_string(int code) {
         case NCN_ERR_DTYPE: return "unknown element type (0 = float32, 1 = bfloat16)";
         case NCN_ERR_ACTIVATION: return "unknown activation code (0 tanh, 1 relu, 2 sigmoid, -1 linear)";
         case NCN_ERR_WORKSPACE: return "workspace is NULL or smaller than ncn_workspace_bytes()";
-        case NCN_ERR_UNSUPPORTED: return "unsupported shape: n_cache must be <= 64 and the head width <= 64 (128 for power-of-two n_cache <= 16 with tanh)";
+        case NCN_ERR_UNSUPPORTED: return "unsupported shape: n_cache must be <= 64 and the head width <= 64 (128 for power-of-two n_cache <= 16)";
         case NCN_ERR_ALIGN: return "a pointer is not 16-byte aligned";
         case NCN_ERR_ALIAS: return "n_stages > 1 needs float32 x_rec, xa_rec, dx, dxa to carry the state";
         default: break;

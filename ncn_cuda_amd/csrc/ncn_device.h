@@ -10,6 +10,8 @@ namespace ncn {
 // Scalars of the recurrence, made on the host in double precision and read by the kernels through scalar loads.
 struct StepTable {
     float alpha, m;
+    int32_t activation;          // activation code (only read by kernels built for more than tanh)
+    int32_t reserved;
     float m_pow_n, inv_m_pow_n;  // m^n_cache and its reciprocal
     // Per-step scalars of the reversible backward / inverse, index t = number of inversion steps already done
     // (t = 0 is the stage's last step):

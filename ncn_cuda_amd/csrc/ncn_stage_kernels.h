@@ -76,6 +76,30 @@ __device__ __forceinline__ void load_w(const float* W, int64_t E, int head, int 
     }
 }
 
+// Activation from z = 2 log2(e) T (the form the step code produces): F(T) and w = F'(T) / 4.
+//   tanh:    r = 1/(1 + 2^z), F = 1 - 2r, F'/4 = r - r^2                (ncn_fwd_cuda_kernel.cu:86-87)
+//   relu, sigmoid, linear: codes of ncn_fwd_cuda_kernel.cu:88-95 / ncn_bwd_cuda_kernel.cu:137-150
+// TANH_ONLY kernels have no branch; the others pick the activation with a wave-uniform branch on `code`.
+constexpr float kHalfLn2 = 0.34657359027997264f;  // T = z * ln(2)/2
+template <bool TANH_ONLY>
+__device__ __forceinline__ void act_Fw(float z, int code, float& Fv, float& w) {
+    if (TANH_ONLY || code == NCN_ACT_TANH) {
+        const float r = __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(z) + 1.0f);
+        Fv = fmaf(-2.0f, r, 1.0f);
+        w = fmaf(-r, r, r);
+    } else if (code == NCN_ACT_RELU) {
+        const float Tv = z * kHalfLn2;
+        Fv = fmaxf(Tv, 0.f);
+        w = Tv > 0.f ? 0.25f : 0.f;
+    } else if (code == NCN_ACT_SIGMOID) {
+        Fv = __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(-0.5f * z) + 1.0f);
+        w = 0.25f * fmaf(-Fv, Fv, Fv);
+    } else {
+        Fv = z * kHalfLn2;
+        w = 0.25f;
+    }
+}
+
 template <int F>
 __device__ __forceinline__ float dot_frag(const float (&a)[F], const float (&b)[F]) {
     float s0 = 0.f, s1 = 0.f;
@@ -96,7 +120,7 @@ __device__ __forceinline__ float dot_frag(const float (&a)[F], const float (&b)[
 // ---------------------------------------------------------------------------------------------
 // forward_core runs the n_cache steps of one stage on registers that already hold x / m^t0, xa / m^t0 with
 // t0 = step_base steps done before (several stages in a row just keep counting) and leaves them scaled.
-template <int NC, int EC, int R, int F>
+template <int NC, int EC, int R, int F, bool TANH_ONLY = true>
 __device__ __forceinline__ void forward_core(float (&x)[R][F], float (&a)[R][F], const float (&wi)[F],
                                              const float (&wj)[F], const StepTable& S, int step_base, int lane,
                                              float4* slots) {
@@ -122,8 +146,9 @@ __device__ __forceinline__ void forward_core(float (&x)[R][F], float (&a)[R][F],
 #pragma unroll
                 for (int f = 0; f < F; ++f) {
                     const float z = fmaf(c, xj[f], lam * x[rr][f]);
-                    const float r = __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(z) + 1.0f);
-                    a[rr][f] = fmaf(-2.0f * kap, r, a[rr][f] + kap);
+                    float Fv, w;
+                    act_Fw<TANH_ONLY>(z, S.activation, Fv, w);
+                    a[rr][f] = fmaf(kap, Fv, a[rr][f]);
                     x[rr][f] = fmaf(om, a[rr][f], x[rr][f]);
                 }
             }
@@ -132,10 +157,10 @@ __device__ __forceinline__ void forward_core(float (&x)[R][F], float (&a)[R][F],
 }
 
 // one stage from true values to true values
-template <int NC, int EC, int R, int F>
+template <int NC, int EC, int R, int F, bool TANH_ONLY>
 __device__ __forceinline__ void forward_steps(float (&x)[R][F], float (&a)[R][F], const float (&wi)[F],
                                               const float (&wj)[F], const StepTable& S, int lane, float4* slots) {
-    forward_core<NC, EC, R, F>(x, a, wi, wj, S, 0, lane, slots);
+    forward_core<NC, EC, R, F, TANH_ONLY>(x, a, wi, wj, S, 0, lane, slots);
     const float dn = S.m_pow_n;
 #pragma unroll
     for (int rr = 0; rr < R; ++rr)
@@ -151,7 +176,7 @@ __device__ __forceinline__ void forward_steps(float (&x)[R][F], float (&a)[R][F]
 //   x = (y - (1-m) b)/m       recompute r from x        a = (b - (1-m) F)/m
 // with the same m^t scaling of the registers as the backward below (Y = m^t x, B = m^t xa).
 // ---------------------------------------------------------------------------------------------
-template <int NC, int EC, int R, int F>
+template <int NC, int EC, int R, int F, bool TANH_ONLY>
 __device__ __forceinline__ void inverse_steps(float (&y)[R][F], float (&b)[R][F], const float (&wi)[F],
                                               const float (&wj)[F], const StepTable& S, int lane, float4* slots) {
     using T = Tile<NC, EC, R, F>;
@@ -176,8 +201,9 @@ __device__ __forceinline__ void inverse_steps(float (&y)[R][F], float (&b)[R][F]
 #pragma unroll
                 for (int f = 0; f < F; ++f) {
                     const float z = fmaf(c, xj[f], lam * y[rr][f]);
-                    const float r = __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(z) + 1.0f);
-                    b[rr][f] = fmaf(2.0f * kap, r, b[rr][f] - kap);
+                    float Fv, w;
+                    act_Fw<TANH_ONLY>(z, S.activation, Fv, w);
+                    b[rr][f] = fmaf(-kap, Fv, b[rr][f]);
                 }
             }
         }
@@ -214,7 +240,7 @@ __device__ __forceinline__ void inverse_steps(float (&y)[R][F], float (&b)[R][F]
 // ---------------------------------------------------------------------------------------------
 // backward_core: the n_cache steps of one stage on registers in the scaled form above with t0 = step_base
 // inversion steps done before (P holds p / m^t0, not h); leaves them scaled by t0 + n_cache steps.
-template <int NC, int EC, int R, int F, bool MASKED>
+template <int NC, int EC, int R, int F, bool MASKED, bool TANH_ONLY = true>
 __device__ __forceinline__ void backward_core(float (&Y)[R][F], float (&B)[R][F], float (&G)[R][F], float (&P)[R][F],
                                               const float (&wi)[F], const float (&wj)[F], float (&dwi)[F],
                                               float (&dwj)[F], float own, const StepTable& S, int step_base, int lane,
@@ -253,9 +279,10 @@ __device__ __forceinline__ void backward_core(float (&Y)[R][F], float (&B)[R][F]
 #pragma unroll
                 for (int f = 0; f < F; ++f) {
                     const float z = fmaf(chat, xj[f], lam * Y[rr][f]);
-                    const float r = __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(z) + 1.0f);
-                    B[rr][f] = fmaf(2.0f * kap, r, B[rr][f] - kap);   // m^(t+1) xa of this step
-                    u[f] = P[rr][f] * fmaf(-r, r, r);
+                    float Fv, w;
+                    act_Fw<TANH_ONLY>(z, S.activation, Fv, w);
+                    B[rr][f] = fmaf(-kap, Fv, B[rr][f]);   // m^(t+1) xa of this step
+                    u[f] = P[rr][f] * w;
                     rh = fmaf(u[f], xj[f], rh);
                 }
                 rh = lane_sum<1, T::LF>(rh);
@@ -285,7 +312,7 @@ __device__ __forceinline__ void backward_core(float (&Y)[R][F], float (&B)[R][F]
 }
 
 // one stage: G, H true gradients in and out; Y, B true outputs in, m^n_cache times the stage inputs out
-template <int NC, int EC, int R, int F, bool MASKED>
+template <int NC, int EC, int R, int F, bool MASKED, bool TANH_ONLY>
 __device__ __forceinline__ void backward_steps(float (&Y)[R][F], float (&B)[R][F], float (&G)[R][F], float (&P)[R][F],
                                                const float (&wi)[F], const float (&wj)[F], float (&dwi)[F],
                                                float (&dwj)[F], float own, const StepTable& S, int lane,
@@ -296,7 +323,7 @@ __device__ __forceinline__ void backward_steps(float (&Y)[R][F], float (&B)[R][F
     for (int rr = 0; rr < R; ++rr)
 #pragma unroll
         for (int f = 0; f < F; ++f) P[rr][f] = fmaf(om, G[rr][f], P[rr][f]);  // h -> p
-    backward_core<NC, EC, R, F, MASKED>(Y, B, G, P, wi, wj, dwi, dwj, own, S, 0, lane, slots);
+    backward_core<NC, EC, R, F, MASKED, TANH_ONLY>(Y, B, G, P, wi, wj, dwi, dwj, own, S, 0, lane, slots);
     // undo the scaling of the gradients: NC steps done
     const float dn = S.m_pow_n;       // m^NC
 #pragma unroll
@@ -325,8 +352,8 @@ __device__ __forceinline__ void backward_steps(float (&Y)[R][F], float (&B)[R][F
     float wi[F], wj[F];                                                                         \
     load_w<F>(A.W, A.E, head, EC, fl, wi, wj);
 
-template <int NC, int EC, int R, int F, int WPE = 1>
-__global__ void __launch_bounds__(kBlockThreads, WPE) stage_forward_kernel(const StageArgs A) {
+template <int NC, int EC, int R, int F, bool TANH_ONLY = true>
+__global__ void __launch_bounds__(kBlockThreads) stage_forward_kernel(const StageArgs A) {
     NCN_WAVE_PROLOGUE
     for (uint32_t t = gwave / A.n_head; t < A.total_tiles; t += tile_step) {
         int64_t off[R];
@@ -337,7 +364,7 @@ __global__ void __launch_bounds__(kBlockThreads, WPE) stage_forward_kernel(const
             load_frag<F>(A.in0, A.in_dtype, off[rr], valid, x[rr]);
             load_frag<F>(A.in1, A.in_dtype, off[rr], valid, a[rr]);
         }
-        forward_steps<NC, EC, R, F>(x, a, wi, wj, A.tab, lane, slots);
+        forward_steps<NC, EC, R, F, TANH_ONLY>(x, a, wi, wj, A.tab, lane, slots);
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) {
             store_frag<F>(A.out0, A.out_dtype, off[rr], valid, x[rr]);
@@ -350,8 +377,8 @@ __global__ void __launch_bounds__(kBlockThreads, WPE) stage_forward_kernel(const
     }
 }
 
-template <int NC, int EC, int R, int F, int WPE = 1>
-__global__ void __launch_bounds__(kBlockThreads, WPE) stage_inverse_kernel(const StageArgs A) {
+template <int NC, int EC, int R, int F, bool TANH_ONLY = true>
+__global__ void __launch_bounds__(kBlockThreads) stage_inverse_kernel(const StageArgs A) {
     NCN_WAVE_PROLOGUE
     for (uint32_t t = gwave / A.n_head; t < A.total_tiles; t += tile_step) {
         int64_t off[R];
@@ -362,7 +389,7 @@ __global__ void __launch_bounds__(kBlockThreads, WPE) stage_inverse_kernel(const
             load_frag<F>(A.in0, A.in_dtype, off[rr], valid, y[rr]);
             load_frag<F>(A.in1, A.in_dtype, off[rr], valid, b[rr]);
         }
-        inverse_steps<NC, EC, R, F>(y, b, wi, wj, A.tab, lane, slots);
+        inverse_steps<NC, EC, R, F, TANH_ONLY>(y, b, wi, wj, A.tab, lane, slots);
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) {
             store_frag<F>(A.out0, A.out_dtype, off[rr], valid, y[rr]);
@@ -371,8 +398,8 @@ __global__ void __launch_bounds__(kBlockThreads, WPE) stage_inverse_kernel(const
     }
 }
 
-template <int NC, int EC, int R, int F, int WPE = 1>
-__global__ void __launch_bounds__(kBlockThreads, WPE) stage_backward_kernel(const StageArgs A) {
+template <int NC, int EC, int R, int F, bool TANH_ONLY = true>
+__global__ void __launch_bounds__(kBlockThreads) stage_backward_kernel(const StageArgs A) {
     NCN_WAVE_PROLOGUE
     float dwi[F], dwj[F];
 #pragma unroll
@@ -389,7 +416,7 @@ __global__ void __launch_bounds__(kBlockThreads, WPE) stage_backward_kernel(cons
             load_frag<F>(A.g0, A.g_dtype, off[rr], valid, G[rr]);
             load_frag<F>(A.g1, A.g_dtype, off[rr], valid && A.g1 != nullptr, H[rr]);
         }
-        backward_steps<NC, EC, R, F, false>(Y, B, G, H, wi, wj, dwi, dwj, 1.0f, A.tab, lane, slots);
+        backward_steps<NC, EC, R, F, false, TANH_ONLY>(Y, B, G, H, wi, wj, dwi, dwj, 1.0f, A.tab, lane, slots);
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) {
             store_frag<F>(A.out0, A.out_dtype, off[rr], valid, G[rr]);

@@ -152,10 +152,13 @@ def test_dya_none_equals_zeros(M):
         assert torch.equal(u, v)
 
 
+@pytest.mark.parametrize("shape", [(2, 32, 16, 2, 4, 3), (2, 128, 128, 4, 16, 2), (2, 36, 20, 2, 3, 3)],
+                         ids=["register_n4_Ec8", "register_n16_Ec32", "generic_n3_Ec10"])
 @pytest.mark.parametrize("act", [1, 2, -1], ids=["relu", "sigmoid", "linear"])
-def test_other_activations_vs_oracle(M, act):
-    """relu / sigmoid / linear run on the generic kernel; the oracle for them is pinned by autograd only."""
-    batch, N, E, C, n, L = 2, 32, 16, 2, 4, 3
+def test_other_activations_vs_oracle(M, act, shape):
+    """relu / sigmoid / linear (codes of ncn_fwd_cuda_kernel.cu:86-95) on the register kernels and on the generic
+    kernel; the oracle for them is pinned by autograd only."""
+    batch, N, E, C, n, L = shape
     alpha = 0.9
     x, xa, Ws, dyi, dya = O.make_inputs(batch, N, E, L, n, seed=21, xa_zero=False)
     d = torch.float64
@@ -166,6 +169,9 @@ def test_other_activations_vs_oracle(M, act):
     outs = _stack_forward(M, gx, gxa, gWs, alpha, n, C, act)
     assert O.rel_err(outs[-1][0], ref_yi) < TOL_F32
     assert O.rel_err(outs[-1][1], ref_ya) < TOL_F32
+    ix, ixa = M.inverse(outs[-1][0], outs[-1][1], gWs[-1], alpha, act, n, C, L - 1)
+    prev = outs[-2]
+    assert O.rel_err(ix, prev[0]) < 3e-5 and O.rel_err(ixa, prev[1]) < 3e-5
     if act == 1:
         return  # relu's kink makes the reversible recomputation flip F' for |T| ~ eps: gradients not compared
     _, _, dx, dxa, dWs = _stack_backward(M, outs, gdyi, gdya, gWs, alpha, n, C, act)

@@ -56,7 +56,7 @@ def test_check_shape_codes(lib):
     assert h.ncn_check_shape(ctypes.byref(ok), 0, 1, 7) == -4                             # activation
     assert h.ncn_check_shape(ctypes.byref(_shape(lib, 1, 256, 32, 4, 128)), 0, 1, 0) == -6  # n_cache > 64
     assert h.ncn_check_shape(ctypes.byref(_shape(lib, 1, 64, 512, 4, 4)), 0, 1, 0) == 0     # head width 128: register kernel
-    assert h.ncn_check_shape(ctypes.byref(_shape(lib, 1, 64, 512, 4, 4)), 0, 1, 1) == -6    # .. but not with relu
+    assert h.ncn_check_shape(ctypes.byref(_shape(lib, 1, 64, 512, 4, 4)), 0, 1, 1) == 0     # .. with relu too
     assert h.ncn_check_shape(ctypes.byref(_shape(lib, 1, 64, 1024, 4, 4)), 0, 1, 0) == -6   # head width 256
     for code in (0, -1, -2, -3, -4, -5, -6, -7, -8):
         assert len(h.ncn_error_string(code)) > 0
