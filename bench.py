@@ -150,7 +150,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32" if not bf16 else "f32 arithmetic, bf16 storage",
+        "dtype": "f32",  # arithmetic type; storage is named in config.workload
         "data": "synthetic",
         "config": {"workload": f"{args.config}: B={tokens} D={N} g={n} -> x[batch={batch},N={N},E={E}], "
                                f"{C} heads of {E // C}, n_cache={n}, {L} stages, alpha=0.9, m=0.9, tanh, "
