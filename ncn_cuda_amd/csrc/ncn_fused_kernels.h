@@ -46,7 +46,7 @@ struct FusedArgs {
     float* dw_partials;  // backward: [gridDim.x / n_head][n_stages][2E]
     int64_t N, E;
     int32_t n_head, n_stages;
-    int32_t in_dtype, g_dtype, out_dtype, aux_dtype_unused;
+    int32_t in_dtype, g_dtype, out_dtype, reserved;
     uint32_t class_stride;    // S0, in blocks
     uint32_t ring;            // sub-blocks per class = groups / S0 (power of two)
     uint32_t window;          // sub-blocks held in LDS
@@ -136,20 +136,6 @@ __device__ __forceinline__ void fused_load_rows(const FusedArgs& A, const FusedI
         if (src) load_frag<4>(src, dtype, fused_row_offset<NC>(A, it, lr) + c4 * 4, true, v);
         else v[0] = v[1] = v[2] = v[3] = 0.f;
         lds_store_frag<4>(dst + lr * EC + c4 * 4, v);
-    }
-}
-
-// LDS -> global for the owned rows
-template <int NC, int EC, int NW>
-__device__ __forceinline__ void fused_store_rows(const FusedArgs& A, const FusedItem& it, const float* src, void* dst,
-                                                 int dtype) {
-    constexpr uint32_t CPR = EC / 4;
-    const uint32_t r0 = it.own_lo * NC, rows = it.own_cnt * NC;
-    for (uint32_t c = threadIdx.x; c < rows * CPR; c += 64 * NW) {
-        const uint32_t lr = r0 + c / CPR, c4 = c % CPR;
-        float v[4];
-        lds_load_frag<4>(src + lr * EC + c4 * 4, v);
-        store_frag<4>(dst, dtype, fused_row_offset<NC>(A, it, lr) + c4 * 4, true, v);
     }
 }
 

@@ -210,3 +210,20 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libncn_hip.so"))
     with pytest.raises(RuntimeError, match="no CPU or PyTorch fallback"):
         _lib.load()
+
+
+def test_header_is_valid_c(tmp_path):
+    """include/ncn_hip.h is a C header: a C translation unit that only includes it and takes the address of every
+    entry point must compile with gcc -std=c99 -Wall -Werror."""
+    import shutil
+    import subprocess
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc")
+    src = tmp_path / "use_header.c"
+    names = _declared_functions()
+    body = "\n".join(f"    p[{k}] = (void*)&{n};" for k, n in enumerate(names))
+    src.write_text(f'#include "ncn_hip.h"\nvoid* p[{len(names)}];\nvoid take(void) {{\n{body}\n}}\n'
+                   "int size_ok[sizeof(ncn_shape) == 32 ? 1 : -1];\n")
+    subprocess.run([gcc, "-std=c99", "-Wall", "-Werror", "-Wno-pedantic", "-I", os.path.join(ROOT, "include"), "-c",
+                    str(src), "-o", str(tmp_path / "use_header.o")], check=True)
