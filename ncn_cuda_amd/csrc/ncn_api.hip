@@ -52,7 +52,8 @@ struct Plan {
     int path;
     int groups_per_tile;
     uint32_t groups, tiles_per_inst, total_tiles;
-    int grid_x;
+    int grid_x;        // backward launch
+    int grid_fwd;      // forward / inverse launch
     int partial_rows;  // rows of the dW partial buffer the backward launch writes
 };
 
@@ -73,12 +74,20 @@ Plan make_plan(const ncn_shape* sh, int activation) {
         const int64_t cap = (int64_t)kMaxGridX * C / 4 / quantum * quantum;  // rows = blocks * 4 / C <= kMaxGridX
         int64_t blocks = ((int64_t)p.total_tiles * C + 3) / 4;
         blocks = (blocks + quantum - 1) / quantum * quantum;
+        // forward / inverse write no partials: one wave tile per wave where possible (measured 8 % faster than a
+        // persistent loop over 4096 blocks: retiring blocks balance the load)
+        int64_t fblocks = blocks;
+        const int64_t fcap = (int64_t)kMaxForwardGridX / quantum * quantum;
+        if (fblocks > fcap) fblocks = fcap;
+        if (fblocks < quantum) fblocks = quantum;
+        p.grid_fwd = (int)fblocks;
         if (blocks > cap) blocks = cap;
         if (blocks < quantum) blocks = quantum;
         p.grid_x = (int)blocks;
         p.partial_rows = (int)(blocks * 4 / C);
     } else {
         p.grid_x = (int)(p.total_tiles < (uint32_t)kMaxGridX ? p.total_tiles : (uint32_t)kMaxGridX);
+        p.grid_fwd = p.grid_x;
         p.partial_rows = p.grid_x;
     }
     return p;
@@ -248,7 +257,7 @@ int ncn_forward(const void* x, const void* xa, int in_dtype, void* y, void* ya, 
                 a.out0 = d0; a.out1 = d1; a.out_dtype = d_dtype;
                 a.aux0 = last ? y32 : nullptr; a.aux1 = last ? ya32 : nullptr;
                 a.W = W + ps.first * wstride;
-                err = launch_fast_forward(kForward, a, shape->n_head, p.grid_x, s);
+                err = launch_fast_forward(kForward, a, shape->n_head, p.grid_fwd, s);
             } else {
                 FusedArgs a{};
                 a.in0 = cur0; a.in1 = cur1; a.in_dtype = cur_dtype;
@@ -277,8 +286,8 @@ int ncn_forward(const void* x, const void* xa, int in_dtype, void* y, void* ya, 
         a.aux0 = last ? y32 : nullptr;
         a.aux1 = last ? ya32 : nullptr;
         a.W = W + k * wstride;
-        hipError_t err = (p.path == 2) ? launch_fast_forward(kForward, a, shape->n_head, p.grid_x, s)
-                                       : launch_generic(kForward, a, shape->n_head, p.grid_x, s);
+        hipError_t err = (p.path == 2) ? launch_fast_forward(kForward, a, shape->n_head, p.grid_fwd, s)
+                                       : launch_generic(kForward, a, shape->n_head, p.grid_fwd, s);
         if (err != hipSuccess) return (int)err;
     }
     return NCN_OK;
@@ -305,8 +314,8 @@ int ncn_inverse(const void* y, const void* ya, int in_dtype, void* x, void* xa, 
         a.out1 = xa;
         a.out_dtype = out_dtype;
         a.W = W + (int64_t)k * 2 * shape->E;
-        hipError_t err = (p.path == 2) ? launch_fast_forward(kInverse, a, shape->n_head, p.grid_x, s)
-                                       : launch_generic(kInverse, a, shape->n_head, p.grid_x, s);
+        hipError_t err = (p.path == 2) ? launch_fast_forward(kInverse, a, shape->n_head, p.grid_fwd, s)
+                                       : launch_generic(kInverse, a, shape->n_head, p.grid_fwd, s);
         if (err != hipSuccess) return (int)err;
     }
     return NCN_OK;

@@ -36,6 +36,8 @@ constexpr int kGenericArrays = 7;
 
 // Upper bound on gridDim.x of a stage launch == rows of the dW partial buffer.
 constexpr int kMaxGridX = 4096;
+// Upper bound on gridDim.x of a forward / inverse launch (no partial rows to pay for).
+constexpr int kMaxForwardGridX = 1 << 18;
 // dW partial rows are summed in two levels: chunks of kReduceRowsPerBlock rows, then the chunk sums.
 constexpr int kReduceRowsPerBlock = 32;
 constexpr int kReduceLevel1Rows = kMaxGridX / kReduceRowsPerBlock;
