@@ -389,7 +389,7 @@ int ncn_backward(const void* y, const void* ya, int y_dtype, const void* dy, con
                 fill_step_table(a.tab, shape->n_cache, alpha, m);
                 err = launch_fused(true, a, shape, ps, s);
                 if (err != hipSuccess) return (int)err;
-                const int rows = fused_grid(shape, ps) / shape->n_head;
+                const int rows = fused_grid(shape, ps, true) / shape->n_head;
                 for (int k = 0; k < ps.count && err == hipSuccess; ++k)
                     err = launch_reduce_dw(partials + k * wstride, rows, (int64_t)ps.count * wstride, wstride, level1,
                                            dW + (ps.first + k) * wstride, s);

@@ -15,7 +15,8 @@ namespace {
     X(2, 16) X(4, 16) X(2, 32) X(4, 32)
 
 constexpr size_t kFusedStateBytes = 64 * 1024;  // LDS for the row arrays of one workgroup (2 forward, 4 backward)
-constexpr int kFusedMaxGrid = 512;              // two workgroups per CU
+constexpr int kFusedMaxGridFwd = 16384;          // forward: no partial rows to pay for, let retiring workgroups balance
+constexpr int kFusedMaxGridBwd = 2048;           // backward: one dW partial row per n_head workgroups and stage
 
 size_t fused_lds_bytes(int nc, int ec, bool backward, uint32_t window, int n_stages) {
     const TileShape t = fast_tile(nc, ec);
@@ -155,9 +156,14 @@ static hipError_t launch_fused_t(bool backward, const FusedArgs& a, int grid, si
     return hipGetLastError();
 }
 
-int fused_grid(const ncn_shape* sh, const FusedPass& p) {
+int fused_grid(const ncn_shape* sh, const FusedPass& p, bool backward) {
     const int64_t items = sh->batch * (int64_t)p.class_groups * p.tiles_per_ring * sh->n_head;
-    int64_t g = items < kFusedMaxGrid ? items : kFusedMaxGrid;
+    int64_t cap = backward ? kFusedMaxGridBwd : kFusedMaxGridFwd;
+    if (backward) {  // partial rows (grid / n_head) * stages must fit the kMaxGridX rows of the dW scratch
+        const int64_t by_rows = (int64_t)kMaxGridX / p.count * sh->n_head;
+        if (by_rows < cap) cap = by_rows;
+    }
+    int64_t g = items < cap ? items : cap;
     g = g / sh->n_head * sh->n_head;
     if (g < sh->n_head) g = sh->n_head;
     return (int)g;
@@ -181,7 +187,7 @@ hipError_t launch_fused(bool backward, FusedArgs& a, const ncn_shape* sh, const 
     for (int k = 0; k < kFusedMaxStages; ++k) a.sub_stride[k] = k < p.count ? p.sub_stride[k] : 0;
     a.scale_dn = (float)std::pow((double)a.tab.m, (double)(nc * p.count));
     a.scale_up = (float)std::pow((double)a.tab.m, -(double)(nc * p.count));
-    const int grid = fused_grid(sh, p);
+    const int grid = fused_grid(sh, p, backward);
     const size_t lds = fused_lds_bytes(nc, ec, backward, p.window, p.count);
 #define NCN_CASE(NC, EC) \
     if (nc == NC && ec == EC) return launch_fused_t<NC, EC>(backward, a, grid, lds, s);

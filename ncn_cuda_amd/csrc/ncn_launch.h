@@ -59,7 +59,7 @@ struct FusedPass {
 };
 bool fused_supported(const ncn_shape* sh, int activation);
 std::vector<FusedPass> plan_fused(const ncn_shape* sh, int first, int count, bool backward);
-int fused_grid(const ncn_shape* sh, const FusedPass& p);
+int fused_grid(const ncn_shape* sh, const FusedPass& p, bool backward);
 hipError_t launch_fused(bool backward, FusedArgs& a, const ncn_shape* sh, const FusedPass& p, hipStream_t s);
 
 }  // namespace ncn
