@@ -41,10 +41,13 @@ extern "C" {
 
 /* activation codes: those of the reference's CUDA surface (ncn_pytorch_wrapper_v2.py:111,
  * ncn_fwd_cuda_kernel.cu:86-95): 0 tanh, 1 relu, 2 sigmoid, anything else the reference treats as
- * linear; here only -1 is accepted for linear. */
+ * linear; here only -1 is accepted for linear.  Code 3 is the leaky relu of the reference's Triton kernels
+ * (ncn_triton/ncn_triton.py:22-28, 101-102: slope 0.01 below zero, value and slope of the upper branch at 0),
+ * which the CUDA surface does not have. */
 #define NCN_ACT_TANH 0
 #define NCN_ACT_RELU 1
 #define NCN_ACT_SIGMOID 2
+#define NCN_ACT_LEAKY_RELU 3
 #define NCN_ACT_LINEAR (-1)
 
 /* error codes (negative: rejected before any GPU work; positive: a hipError_t from the runtime) */

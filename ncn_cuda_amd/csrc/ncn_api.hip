@@ -12,7 +12,7 @@ namespace {
 using namespace ncn;
 
 bool known_activation(int a) {
-    return a == NCN_ACT_TANH || a == NCN_ACT_RELU || a == NCN_ACT_SIGMOID || a == NCN_ACT_LINEAR;
+    return a == NCN_ACT_TANH || a == NCN_ACT_RELU || a == NCN_ACT_SIGMOID || a == NCN_ACT_LEAKY_RELU || a == NCN_ACT_LINEAR;
 }
 bool known_dtype(int d) { return d == NCN_F32 || d == NCN_BF16; }
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -178,7 +178,7 @@ const char* ncn_error_string(int code) {
         case NCN_ERR_NULL: return "a required pointer is NULL";
         case NCN_ERR_SHAPE: return "bad shape: sizes must be positive, N % n_cache == 0, E % n_head == 0, n_stages >= 1";
         case NCN_ERR_DTYPE: return "unknown element type (0 = float32, 1 = bfloat16)";
-        case NCN_ERR_ACTIVATION: return "unknown activation code (0 tanh, 1 relu, 2 sigmoid, -1 linear)";
+        case NCN_ERR_ACTIVATION: return "unknown activation code (0 tanh, 1 relu, 2 sigmoid, 3 leaky relu, -1 linear)";
         case NCN_ERR_WORKSPACE: return "workspace is NULL or smaller than ncn_workspace_bytes()";
         case NCN_ERR_UNSUPPORTED: return "unsupported shape: n_cache must be <= 64 and the head width <= 64 (128 for power-of-two n_cache <= 16)";
         case NCN_ERR_ALIGN: return "a pointer is not 16-byte aligned";

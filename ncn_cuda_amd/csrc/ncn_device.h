@@ -220,6 +220,9 @@ __device__ __forceinline__ void act_fd(int code, float T, float& F, float& dF) {
         const float t = __builtin_amdgcn_exp2f(-T * 1.4426950408889634f);
         F = __builtin_amdgcn_rcpf(1.0f + t);
         dF = F * (1.0f - F);
+    } else if (code == NCN_ACT_LEAKY_RELU) {
+        F = T >= 0.f ? T : 0.01f * T;
+        dF = T >= 0.f ? 1.f : 0.01f;
     } else {
         F = T;
         dF = 1.f;

@@ -94,6 +94,10 @@ __device__ __forceinline__ void act_Fw(float z, int code, float& Fv, float& w) {
     } else if (code == NCN_ACT_SIGMOID) {
         Fv = __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(-0.5f * z) + 1.0f);
         w = 0.25f * fmaf(-Fv, Fv, Fv);
+    } else if (code == NCN_ACT_LEAKY_RELU) {
+        const float Tv = z * kHalfLn2;
+        Fv = Tv >= 0.f ? Tv : 0.01f * Tv;
+        w = Tv >= 0.f ? 0.25f : 0.0025f;
     } else {
         Fv = z * kHalfLn2;
         w = 0.25f;

@@ -22,7 +22,8 @@ from . import ncn_cuda_module
 __all__ = ["ACTIVATION_CODES", "NCNFunction", "NCNNetFunction", "NCNModuleCuda", "NCNNetCuda", "NCNNetTestCuda",
            "default_save_every", "fused_ncn_cuda_v2", "fused_ncn_net", "ncn_inverse"]
 
-ACTIVATION_CODES = {"tanh": 0, "relu": 1, "sigmoid": 2, "linear": -1}  # ncn_pytorch_wrapper_v2.py:111
+# names and codes of ncn_pytorch_wrapper_v2.py:111, plus the leaky relu of the Triton kernels (ncn_triton.py:101)
+ACTIVATION_CODES = {"tanh": 0, "relu": 1, "sigmoid": 2, "linear": -1, "leaky-relu": 3}
 
 
 class NCNFunction(torch.autograd.Function):

@@ -25,7 +25,7 @@ from . import _lib
 M_DEFAULT = 0.9  # hard-coded by the reference: ncn_fwd_cuda_kernel.cu:72, ncn_pytorch.py:89
 
 _DTYPES = {torch.float32: _lib.NCN_F32, torch.bfloat16: _lib.NCN_BF16}
-_ACT_CODES = (_lib.ACT_TANH, _lib.ACT_RELU, _lib.ACT_SIGMOID, _lib.ACT_LINEAR)
+_ACT_CODES = (_lib.ACT_TANH, _lib.ACT_RELU, _lib.ACT_SIGMOID, _lib.ACT_LEAKY_RELU, _lib.ACT_LINEAR)
 
 
 def validate(x, xa, W, n_cache, n_head, activation, module_l=0, n_stages=1, what="x"):
@@ -53,7 +53,7 @@ def validate(x, xa, W, n_cache, n_head, activation, module_l=0, n_stages=1, what
     if W.numel() != n_stages * 2 * E:
         raise ValueError(f"W must hold {n_stages} x 2E = {n_stages * 2 * E} values, got {W.numel()}")
     if int(activation) not in _ACT_CODES:
-        raise ValueError(f"unknown activation code {activation} (0 tanh, 1 relu, 2 sigmoid, -1 linear)")
+        raise ValueError(f"unknown activation code {activation} (0 tanh, 1 relu, 2 sigmoid, 3 leaky relu, -1 linear)")
     shape = _lib.NcnShape(batch, N, E, n_head, n_cache)
     rc = _lib.load().ncn_check_shape(ctypes.byref(shape), module_l, n_stages, int(activation))
     if rc != 0:

@@ -19,8 +19,9 @@ vectors that tests/golden/make_golden.py wrote from the reference's own CPU code
 backward additionally against autograd through stage_forward in float64, the inverse against
 forward round trips, the index map against the bijection/hand values.  No function here is
 "parity unpinned" for activation == tanh.  The relu / sigmoid / linear activations exist only in the
-reference's CUDA kernels (ncn_fwd_cuda_kernel.cu:86-95), which cannot be built here; for them the
-oracle is pinned only by autograd-vs-closed-form and special cases: parity unpinned.
+reference's CUDA kernels (ncn_fwd_cuda_kernel.cu:86-95) and leaky relu only in its Triton kernels
+(ncn_triton/ncn_triton.py:22-28), none of which can be built or run here; for them the oracle is
+pinned only by autograd-vs-closed-form and special cases: parity unpinned.
 """
 import math
 
@@ -30,11 +31,13 @@ M_DEFAULT = 0.9  # hard-coded in the reference: ncn_pytorch.py:89, ncn_fwd_cuda_
 
 # activation codes of the reference's CUDA surface (ncn_pytorch_wrapper_v2.py:111)
 ACT_TANH, ACT_RELU, ACT_SIGMOID, ACT_LINEAR = 0, 1, 2, -1
+ACT_LEAKY_RELU = 3  # not a CUDA code: the leaky relu of ncn_triton/ncn_triton.py:22-28 (slope 0.01)
 
 
 def act_code(activation):
     if isinstance(activation, str):
-        return {"tanh": ACT_TANH, "relu": ACT_RELU, "sigmoid": ACT_SIGMOID, "linear": ACT_LINEAR}[activation]
+        return {"tanh": ACT_TANH, "relu": ACT_RELU, "sigmoid": ACT_SIGMOID, "linear": ACT_LINEAR,
+                "leaky-relu": ACT_LEAKY_RELU}[activation]
     return int(activation)
 
 
@@ -49,6 +52,9 @@ def _act(T, code):
     if code == ACT_SIGMOID:
         F = torch.sigmoid(T)
         return F, F * (1.0 - F)
+    if code == ACT_LEAKY_RELU:  # ncn_triton.py:22-28: x >= 0 keeps x and slope 1
+        pos = T >= 0
+        return torch.where(pos, T, 0.01 * T), torch.where(pos, torch.ones_like(T), torch.full_like(T, 0.01))
     return T, torch.ones_like(T)
 
 

@@ -154,10 +154,10 @@ def test_dya_none_equals_zeros(M):
 
 @pytest.mark.parametrize("shape", [(2, 32, 16, 2, 4, 3), (2, 128, 128, 4, 16, 2), (2, 36, 20, 2, 3, 3)],
                          ids=["register_n4_Ec8", "register_n16_Ec32", "generic_n3_Ec10"])
-@pytest.mark.parametrize("act", [1, 2, -1], ids=["relu", "sigmoid", "linear"])
+@pytest.mark.parametrize("act", [1, 2, -1, 3], ids=["relu", "sigmoid", "linear", "leaky_relu"])
 def test_other_activations_vs_oracle(M, act, shape):
-    """relu / sigmoid / linear (codes of ncn_fwd_cuda_kernel.cu:86-95) on the register kernels and on the generic
-    kernel; the oracle for them is pinned by autograd only."""
+    """relu / sigmoid / linear (codes of ncn_fwd_cuda_kernel.cu:86-95) and the Triton kernels' leaky relu
+    (ncn_triton.py:22-28) on the register kernels and on the generic kernel; the oracle for them is pinned by autograd only."""
     batch, N, E, C, n, L = shape
     alpha = 0.9
     x, xa, Ws, dyi, dya = O.make_inputs(batch, N, E, L, n, seed=21, xa_zero=False)

@@ -140,7 +140,9 @@ def test_surface_matches_reference_names():
     net = pkg.NCNNetCuda(0.9, "tanh", 4, 2, 3, 16)
     assert sorted(net.state_dict()) == ["ncn_modules.0.weight", "ncn_modules.1.weight", "ncn_modules.2.weight"]
     assert net.ncn_modules[1].weight.shape == (32,)
-    assert pkg.ACTIVATION_CODES == {"tanh": 0, "relu": 1, "sigmoid": 2, "linear": -1}
+    reference_map = {"tanh": 0, "relu": 1, "sigmoid": 2, "linear": -1}  # ncn_pytorch_wrapper_v2.py:111
+    assert {k: pkg.ACTIVATION_CODES[k] for k in reference_map} == reference_map
+    assert pkg.ACTIVATION_CODES["leaky-relu"] == 3 and len(pkg.ACTIVATION_CODES) == 5
 
 
 def test_product_code_never_imports_the_oracle():

@@ -104,7 +104,27 @@ def test_pivot_row_uses_pre_step_value_and_step_order():
     assert torch.allclose(ya.reshape(-1), torch.tensor(a, dtype=D), atol=1e-15)
 
 
-@pytest.mark.parametrize("act", ["tanh", "sigmoid", "linear"])
+def test_leaky_relu_by_hand():
+    """One row, one step (n = 1): a negative T is scaled by 0.01 and a positive one kept, as in
+    ncn_triton/ncn_triton.py:22-28; the slope seen by autograd is 0.01 / 1."""
+    alpha, m = 0.5, 0.9
+    x = torch.tensor([[[-1.0, 2.0]]], dtype=D, requires_grad=True)
+    xa = torch.zeros(1, 1, 2, dtype=D)
+    W = torch.tensor([0.3, 0.1, -0.2, 0.05], dtype=D)       # Wi = (0.3, 0.1), Wj = (-0.2, 0.05)
+    y, ya = O.stage_forward(x, xa, W, alpha, 1, 1, 0, m, activation="leaky-relu")
+    s = -1.0 * (0.3 - 0.2) + 2.0 * (0.1 + 0.05)             # the row is its own pivot
+    T = [alpha * v + (1 - alpha) * s * v for v in (-1.0, 2.0)]
+    assert T[0] < 0 < T[1]
+    F = [0.01 * T[0], T[1]]
+    a = [(1 - m) * f for f in F]
+    r = [m * v + (1 - m) * a_ for v, a_ in zip((-1.0, 2.0), a)]
+    assert torch.allclose(ya.reshape(-1), torch.tensor(a, dtype=D), atol=1e-15)
+    assert torch.allclose(y.reshape(-1), torch.tensor(r, dtype=D), atol=1e-15)
+    F2, dF = O._act(torch.tensor([-3.0, 0.0, 4.0], dtype=D), O.ACT_LEAKY_RELU)
+    assert F2.tolist() == [-0.03, 0.0, 4.0] and dF.tolist() == [0.01, 1.0, 1.0]
+
+
+@pytest.mark.parametrize("act", ["tanh", "sigmoid", "linear", "leaky-relu"])
 def test_closed_form_backward_equals_autograd(act):
     batch, N, E, C, n, L, alpha = 2, 24, 6, 2, 4, 4, 0.8
     x, xa = _rand(batch, N, E, seed=12), _rand(batch, N, E, seed=13)
