@@ -132,6 +132,20 @@ def main():
     ms_per_step = (t1 - t0) * 1e3 / args.steps
     value = tokens / (ms_per_step * 1e-3)
 
+    # what a plain device-to-device copy reaches on this GPU (reads 1 GiB and writes 1 GiB per copy): quoted beside
+    # the published 8 TB/s peak, outside the timed region
+    src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+    dst = torch.empty_like(src)
+    dst.copy_(src)
+    c0, c1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    c0.record()
+    for _ in range(5):
+        dst.copy_(src)
+    c1.record()
+    torch.cuda.synchronize()
+    copy_gbps = 5 * 2.0 * src.numel() * 4 / (c0.elapsed_time(c1) * 1e-3) / 1e9
+    del src, dst
+
     # dominant kernel: backward stage launch (its event bracket also holds the microsecond-scale dW reduce)
     # (with multi-stage segments the bracket holds a whole segment: per-stage figures are the segment's / its stages)
     bwd_ms = sum(e0.elapsed_time(e1) for e0, e1, _ in events) / sum(cnt for _, _, cnt in events)
@@ -160,6 +174,7 @@ def main():
                      "kernel": (f"stage_backward_kernel<{n},{E // C}>" if save_every == 1 else
                                 f"backward of {save_every}-stage segments (multi-stage passes), per stage"),
                      "avg_launch_ms": bwd_ms,
+                     "attainable_copy_GBps": copy_gbps, "frac_of_attainable_copy": achieved / copy_gbps,
                      "algorithmic_bytes_per_launch": bytes_bwd_launch},
         "stack": {"algorithmic_bytes_fused": 10.0 * P * sbytes,
                   "achieved_GBps_fused_bytes": 10.0 * P * sbytes / (ms_per_step * 1e-3) / 1e9,
