@@ -58,7 +58,7 @@ extern "C" {
 #define NCN_ERR_ACTIVATION (-4)  /* unknown activation code */
 #define NCN_ERR_WORKSPACE (-5)   /* workspace missing or smaller than ncn_workspace_bytes() */
 #define NCN_ERR_UNSUPPORTED (-6) /* n_cache > 64, or head width too large for the generic kernel */
-#define NCN_ERR_ALIGN (-7)       /* a pointer is not 16-byte aligned */
+#define NCN_ERR_ALIGN (-7)       /* a pointer is not 16-byte aligned (4-byte for the int32 tables) */
 #define NCN_ERR_ALIAS (-8)       /* n_stages > 1 needs the state buffers the call would carry it in */
 
 /* Shape of one problem; shared by all entry points. */
@@ -134,6 +134,48 @@ int ncn_inverse(const void* y, const void* ya, int in_dtype,
                 const float* W,
                 const ncn_shape* shape, int first_stage, int n_stages,
                 float alpha, float m, int activation, void* stream);
+
+/*
+ * The same three operations with the grouping given as a table and, optionally, one context length per batch entry.
+ * Replaces: the group_tensor / ctxlen_tensor arguments of fused_chunk_linear_ncn and its kernels
+ *           (ncn_triton/ncn_triton_old.py:53-57, 66-71, 93-96, 362-387), whose tables come from helpers such as the
+ *           radix-n digit grouping of ncn_triton/group_tensors.py:8-18.
+ * group_index in  int32 [n_stages, N], or NULL for the stride permutation of first_stage + k (first_stage is only
+ *                 read then).  For stage k, slot o of group g is the row at position group_index[k*N + g*n_cache + o]
+ *                 of the N axis.  Every row of the table must be a permutation of 0 .. N-1: the library cannot check
+ *                 that; entries are clamped into range, so a bad table gives wrong numbers but no stray access.
+ * ctx_len     in  int32 [batch], or NULL for N everywhere.  Batch entry b only has its first ctx_len[b] slots (in the
+ *                 order of the table): groups wholly below the length run as usual; the group the length cuts runs
+ *                 on its live rows only, with as many steps as it has live rows; rows past the length pass through
+ *                 (forward, inverse: out = in; backward: dx = dy, dxa = dya, x_rec = y, no share in dW).  Values are
+ *                 clamped to [0, N].  Needs a head width <= 64 (NCN_ERR_UNSUPPORTED otherwise).
+ * Everything else as in ncn_forward / ncn_backward / ncn_inverse, except that these always run stage by stage (no
+ * multi-stage passes, so forward takes no workspace) and ncn_backward_indexed needs ncn_workspace_bytes(shape).
+ */
+int ncn_forward_indexed(const void* x, const void* xa, int in_dtype,
+                        void* y, void* ya, int out_dtype,
+                        float* y32, float* ya32,
+                        const float* W,
+                        const int32_t* group_index, const int32_t* ctx_len,
+                        const ncn_shape* shape, int first_stage, int n_stages,
+                        float alpha, float m, int activation, void* stream);
+
+int ncn_backward_indexed(const void* y, const void* ya, int y_dtype,
+                         const void* dy, const void* dya, int dy_dtype,
+                         void* dx, void* dxa, int dx_dtype,
+                         float* x_rec, float* xa_rec,
+                         const float* W, float* dW,
+                         void* workspace, size_t workspace_bytes,
+                         const int32_t* group_index, const int32_t* ctx_len,
+                         const ncn_shape* shape, int first_stage, int n_stages,
+                         float alpha, float m, int activation, void* stream);
+
+int ncn_inverse_indexed(const void* y, const void* ya, int in_dtype,
+                        void* x, void* xa, int out_dtype,
+                        const float* W,
+                        const int32_t* group_index, const int32_t* ctx_len,
+                        const ncn_shape* shape, int first_stage, int n_stages,
+                        float alpha, float m, int activation, void* stream);
 
 /* Bytes of scratch ncn_backward needs for this shape (0 on an invalid shape).  No reference counterpart:
  * the reference allocates a [batch,N,2E] partial-dW tensor per call (ncn_bwd_cuda_kernel.cu:251). */

@@ -11,7 +11,8 @@ LIB_PATH = os.path.join(PKG_DIR, "libncn_hip.so")
 NCN_F32, NCN_BF16 = 0, 1
 ACT_TANH, ACT_RELU, ACT_SIGMOID, ACT_LEAKY_RELU, ACT_LINEAR = 0, 1, 2, 3, -1
 
-EXPORTS = ("ncn_forward", "ncn_backward", "ncn_inverse", "ncn_workspace_bytes", "ncn_workspace_bytes_stages",
+EXPORTS = ("ncn_forward", "ncn_backward", "ncn_inverse", "ncn_forward_indexed", "ncn_backward_indexed",
+           "ncn_inverse_indexed", "ncn_workspace_bytes", "ncn_workspace_bytes_stages",
            "ncn_plan_passes", "ncn_kernel_path",
            "ncn_check_shape", "ncn_error_string", "ncn_version")
 
@@ -43,6 +44,13 @@ def load():
                                  shp, i, i, fl, fl, i, vp]
     lib.ncn_inverse.restype = i
     lib.ncn_inverse.argtypes = [vp, vp, i, vp, vp, i, f32p, shp, i, i, fl, fl, i, vp]
+    lib.ncn_forward_indexed.restype = i
+    lib.ncn_forward_indexed.argtypes = [vp, vp, i, vp, vp, i, f32p, f32p, f32p, vp, vp, shp, i, i, fl, fl, i, vp]
+    lib.ncn_backward_indexed.restype = i
+    lib.ncn_backward_indexed.argtypes = [vp, vp, i, vp, vp, i, vp, vp, i, f32p, f32p, f32p, f32p, vp, ctypes.c_size_t,
+                                         vp, vp, shp, i, i, fl, fl, i, vp]
+    lib.ncn_inverse_indexed.restype = i
+    lib.ncn_inverse_indexed.argtypes = [vp, vp, i, vp, vp, i, f32p, vp, vp, shp, i, i, fl, fl, i, vp]
     lib.ncn_workspace_bytes.restype = ctypes.c_size_t
     lib.ncn_workspace_bytes.argtypes = [shp]
     lib.ncn_workspace_bytes_stages.restype = ctypes.c_size_t

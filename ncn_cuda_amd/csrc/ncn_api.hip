@@ -57,8 +57,10 @@ struct Plan {
     int partial_rows;  // rows of the dW partial buffer the backward launch writes
 };
 
-Plan make_plan(const ncn_shape* sh, int activation) {
+// reserve_rows: rows of the dW partial buffer kept free for another launch of the same stage
+Plan make_plan(const ncn_shape* sh, int activation, int reserve_rows = 0) {
     Plan p;
+    const int max_rows = kMaxGridX - reserve_rows;
     p.path = kernel_path(sh, activation);
     const int ec = (int)(sh->E / sh->n_head);
     p.groups_per_tile = (p.path == 2) ? fast_groups_per_tile(sh->n_cache, ec) : generic_groups_per_tile(sh->n_cache);
@@ -71,7 +73,7 @@ Plan make_plan(const ncn_shape* sh, int activation) {
         const int C = sh->n_head;
         const int g4 = (C % 4 == 0) ? 4 : (C % 2 == 0 ? 2 : 1);
         const int64_t quantum = C / g4;                                   // blocks per multiple of n_head waves
-        const int64_t cap = (int64_t)kMaxGridX * C / 4 / quantum * quantum;  // rows = blocks * 4 / C <= kMaxGridX
+        const int64_t cap = (int64_t)max_rows * C / 4 / quantum * quantum;  // rows = blocks * 4 / C <= max_rows
         int64_t blocks = ((int64_t)p.total_tiles * C + 3) / 4;
         blocks = (blocks + quantum - 1) / quantum * quantum;
         // forward / inverse write no partials: one wave tile per wave where possible (measured 8 % faster than a
@@ -86,7 +88,7 @@ Plan make_plan(const ncn_shape* sh, int activation) {
         p.grid_x = (int)blocks;
         p.partial_rows = (int)(blocks * 4 / C);
     } else {
-        p.grid_x = (int)(p.total_tiles < (uint32_t)kMaxGridX ? p.total_tiles : (uint32_t)kMaxGridX);
+        p.grid_x = (int)(p.total_tiles < (uint32_t)max_rows ? p.total_tiles : (uint32_t)max_rows);
         p.grid_fwd = p.grid_x;
         p.partial_rows = p.grid_x;
     }
@@ -113,7 +115,25 @@ void fill_step_table(StepTable& t, int n_cache, float alpha, float m, int activa
     }
 }
 
-void fill_common(StageArgs& a, const ncn_shape* sh, const Plan& p, int stage, float alpha, float m, int activation) {
+// How the rows are grouped and which of them are live: caller's tables of the *_indexed entry points, or nothing.
+struct Grouping {
+    const int32_t* table;    // [n_stages, N] or null
+    const int32_t* ctx_len;  // [batch] or null
+    bool plain() const { return !table && !ctx_len; }
+};
+
+int check_grouping(const Grouping& g, const ncn_shape* sh) {
+    if ((reinterpret_cast<uintptr_t>(g.table) & 3u) || (reinterpret_cast<uintptr_t>(g.ctx_len) & 3u)) return NCN_ERR_ALIGN;
+    // the partly live group of a batch entry runs on the generic kernel
+    if (g.ctx_len && sh->E / sh->n_head > kGenericMaxHeadDim) return NCN_ERR_UNSUPPORTED;
+    return NCN_OK;
+}
+
+void fill_common(StageArgs& a, const ncn_shape* sh, const Plan& p, int stage, float alpha, float m, int activation,
+                 const Grouping& g = Grouping{nullptr, nullptr}, int rel_stage = 0) {
+    a.table = g.table ? g.table + (int64_t)rel_stage * sh->N : nullptr;
+    a.ctx_len = g.ctx_len;
+    a.edge = 0;
     a.N = sh->N;
     a.E = sh->E;
     a.total_tiles = p.total_tiles;
@@ -127,6 +147,21 @@ void fill_common(StageArgs& a, const ncn_shape* sh, const Plan& p, int stage, fl
     a.activation = activation;
     fill_step_table(a.tab, sh->n_cache, alpha, m, activation);
 }
+
+// With context lengths: the partly live group of every batch entry (generic kernel, one tile per batch entry),
+// then the rows past the lengths.  `a` is the stage's argument block as the main launch used it.
+hipError_t launch_ragged_rest(Pass pass, StageArgs a, const ncn_shape* sh, int partial_rows_used, hipStream_t s) {
+    StageArgs e = a;
+    e.edge = 1;
+    e.total_tiles = (uint32_t)sh->batch;
+    e.tiles_per_inst = 1;
+    if (pass == kBackward) e.dw_partials = a.dw_partials + (int64_t)partial_rows_used * 2 * sh->E;
+    const int grid = (int)(sh->batch < kEdgeGridX ? sh->batch : kEdgeGridX);
+    hipError_t err = launch_generic(pass, e, sh->n_head, grid, s);
+    if (err != hipSuccess) return err;
+    return launch_pass_through(pass, a, sh->batch, s);
+}
+int edge_rows(const ncn_shape* sh) { return (int)(sh->batch < kEdgeGridX ? sh->batch : kEdgeGridX); }
 
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
@@ -212,10 +247,13 @@ size_t ncn_workspace_bytes_stages(const ncn_shape* shape, int first_stage, int n
     return passes.size() >= 2 ? base + temp_bytes(shape, backward != 0) : base;
 }
 
-int ncn_forward(const void* x, const void* xa, int in_dtype, void* y, void* ya, int out_dtype, float* y32, float* ya32,
-                const float* W, void* workspace, size_t workspace_bytes, const ncn_shape* shape, int first_stage,
-                int n_stages, float alpha, float m, int activation, void* stream) {
+static int forward_impl(const void* x, const void* xa, int in_dtype, void* y, void* ya, int out_dtype, float* y32,
+                        float* ya32, const float* W, void* workspace, size_t workspace_bytes, const Grouping& grouping,
+                        const ncn_shape* shape, int first_stage, int n_stages, float alpha, float m, int activation,
+                        void* stream) {
     int rc = check_shape(shape, first_stage, n_stages, activation);
+    if (rc != NCN_OK) return rc;
+    rc = check_grouping(grouping, shape);
     if (rc != NCN_OK) return rc;
     if (!x || !xa || !y || !ya || !W) return NCN_ERR_NULL;
     if ((y32 == nullptr) != (ya32 == nullptr)) return NCN_ERR_NULL;
@@ -228,7 +266,8 @@ int ncn_forward(const void* x, const void* xa, int in_dtype, void* y, void* ya, 
     const int64_t wstride = 2 * shape->E;
 
     // several stages: LDS-resident passes when the shape allows and the buffers permit the ping-pong
-    std::vector<FusedPass> passes = multi_stage_plan(shape, first_stage, n_stages, activation, false);
+    std::vector<FusedPass> passes;
+    if (grouping.plain()) passes = multi_stage_plan(shape, first_stage, n_stages, activation, false);
     const size_t np = passes.size();
     bool fused_ok = np > 0;
     if (np >= 2 && (out_dtype != NCN_F32 || !workspace || workspace_bytes < temp_bytes(shape, false))) fused_ok = false;
@@ -275,7 +314,7 @@ int ncn_forward(const void* x, const void* xa, int in_dtype, void* y, void* ya, 
 
     for (int k = 0; k < n_stages; ++k) {
         StageArgs a{};
-        fill_common(a, shape, p, first_stage + k, alpha, m, activation);
+        fill_common(a, shape, p, first_stage + k, alpha, m, activation, grouping, k);
         a.in0 = k == 0 ? x : y;
         a.in1 = k == 0 ? xa : ya;
         a.in_dtype = k == 0 ? in_dtype : out_dtype;
@@ -286,17 +325,21 @@ int ncn_forward(const void* x, const void* xa, int in_dtype, void* y, void* ya, 
         a.aux0 = last ? y32 : nullptr;
         a.aux1 = last ? ya32 : nullptr;
         a.W = W + k * wstride;
-        hipError_t err = (p.path == 2) ? launch_fast_forward(kForward, a, shape->n_head, p.grid_fwd, s)
-                                       : launch_generic(kForward, a, shape->n_head, p.grid_fwd, s);
+        hipError_t err = (p.path != 2)      ? launch_generic(kForward, a, shape->n_head, p.grid_fwd, s)
+                         : grouping.plain() ? launch_fast_forward(kForward, a, shape->n_head, p.grid_fwd, s)
+                                            : launch_fast_forward_indexed(kForward, a, shape->n_head, p.grid_fwd, s);
+        if (err == hipSuccess && grouping.ctx_len) err = launch_ragged_rest(kForward, a, shape, 0, s);
         if (err != hipSuccess) return (int)err;
     }
     return NCN_OK;
 }
 
-int ncn_inverse(const void* y, const void* ya, int in_dtype, void* x, void* xa, int out_dtype, const float* W,
-                const ncn_shape* shape, int first_stage, int n_stages, float alpha, float m, int activation,
-                void* stream) {
+static int inverse_impl(const void* y, const void* ya, int in_dtype, void* x, void* xa, int out_dtype, const float* W,
+                        const Grouping& grouping, const ncn_shape* shape, int first_stage, int n_stages, float alpha,
+                        float m, int activation, void* stream) {
     int rc = check_shape(shape, first_stage, n_stages, activation);
+    if (rc != NCN_OK) return rc;
+    rc = check_grouping(grouping, shape);
     if (rc != NCN_OK) return rc;
     if (!x || !xa || !y || !ya || !W) return NCN_ERR_NULL;
     if (!known_dtype(in_dtype) || !known_dtype(out_dtype)) return NCN_ERR_DTYPE;
@@ -305,7 +348,7 @@ int ncn_inverse(const void* y, const void* ya, int in_dtype, void* x, void* xa, 
     hipStream_t s = static_cast<hipStream_t>(stream);
     for (int k = n_stages - 1; k >= 0; --k) {
         StageArgs a{};
-        fill_common(a, shape, p, first_stage + k, alpha, m, activation);
+        fill_common(a, shape, p, first_stage + k, alpha, m, activation, grouping, k);
         const bool first = (k == n_stages - 1);
         a.in0 = first ? y : x;
         a.in1 = first ? ya : xa;
@@ -314,18 +357,22 @@ int ncn_inverse(const void* y, const void* ya, int in_dtype, void* x, void* xa, 
         a.out1 = xa;
         a.out_dtype = out_dtype;
         a.W = W + (int64_t)k * 2 * shape->E;
-        hipError_t err = (p.path == 2) ? launch_fast_forward(kInverse, a, shape->n_head, p.grid_fwd, s)
-                                       : launch_generic(kInverse, a, shape->n_head, p.grid_fwd, s);
+        hipError_t err = (p.path != 2)      ? launch_generic(kInverse, a, shape->n_head, p.grid_fwd, s)
+                         : grouping.plain() ? launch_fast_forward(kInverse, a, shape->n_head, p.grid_fwd, s)
+                                            : launch_fast_forward_indexed(kInverse, a, shape->n_head, p.grid_fwd, s);
+        if (err == hipSuccess && grouping.ctx_len) err = launch_ragged_rest(kInverse, a, shape, 0, s);
         if (err != hipSuccess) return (int)err;
     }
     return NCN_OK;
 }
 
-int ncn_backward(const void* y, const void* ya, int y_dtype, const void* dy, const void* dya, int dy_dtype, void* dx,
-                 void* dxa, int dx_dtype, float* x_rec, float* xa_rec, const float* W, float* dW, void* workspace,
-                 size_t workspace_bytes, const ncn_shape* shape, int first_stage, int n_stages, float alpha, float m,
-                 int activation, void* stream) {
+static int backward_impl(const void* y, const void* ya, int y_dtype, const void* dy, const void* dya, int dy_dtype,
+                         void* dx, void* dxa, int dx_dtype, float* x_rec, float* xa_rec, const float* W, float* dW,
+                         void* workspace, size_t workspace_bytes, const Grouping& grouping, const ncn_shape* shape,
+                         int first_stage, int n_stages, float alpha, float m, int activation, void* stream) {
     int rc = check_shape(shape, first_stage, n_stages, activation);
+    if (rc != NCN_OK) return rc;
+    rc = check_grouping(grouping, shape);
     if (rc != NCN_OK) return rc;
     if (!y || !ya || !dy || !dx || !dxa || !W || !dW) return NCN_ERR_NULL;
     if ((x_rec == nullptr) != (xa_rec == nullptr)) return NCN_ERR_NULL;
@@ -335,7 +382,8 @@ int ncn_backward(const void* y, const void* ya, int y_dtype, const void* dy, con
     if (!aligned16(y) || !aligned16(ya) || !aligned16(dy) || !aligned16(dya) || !aligned16(dx) || !aligned16(dxa) ||
         !aligned16(x_rec) || !aligned16(xa_rec) || !aligned16(W) || !aligned16(dW) || !aligned16(workspace))
         return NCN_ERR_ALIGN;
-    const Plan p = make_plan(shape, activation);
+    const int extra_rows = grouping.ctx_len ? edge_rows(shape) : 0;  // partial rows of the edge launch
+    const Plan p = make_plan(shape, activation, extra_rows);
     hipStream_t s = static_cast<hipStream_t>(stream);
     float* partials = static_cast<float*>(workspace);
     float* level1 = partials + (int64_t)kMaxGridX * 2 * shape->E;
@@ -343,7 +391,8 @@ int ncn_backward(const void* y, const void* ya, int y_dtype, const void* dy, con
 
     // several stages: LDS-resident passes, last pass of the range first; the state ping-pongs between the
     // output arrays and four float32 arrays behind the dW scratch
-    std::vector<FusedPass> passes = multi_stage_plan(shape, first_stage, n_stages, activation, true);
+    std::vector<FusedPass> passes;
+    if (grouping.plain()) passes = multi_stage_plan(shape, first_stage, n_stages, activation, true);
     const size_t np = passes.size();
     bool fused_ok = np > 0;
     if (np >= 2 && workspace_bytes < base_workspace_bytes(shape) + temp_bytes(shape, true)) fused_ok = false;
@@ -403,7 +452,7 @@ int ncn_backward(const void* y, const void* ya, int y_dtype, const void* dy, con
 
     for (int k = n_stages - 1; k >= 0; --k) {
         StageArgs a{};
-        fill_common(a, shape, p, first_stage + k, alpha, m, activation);
+        fill_common(a, shape, p, first_stage + k, alpha, m, activation, grouping, k);
         const bool top = (k == n_stages - 1);
         a.in0 = top ? y : x_rec;
         a.in1 = top ? ya : xa_rec;
@@ -418,13 +467,63 @@ int ncn_backward(const void* y, const void* ya, int y_dtype, const void* dy, con
         a.aux1 = xa_rec;
         a.W = W + (int64_t)k * 2 * shape->E;
         a.dw_partials = partials;
-        hipError_t err = (p.path == 2) ? launch_fast_backward(a, shape->n_head, p.grid_x, s)
-                                       : launch_generic(kBackward, a, shape->n_head, p.grid_x, s);
+        hipError_t err = (p.path != 2)      ? launch_generic(kBackward, a, shape->n_head, p.grid_x, s)
+                         : grouping.plain() ? launch_fast_backward(a, shape->n_head, p.grid_x, s)
+                                            : launch_fast_backward_indexed(a, shape->n_head, p.grid_x, s);
+        if (err == hipSuccess && grouping.ctx_len) err = launch_ragged_rest(kBackward, a, shape, p.partial_rows, s);
         if (err != hipSuccess) return (int)err;
-        err = launch_reduce_dw(partials, p.partial_rows, wstride, wstride, level1, dW + k * wstride, s);
+        err = launch_reduce_dw(partials, p.partial_rows + extra_rows, wstride, wstride, level1, dW + k * wstride, s);
         if (err != hipSuccess) return (int)err;
     }
     return NCN_OK;
+}
+
+int ncn_forward(const void* x, const void* xa, int in_dtype, void* y, void* ya, int out_dtype, float* y32, float* ya32,
+                const float* W, void* workspace, size_t workspace_bytes, const ncn_shape* shape, int first_stage,
+                int n_stages, float alpha, float m, int activation, void* stream) {
+    return forward_impl(x, xa, in_dtype, y, ya, out_dtype, y32, ya32, W, workspace, workspace_bytes,
+                        Grouping{nullptr, nullptr}, shape, first_stage, n_stages, alpha, m, activation, stream);
+}
+
+int ncn_forward_indexed(const void* x, const void* xa, int in_dtype, void* y, void* ya, int out_dtype, float* y32,
+                        float* ya32, const float* W, const int32_t* group_index, const int32_t* ctx_len,
+                        const ncn_shape* shape, int first_stage, int n_stages, float alpha, float m, int activation,
+                        void* stream) {
+    return forward_impl(x, xa, in_dtype, y, ya, out_dtype, y32, ya32, W, nullptr, 0, Grouping{group_index, ctx_len},
+                        shape, first_stage, n_stages, alpha, m, activation, stream);
+}
+
+int ncn_inverse(const void* y, const void* ya, int in_dtype, void* x, void* xa, int out_dtype, const float* W,
+                const ncn_shape* shape, int first_stage, int n_stages, float alpha, float m, int activation,
+                void* stream) {
+    return inverse_impl(y, ya, in_dtype, x, xa, out_dtype, W, Grouping{nullptr, nullptr}, shape, first_stage, n_stages,
+                        alpha, m, activation, stream);
+}
+
+int ncn_inverse_indexed(const void* y, const void* ya, int in_dtype, void* x, void* xa, int out_dtype, const float* W,
+                        const int32_t* group_index, const int32_t* ctx_len, const ncn_shape* shape, int first_stage,
+                        int n_stages, float alpha, float m, int activation, void* stream) {
+    return inverse_impl(y, ya, in_dtype, x, xa, out_dtype, W, Grouping{group_index, ctx_len}, shape, first_stage,
+                        n_stages, alpha, m, activation, stream);
+}
+
+int ncn_backward(const void* y, const void* ya, int y_dtype, const void* dy, const void* dya, int dy_dtype, void* dx,
+                 void* dxa, int dx_dtype, float* x_rec, float* xa_rec, const float* W, float* dW, void* workspace,
+                 size_t workspace_bytes, const ncn_shape* shape, int first_stage, int n_stages, float alpha, float m,
+                 int activation, void* stream) {
+    return backward_impl(y, ya, y_dtype, dy, dya, dy_dtype, dx, dxa, dx_dtype, x_rec, xa_rec, W, dW, workspace,
+                         workspace_bytes, Grouping{nullptr, nullptr}, shape, first_stage, n_stages, alpha, m, activation,
+                         stream);
+}
+
+int ncn_backward_indexed(const void* y, const void* ya, int y_dtype, const void* dy, const void* dya, int dy_dtype,
+                         void* dx, void* dxa, int dx_dtype, float* x_rec, float* xa_rec, const float* W, float* dW,
+                         void* workspace, size_t workspace_bytes, const int32_t* group_index, const int32_t* ctx_len,
+                         const ncn_shape* shape, int first_stage, int n_stages, float alpha, float m, int activation,
+                         void* stream) {
+    return backward_impl(y, ya, y_dtype, dy, dya, dy_dtype, dx, dxa, dx_dtype, x_rec, xa_rec, W, dW, workspace,
+                         workspace_bytes, Grouping{group_index, ctx_len}, shape, first_stage, n_stages, alpha, m,
+                         activation, stream);
 }
 
 }  // extern "C"

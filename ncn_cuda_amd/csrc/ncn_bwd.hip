@@ -1,18 +1,29 @@
 // Instantiations and dispatch of the register-resident reversible backward stage kernel.
+// Compiled twice: as it stands for the stride permutation, and through ncn_bwd_indexed.hip (NCN_INDEXED_BUILD = 1)
+// for launches that carry a grouping table or context lengths.
 #include "ncn_configs.h"
 #include "ncn_launch.h"
 #include "ncn_stage_kernels.h"
 
+#ifndef NCN_INDEXED_BUILD
+#define NCN_INDEXED_BUILD 0
+#endif
+
 namespace ncn {
 
+#if NCN_INDEXED_BUILD
+hipError_t launch_fast_backward_indexed(const StageArgs& a, int n_head, int grid_x, hipStream_t s) {
+#else
 hipError_t launch_fast_backward(const StageArgs& a, int n_head, int grid_x, hipStream_t s) {
+#endif
+    constexpr bool kIndexed = NCN_INDEXED_BUILD != 0;
     const dim3 grid(grid_x), block(kBlockThreads);
     const bool tanh_only = a.activation == NCN_ACT_TANH;
 #define NCN_CASE(NC, EC, R, F)                                                                  \
     static_assert(fast_tile(NC, EC).r == R && fast_tile(NC, EC).f == F, "duplicate config entry");          \
     if (a.n_cache == NC && a.head_dim == EC) {                                                 \
-        if (tanh_only) hipLaunchKernelGGL((stage_backward_kernel<NC, EC, R, F, true>), grid, block, 0, s, a); \
-        else hipLaunchKernelGGL((stage_backward_kernel<NC, EC, R, F, false>), grid, block, 0, s, a);          \
+        if (tanh_only) hipLaunchKernelGGL((stage_backward_kernel<NC, EC, R, F, true, kIndexed>), grid, block, 0, s, a); \
+        else hipLaunchKernelGGL((stage_backward_kernel<NC, EC, R, F, false, kIndexed>), grid, block, 0, s, a);          \
         return hipGetLastError();                                                              \
     }
     NCN_FOR_EACH_FAST_CONFIG(NCN_CASE)

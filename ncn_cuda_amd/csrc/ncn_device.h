@@ -30,6 +30,10 @@ struct StepTable {
 //   inverse : in0,in1 = y,ya        out0,out1 = x,xa
 //   backward: in0,in1 = y,ya        g0,g1 = dy,dya (g1 may be null = zeros)
 //             out0,out1 = dx,dxa    aux0,aux1 = optional float32 reconstructed x,xa
+// Grouping: slot o of group g sits at position table[g * n_cache + o] when a table is given, else at the stride
+// permutation's ((g + o * stride) % groups) * n_cache + o.  With ctx_len, batch entry b only has its first
+// ctx_len[b] slots (in group order); the launches split the work: `edge == 0` runs the groups that are wholly
+// live, `edge == 1` (generic kernel only) the one partly live group of each batch entry.
 struct StageArgs {
     const void* in0;
     const void* in1;
@@ -41,6 +45,8 @@ struct StageArgs {
     float* aux1;
     const float* W;      // [2E] of this stage
     float* dw_partials;  // backward: [partial rows][2E]
+    const int32_t* table;    // [N] slot -> position, or null
+    const int32_t* ctx_len;  // [batch] live slots per batch entry, or null
     int64_t N, E;
     uint32_t total_tiles;     // batch * tiles_per_instance
     uint32_t tiles_per_inst;  // ceil(groups / groups-per-wave-tile)
@@ -50,6 +56,7 @@ struct StageArgs {
     int32_t n_cache, head_dim, n_head;
     int32_t in_dtype, g_dtype, out_dtype;
     int32_t activation;
+    int32_t edge;
     StepTable tab;
 };
 
@@ -235,6 +242,28 @@ __device__ __forceinline__ void act_fd(int code, float T, float& F, float& dF) {
 __device__ __forceinline__ uint32_t stage_block(const StageArgs& A, uint32_t group, uint32_t slot) {
     const uint32_t t = group + slot * A.stride;  // < 65 * groups, checked on the host to fit 32 bits
     return A.groups_pow2 ? (t & (A.groups - 1u)) : (t % A.groups);
+}
+
+// Position on the N axis of slot `slot` of group `group`.  A table entry is clamped into [0, N): a table that is
+// not a permutation gives wrong numbers, never an access outside the tensors.
+__device__ __forceinline__ int64_t slot_position(const StageArgs& A, uint32_t group, uint32_t slot) {
+    if (A.table) {
+        const int32_t p = A.table[(int64_t)group * A.n_cache + slot];
+        return (int64_t)max(0, min(p, (int32_t)A.N - 1));
+    }
+    return (int64_t)stage_block(A, group, slot) * A.n_cache + slot;
+}
+
+// Live slots of batch entry b (ncn_triton/ncn_triton_old.py:66: one context length per batch entry).
+__device__ __forceinline__ int32_t live_slots(const StageArgs& A, uint32_t b) {
+    return A.ctx_len ? max(0, min(A.ctx_len[b], (int32_t)A.N)) : (int32_t)A.N;
+}
+
+// Live rows of group `group` of batch entry b: n_cache, fewer for the group the length cuts, 0 beyond it.
+__device__ __forceinline__ int32_t live_rows(const StageArgs& A, uint32_t b, uint32_t group) {
+    if (!A.ctx_len) return A.n_cache;
+    const int64_t r = (int64_t)live_slots(A, b) - (int64_t)group * A.n_cache;
+    return (int32_t)max((int64_t)0, min(r, (int64_t)A.n_cache));
 }
 
 }  // namespace ncn

@@ -15,21 +15,35 @@ struct GenericLane {
     int64_t off;   // element offset of this lane's row, feature 0 of the head
     int row;       // slot inside the group
     int base;      // lane of slot 0 of this lane's group
+    int steps;     // steps of the recurrence = live rows of the group (the same for the whole block)
 };
 
+// Wave tile t.  Normal launches: floor(64/n) whole groups, skipping groups a context length cuts.  Edge launches
+// (A.edge): t is a batch entry and the tile is its one partly live group, rows and steps = its live rows
+// (ncn_triton/ncn_triton_old.py:93-96).
 __device__ __forceinline__ GenericLane generic_lane(const StageArgs& A, uint32_t t, int lane, int head) {
     GenericLane L;
     const int n = A.n_cache;
-    const int gpw = 64 / n;
-    const int gw = lane / n;
-    L.row = lane - gw * n;
-    L.base = gw * n;
-    const uint32_t b = t / A.tiles_per_inst;
-    const uint32_t tile = t - b * A.tiles_per_inst;
-    const uint32_t group = tile * gpw + gw;
-    L.valid = (gw < gpw) && (group < A.groups);
-    const uint32_t blk = stage_block(A, L.valid ? group : 0u, (uint32_t)L.row);
-    const int64_t pos = (int64_t)blk * n + L.row;
+    uint32_t b, group;
+    if (A.edge) {
+        b = t;
+        group = (uint32_t)(live_slots(A, b) / n);
+        L.steps = group < A.groups ? live_rows(A, b, group) : 0;
+        L.row = lane;
+        L.base = 0;
+        L.valid = lane < L.steps;
+    } else {
+        const int gpw = 64 / n;
+        const int gw = lane / n;
+        L.row = lane - gw * n;
+        L.base = gw * n;
+        b = t / A.tiles_per_inst;
+        const uint32_t tile = t - b * A.tiles_per_inst;
+        group = tile * gpw + gw;
+        L.steps = n;
+        L.valid = (gw < gpw) && (group < A.groups) && live_rows(A, b, group) == n;
+    }
+    const int64_t pos = slot_position(A, L.valid ? group : 0u, L.valid ? (uint32_t)L.row : 0u);
     L.off = ((int64_t)b * A.N + pos) * A.E + (int64_t)head * A.head_dim;
     if (!L.valid) L.base = lane, L.row = 0;  // idle lanes talk to themselves only
     return L;
@@ -41,7 +55,7 @@ __device__ __forceinline__ GenericLane generic_lane(const StageArgs& A, uint32_t
 // pass 0: forward, pass 1: inverse
 __global__ void __launch_bounds__(64) generic_forward_kernel(const StageArgs A, const int inverse) {
     extern __shared__ float lds[];
-    const int lane = threadIdx.x, head = blockIdx.y, ec = A.head_dim, n = A.n_cache;
+    const int lane = threadIdx.x, head = blockIdx.y, ec = A.head_dim;
     const float alpha = A.tab.alpha, m = A.tab.m, om = 1.f - A.tab.m, oa = 1.f - A.tab.alpha;
     const float inv_m = 1.f / m, k_ba = om / m;
     const float* Wi = A.W + (int64_t)head * ec;
@@ -54,8 +68,8 @@ __global__ void __launch_bounds__(64) generic_forward_kernel(const StageArgs A, 
             LDS(XA, f) = L.valid ? load_elem(A.in1, A.in_dtype, L.off + f) : 0.f;
         }
         __syncthreads();
-        for (int step = 0; step < n; ++step) {
-            const int j = inverse ? n - 1 - step : step;
+        for (int step = 0; step < L.steps; ++step) {
+            const int j = inverse ? L.steps - 1 - step : step;
             const int jl = L.valid ? L.base + j : lane;
             if (inverse) {
                 for (int f = 0; f < ec; ++f) LDS(X, f) = fmaf(LDS(X, f), inv_m, -k_ba * LDS(XA, f));
@@ -99,7 +113,7 @@ __global__ void __launch_bounds__(64) generic_forward_kernel(const StageArgs A, 
 
 __global__ void __launch_bounds__(64) generic_backward_kernel(const StageArgs A) {
     extern __shared__ float lds[];
-    const int lane = threadIdx.x, head = blockIdx.y, ec = A.head_dim, n = A.n_cache;
+    const int lane = threadIdx.x, head = blockIdx.y, ec = A.head_dim;
     const float alpha = A.tab.alpha, m = A.tab.m, om = 1.f - A.tab.m, oa = 1.f - A.tab.alpha;
     const float inv_m = 1.f / m, k_ba = om / m, k1 = om * om, k2 = om, kh1 = m * om;
     const float* Wi = A.W + (int64_t)head * ec;
@@ -115,7 +129,7 @@ __global__ void __launch_bounds__(64) generic_backward_kernel(const StageArgs A)
             LDS(H, f) = (L.valid && A.g1) ? load_elem(A.g1, A.g_dtype, L.off + f) : 0.f;
         }
         __syncthreads();
-        for (int j = n - 1; j >= 0; --j) {
+        for (int j = L.steps - 1; j >= 0; --j) {
             const int jl = L.valid ? L.base + j : lane;
             for (int f = 0; f < ec; ++f) LDS(X, f) = fmaf(LDS(X, f), inv_m, -k_ba * LDS(XA, f));
             __syncthreads();
@@ -145,7 +159,7 @@ __global__ void __launch_bounds__(64) generic_backward_kernel(const StageArgs A)
             if (L.valid && L.row == j) {
                 for (int f = 0; f < ec; ++f) {
                     float v = 0.f;
-                    for (int k = 0; k < n; ++k) v += LDS_AT(U, f, L.base + k);
+                    for (int k = 0; k < L.steps; ++k) v += LDS_AT(U, f, L.base + k);
                     LDS(G, f) += v;
                 }
             }
@@ -192,7 +206,43 @@ __global__ void __launch_bounds__(256) reduce_rows_kernel(const float* __restric
     if (ry == 0 && col < cols) out[(int64_t)blockIdx.y * cols + col] = (red[0][cx] + red[1][cx]) + (red[2][cx] + red[3][cx]);
 }
 
+// Rows past a batch entry's context length take no part in the stage: they pass through.
+//   forward / inverse: out = in (and the float32 copies)     backward: dx = dy, dxa = dya (0 when null), x_rec = y.
+// One wavefront per slot k = 0 .. N-1 of a batch entry, in group order.
+__global__ void __launch_bounds__(256) pass_through_kernel(const StageArgs A, const int backward, const int64_t slots) {
+    const int lane = threadIdx.x & 63;
+    for (int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); r < slots; r += (int64_t)gridDim.x * 4) {
+        const uint32_t b = (uint32_t)(r / A.N);
+        const int64_t k = r - (int64_t)b * A.N;
+        if (k < live_slots(A, b)) continue;
+        const int64_t pos = slot_position(A, (uint32_t)(k / A.n_cache), (uint32_t)(k % A.n_cache));
+        const int64_t off = ((int64_t)b * A.N + pos) * A.E;
+        for (int64_t e = lane; e < A.E; e += 64) {
+            const float v0 = load_elem(A.in0, A.in_dtype, off + e), v1 = load_elem(A.in1, A.in_dtype, off + e);
+            if (backward) {
+                store_elem(A.out0, A.out_dtype, off + e, load_elem(A.g0, A.g_dtype, off + e));
+                store_elem(A.out1, A.out_dtype, off + e, A.g1 ? load_elem(A.g1, A.g_dtype, off + e) : 0.f);
+            } else {
+                store_elem(A.out0, A.out_dtype, off + e, v0);
+                store_elem(A.out1, A.out_dtype, off + e, v1);
+            }
+            if (A.aux0) {
+                A.aux0[off + e] = v0;
+                A.aux1[off + e] = v1;
+            }
+        }
+    }
+}
+
 }  // namespace
+
+hipError_t launch_pass_through(Pass pass, const StageArgs& a, int64_t batch, hipStream_t s) {
+    const int64_t slots = batch * a.N;
+    const int64_t blocks = (slots + 3) / 4;
+    const unsigned grid = (unsigned)(blocks < 65536 ? blocks : 65536);
+    hipLaunchKernelGGL(pass_through_kernel, dim3(grid), dim3(256), 0, s, a, pass == kBackward ? 1 : 0, slots);
+    return hipGetLastError();
+}
 
 hipError_t launch_generic(Pass pass, const StageArgs& a, int n_head, int grid_x, hipStream_t s) {
     const int arrays = (pass == kBackward) ? kGenericArrays : 2;

@@ -44,7 +44,14 @@ constexpr int kReduceLevel1Rows = kMaxGridX / kReduceRowsPerBlock;
 
 hipError_t launch_fast_forward(Pass pass, const StageArgs& a, int n_head, int grid_x, hipStream_t s);
 hipError_t launch_fast_backward(const StageArgs& a, int n_head, int grid_x, hipStream_t s);
+// the same kernels built to honour a.table and a.ctx_len (the plain builds ignore both)
+hipError_t launch_fast_forward_indexed(Pass pass, const StageArgs& a, int n_head, int grid_x, hipStream_t s);
+hipError_t launch_fast_backward_indexed(const StageArgs& a, int n_head, int grid_x, hipStream_t s);
 hipError_t launch_generic(Pass pass, const StageArgs& a, int n_head, int grid_x, hipStream_t s);
+// Rows past the context length of their batch entry: copied through (a.ctx_len must be set).
+hipError_t launch_pass_through(Pass pass, const StageArgs& a, int64_t batch, hipStream_t s);
+// gridDim.x of the generic kernel's edge launch (the partly live group of each batch entry) == its dW partial rows.
+constexpr int kEdgeGridX = 256;
 // dW[col] = sum over `rows` rows of partials[row * row_stride + col]; level1 is scratch of kReduceLevel1Rows * cols floats.
 hipError_t launch_reduce_dw(const float* partials, int rows, int64_t row_stride, int64_t cols, float* level1, float* dW,
                             hipStream_t s);

@@ -45,7 +45,9 @@ struct Tile {
 };
 
 // Element offsets of this lane's R row fragments for wave tile `t`; false when the lane's group is past the end.
-template <int NC, int EC, int R, int F>
+// INDEXED builds read the grouping table and the context lengths when the launch has them; the plain builds only
+// know the stride permutation (and are what every launch without table and lengths uses).
+template <int NC, int EC, int R, int F, bool INDEXED>
 __device__ __forceinline__ bool tile_offsets(const StageArgs& A, uint32_t t, int lane, int head, int64_t (&off)[R]) {
     using T = Tile<NC, EC, R, F>;
     const int fl = lane % T::LF;
@@ -54,13 +56,15 @@ __device__ __forceinline__ bool tile_offsets(const StageArgs& A, uint32_t t, int
     const uint32_t b = t / A.tiles_per_inst;
     const uint32_t tile = t - b * A.tiles_per_inst;
     const uint32_t group = tile * T::GPW + gw;
-    const bool valid = group < A.groups;
+    bool valid = group < A.groups;
+    if (INDEXED) valid = valid && live_rows(A, b, group) == NC;  // partly live groups: generic kernel
     const int64_t base = (int64_t)b * A.N * A.E + (int64_t)head * EC + fl * F;
 #pragma unroll
     for (int rr = 0; rr < R; ++rr) {
         const uint32_t i = rl * R + rr;
-        const uint32_t blk = stage_block(A, valid ? group : 0u, i);
-        off[rr] = base + ((int64_t)blk * NC + i) * A.E;
+        const int64_t pos = INDEXED ? slot_position(A, valid ? group : 0u, i)
+                                    : (int64_t)stage_block(A, valid ? group : 0u, i) * NC + i;
+        off[rr] = base + pos * A.E;
     }
     return valid;
 }
@@ -356,12 +360,12 @@ __device__ __forceinline__ void backward_steps(float (&Y)[R][F], float (&B)[R][F
     float wi[F], wj[F];                                                                         \
     load_w<F>(A.W, A.E, head, EC, fl, wi, wj);
 
-template <int NC, int EC, int R, int F, bool TANH_ONLY = true>
+template <int NC, int EC, int R, int F, bool TANH_ONLY = true, bool INDEXED = false>
 __global__ void __launch_bounds__(kBlockThreads) stage_forward_kernel(const StageArgs A) {
     NCN_WAVE_PROLOGUE
     for (uint32_t t = gwave / A.n_head; t < A.total_tiles; t += tile_step) {
         int64_t off[R];
-        const bool valid = tile_offsets<NC, EC, R, F>(A, t, lane, head, off);
+        const bool valid = tile_offsets<NC, EC, R, F, INDEXED>(A, t, lane, head, off);
         float x[R][F], a[R][F];
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) {
@@ -381,12 +385,12 @@ __global__ void __launch_bounds__(kBlockThreads) stage_forward_kernel(const Stag
     }
 }
 
-template <int NC, int EC, int R, int F, bool TANH_ONLY = true>
+template <int NC, int EC, int R, int F, bool TANH_ONLY = true, bool INDEXED = false>
 __global__ void __launch_bounds__(kBlockThreads) stage_inverse_kernel(const StageArgs A) {
     NCN_WAVE_PROLOGUE
     for (uint32_t t = gwave / A.n_head; t < A.total_tiles; t += tile_step) {
         int64_t off[R];
-        const bool valid = tile_offsets<NC, EC, R, F>(A, t, lane, head, off);
+        const bool valid = tile_offsets<NC, EC, R, F, INDEXED>(A, t, lane, head, off);
         float y[R][F], b[R][F];
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) {
@@ -404,7 +408,7 @@ __global__ void __launch_bounds__(kBlockThreads) stage_inverse_kernel(const Stag
 
 // Tiles of up to 16 elements per lane fit 128 VGPRs (4 waves per SIMD) when the compiler is asked to; measured 3-4 %
 // faster than the 136 it picks by itself.  Larger tiles and the multi-activation build would spill, so they are left alone.
-template <int NC, int EC, int R, int F, bool TANH_ONLY = true>
+template <int NC, int EC, int R, int F, bool TANH_ONLY = true, bool INDEXED = false>
 __global__ void __launch_bounds__(kBlockThreads, (TANH_ONLY && R * F <= 16 && F == 4) ? 4 : 1) stage_backward_kernel(const StageArgs A) {
     NCN_WAVE_PROLOGUE
     float dwi[F], dwj[F];
@@ -413,7 +417,7 @@ __global__ void __launch_bounds__(kBlockThreads, (TANH_ONLY && R * F <= 16 && F 
 
     for (uint32_t t = gwave / A.n_head; t < A.total_tiles; t += tile_step) {
         int64_t off[R];
-        const bool valid = tile_offsets<NC, EC, R, F>(A, t, lane, head, off);
+        const bool valid = tile_offsets<NC, EC, R, F, INDEXED>(A, t, lane, head, off);
         float Y[R][F], B[R][F], G[R][F], H[R][F];
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) {

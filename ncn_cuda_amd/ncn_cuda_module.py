@@ -96,12 +96,56 @@ def _stream(dev):
     return ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
 
 
+def validate_grouping(group_index, ctx_len, batch, N, n_stages):
+    """Host-side checks of a grouping table [n_stages, N] (or [N] for one stage) and of context lengths [batch];
+    either may be None.  Shapes and dtypes only: whether the table is a permutation is checked by
+    check_group_table, which needs the values."""
+    for name, t in (("group_index", group_index), ("ctx_len", ctx_len)):
+        if t is None:
+            continue
+        if not isinstance(t, torch.Tensor):
+            raise TypeError(f"{name} must be a torch tensor")
+        if t.dtype not in (torch.int32, torch.int64):
+            raise TypeError(f"{name} must be int32 or int64, got {t.dtype}")
+    if group_index is not None and group_index.numel() != n_stages * N:
+        raise ValueError(f"group_index must hold {n_stages} x N = {n_stages * N} positions, got {group_index.numel()}")
+    if ctx_len is not None and ctx_len.numel() != batch:
+        raise ValueError(f"ctx_len must hold one length per batch entry ({batch}), got {ctx_len.numel()}")
+
+
+def check_group_table(group_index, N):
+    """Raises ValueError unless every row of the table is a permutation of 0 .. N-1 (the kernels clamp bad entries
+    but cannot repair a table).  Works on CPU or GPU tensors; on the GPU it synchronises."""
+    t = group_index.reshape(-1, N).to(torch.int64)
+    want = torch.arange(N, dtype=torch.int64, device=t.device).expand_as(t)
+    if not torch.equal(torch.sort(t, dim=1).values, want):
+        raise ValueError("group_index: every stage's row must be a permutation of 0 .. N-1")
+
+
+def _grouping(group_index, ctx_len, batch, N, n_stages, dev, check_tables):
+    validate_grouping(group_index, ctx_len, batch, N, n_stages)
+    gi = cl = None
+    if group_index is not None:
+        _require_gpu(group_index)
+        if check_tables:
+            check_group_table(group_index, N)
+        gi = group_index.detach().reshape(-1).to(device=dev, dtype=torch.int32).contiguous()
+    if ctx_len is not None:
+        cl = ctx_len.detach().reshape(-1).to(device=dev, dtype=torch.int32).contiguous()
+    return gi, cl
+
+
 def forward_stages(x, xa, W, alpha, activation, cache_dim, nhead, first_stage, n_stages, *, m=M_DEFAULT,
-                   out_dtype=None, save_fp32=False, out=None):
+                   out_dtype=None, save_fp32=False, out=None, group_index=None, ctx_len=None, check_tables=True):
     """Stages first_stage .. first_stage+n_stages-1 in one call.  W: [n_stages, 2E] (any shape with that many
-    values).  Returns (y, ya) or, with save_fp32, (y, ya, y32, ya32) where y32/ya32 are float32 copies."""
+    values).  Returns (y, ya) or, with save_fp32, (y, ya, y32, ya32) where y32/ya32 are float32 copies.
+    group_index [n_stages, N] replaces the stride permutation by a table of positions in (group, slot) order and
+    ctx_len [batch] gives every batch entry its own number of live slots (the group_tensor / ctxlen_tensor of
+    ncn_triton/ncn_triton_old.py:362-387); rows past the length pass through."""
     shape = validate(x, xa, W, cache_dim, nhead, activation, first_stage, n_stages)
     dev = _require_gpu(x, xa, W)
+    indexed = group_index is not None or ctx_len is not None
+    gi, cl = _grouping(group_index, ctx_len, x.shape[0], x.shape[1], n_stages, dev, check_tables)
     x, xa, w = _prep(x.detach()), _prep(xa.detach()), _w32(W)
     out_dtype = x.dtype if out_dtype is None else out_dtype
     if out is not None:
@@ -119,6 +163,14 @@ def forward_stages(x, xa, W, alpha, activation, cache_dim, nhead, first_stage, n
     aux = (y32, ya32) if (save_fp32 and out_dtype != torch.float32) else (None, None)
     lib = _lib.load()
     ws, ws_bytes = None, 0
+    if indexed:
+        with torch.cuda.device(dev):
+            rc = lib.ncn_forward_indexed(_ptr(x), _ptr(xa), _DTYPES[x.dtype], _ptr(y), _ptr(ya), _DTYPES[out_dtype],
+                                         _ptr(aux[0]), _ptr(aux[1]), _ptr(w), _ptr(gi), _ptr(cl), ctypes.byref(shape),
+                                         int(first_stage), int(n_stages), float(alpha), float(m), int(activation),
+                                         _stream(dev))
+        _lib.check(rc, "ncn_forward_indexed")
+        return (y, ya, y32, ya32) if save_fp32 else (y, ya)
     if n_stages > 1:
         ws_bytes = lib.ncn_workspace_bytes_stages(ctypes.byref(shape), int(first_stage), int(n_stages), int(activation), 0)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
@@ -132,7 +184,7 @@ def forward_stages(x, xa, W, alpha, activation, cache_dim, nhead, first_stage, n
 
 
 def backward_stages(y, ya, dy, dya, W, alpha, activation, cache_dim, nhead, first_stage, n_stages, *, m=M_DEFAULT,
-                    grad_dtype=None, want_inputs=True):
+                    grad_dtype=None, want_inputs=True, group_index=None, ctx_len=None, check_tables=True):
     """Reversible backward of stages first_stage+n_stages-1 .. first_stage from the outputs y, ya of the last one.
     dya may be None (zeros).  Returns (x_rec, xa_rec, dx, dxa, dW[n_stages, 2E]); x_rec/xa_rec are None when
     want_inputs is False and n_stages == 1."""
@@ -142,6 +194,8 @@ def backward_stages(y, ya, dy, dya, W, alpha, activation, cache_dim, nhead, firs
     if dy.dtype not in _DTYPES or (dya is not None and dya.dtype != dy.dtype):
         raise TypeError("dy and dya must both be float32 or bfloat16")
     dev = _require_gpu(y, ya, dy, dya, W)
+    indexed = group_index is not None or ctx_len is not None
+    gi, cl = _grouping(group_index, ctx_len, y.shape[0], y.shape[1], n_stages, dev, check_tables)
     y, ya, dy, w = _prep(y.detach()), _prep(ya.detach()), _prep(dy.detach()), _w32(W)
     dya = _prep(dya.detach()) if dya is not None else None
     grad_dtype = dy.dtype if grad_dtype is None else grad_dtype
@@ -155,6 +209,17 @@ def backward_stages(y, ya, dy, dya, W, alpha, activation, cache_dim, nhead, firs
     E = y.shape[2]
     dW = torch.empty(n_stages, 2 * E, dtype=torch.float32, device=dev)
     lib = _lib.load()
+    if indexed:
+        ws_bytes = lib.ncn_workspace_bytes(ctypes.byref(shape))
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        with torch.cuda.device(dev):
+            rc = lib.ncn_backward_indexed(_ptr(y), _ptr(ya), _DTYPES[y.dtype], _ptr(dy), _ptr(dya), _DTYPES[dy.dtype],
+                                          _ptr(dx), _ptr(dxa), _DTYPES[grad_dtype], _ptr(x_rec), _ptr(xa_rec), _ptr(w),
+                                          _ptr(dW), _ptr(ws), ctypes.c_size_t(ws_bytes), _ptr(gi), _ptr(cl),
+                                          ctypes.byref(shape), int(first_stage), int(n_stages), float(alpha), float(m),
+                                          int(activation), _stream(dev))
+        _lib.check(rc, "ncn_backward_indexed")
+        return x_rec, xa_rec, dx, dxa, dW
     ws_bytes = lib.ncn_workspace_bytes_stages(ctypes.byref(shape), int(first_stage), int(n_stages), int(activation), 1)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
@@ -167,14 +232,24 @@ def backward_stages(y, ya, dy, dya, W, alpha, activation, cache_dim, nhead, firs
 
 
 def inverse_stages(y, ya, W, alpha, activation, cache_dim, nhead, first_stage, n_stages, *, m=M_DEFAULT,
-                   out_dtype=None):
+                   out_dtype=None, group_index=None, ctx_len=None, check_tables=True):
     """x, xa with forward_stages(x, xa, ...) == (y, ya)."""
     shape = validate(y, ya, W, cache_dim, nhead, activation, first_stage, n_stages, what="y")
     dev = _require_gpu(y, ya, W)
+    indexed = group_index is not None or ctx_len is not None
+    gi, cl = _grouping(group_index, ctx_len, y.shape[0], y.shape[1], n_stages, dev, check_tables)
     y, ya, w = _prep(y.detach()), _prep(ya.detach()), _w32(W)
     out_dtype = y.dtype if out_dtype is None else out_dtype
     x = torch.empty(y.shape, dtype=out_dtype, device=dev)
     xa = torch.empty(y.shape, dtype=out_dtype, device=dev)
+    if indexed:
+        with torch.cuda.device(dev):
+            rc = _lib.load().ncn_inverse_indexed(_ptr(y), _ptr(ya), _DTYPES[y.dtype], _ptr(x), _ptr(xa),
+                                                 _DTYPES[out_dtype], _ptr(w), _ptr(gi), _ptr(cl), ctypes.byref(shape),
+                                                 int(first_stage), int(n_stages), float(alpha), float(m),
+                                                 int(activation), _stream(dev))
+        _lib.check(rc, "ncn_inverse_indexed")
+        return x, xa
     with torch.cuda.device(dev):
         rc = _lib.load().ncn_inverse(_ptr(y), _ptr(ya), _DTYPES[y.dtype], _ptr(x), _ptr(xa), _DTYPES[out_dtype],
                                      _ptr(w), ctypes.byref(shape), int(first_stage), int(n_stages), float(alpha),

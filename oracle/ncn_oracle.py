@@ -9,6 +9,8 @@ the CPU, the algorithm of the reference:
                                                                   stage_forward (same math, batched)
   * stage stack          torch_ref/ncn_pytorch.py:103-124      -> net_forward
   * one-step inverse     torch_ref/ncn_pytorch_invertible.py:87-113 -> stage_inverse / net_inverse
+  * tables and lengths   ncn_triton/ncn_triton_old.py:53-96 (group_tensor, ctxlen_tensor), group_tensors.py:8-18
+                                                               -> stage_forward_indexed, radix_group_table
   * backward             autograd through the forward is the reference's definition of the gradients
                          (grad_test_bench.py:72); the closed form used by the GPU kernels follows
                          ncn_triton/ncn_triton.py:176-246 and ncn_cuda/ncn_bwd_cuda_kernel.cu:88-216
@@ -21,7 +23,11 @@ forward round trips, the index map against the bijection/hand values.  No functi
 "parity unpinned" for activation == tanh.  The relu / sigmoid / linear activations exist only in the
 reference's CUDA kernels (ncn_fwd_cuda_kernel.cu:86-95) and leaky relu only in its Triton kernels
 (ncn_triton/ncn_triton.py:22-28), none of which can be built or run here; for them the oracle is
-pinned only by autograd-vs-closed-form and special cases: parity unpinned.
+pinned only by autograd-vs-closed-form and special cases: parity unpinned.  The same holds for
+stage_forward_indexed with context lengths (the reference's only statement of it is a Triton kernel
+that cannot run here and that leaves rows past the length undefined): it is pinned by reduction to the
+pinned stage_forward (full lengths, stride table) and by literal loops on the cut group, but its
+pass-through of dead rows is this build's choice: parity unpinned.
 """
 import math
 
@@ -328,6 +334,89 @@ def net_autograd(x, xa, weights, dy, dya, alpha, n, C, m=M_DEFAULT, activation=A
     yi, ya = net_forward(x, xa, ws, alpha, n, C, m, activation, first_stage)
     torch.autograd.backward([yi, ya], [dy, dya])
     return yi.detach(), ya.detach(), x.grad, xa.grad, [w.grad for w in ws]
+
+
+# ----------------------------------------------------------------------------------------------
+# grouping by table and per-batch context lengths (ncn_triton/ncn_triton_old.py, group_tensors.py)
+# ----------------------------------------------------------------------------------------------
+def stride_group_table(N, n, stage):
+    """The stride permutation written as a table: entry g*n + o is the position of slot o of group g."""
+    return stage_positions(N, n, stage).reshape(-1)
+
+
+def radix_group_table(N, n, level):
+    """Radix-n digit grouping of ncn_triton/group_tensors.py:8-18: position i belongs to the group numbered
+    lower + upper * n^level, where lower = i mod n^level and upper = i div n^(level+1), and sits in slot
+    (i div n^level) mod n: a group holds the n positions that differ only in digit `level`."""
+    stride = n ** level
+    if N % (n * stride) != 0:
+        raise ValueError("n^(level+1) must divide N")
+    table = torch.empty(N, dtype=torch.long)
+    for i in range(N):
+        lower = i % stride
+        slot = (i // stride) % n
+        upper = i // (n * stride)
+        table[(lower + upper * stride) * n + slot] = i
+    return table
+
+
+def stage_forward_indexed(X, Xa, W, alpha, n, C, table, ctx_len=None, m=M_DEFAULT, activation=ACT_TANH, inverse=False):
+    """One stage whose groups come from `table` ([N] positions in (group, slot) order) and where batch entry b only
+    has its first ctx_len[b] slots (ncn_triton_old.py:66-71, 93-96): whole groups below the length run as usual, the
+    group the length cuts runs on its live rows with as many steps as it has live rows, rows past the length pass
+    through.  Differentiable; inverse=True runs the inverse instead."""
+    code = act_code(activation)
+    B, N, E = X.shape
+    Wi, Wj = _split_w(W, C)
+    table = torch.as_tensor(table, dtype=torch.long)
+    ys, yas = [], []
+    for b in range(B):
+        ln = N if ctx_len is None else max(0, min(int(ctx_len[b]), N))
+        y, ya = X[b:b + 1].clone(), Xa[b:b + 1].clone()
+        full, rem = ln // n, ln % n
+        pieces = []
+        if full:
+            pieces.append(table[:full * n].reshape(full, n))
+        if rem:
+            pieces.append(table[full * n:full * n + rem].reshape(1, rem))
+        for pos in pieces:
+            rows = pos.shape[1]
+            x, a = _gather(X[b:b + 1], pos, C), _gather(Xa[b:b + 1], pos, C)
+            steps = range(rows - 1, -1, -1) if inverse else range(rows)
+            for j in steps:
+                if inverse:
+                    x, a, _ = _unstep(x, a, Wi, Wj, j, alpha, m, code)
+                else:
+                    x, a, _ = _step(x, a, Wi, Wj, j, alpha, m, code)
+            flat = pos.reshape(-1)
+            y = y.index_copy(1, flat, x.permute(0, 2, 3, 1, 4).reshape(1, flat.numel(), E))
+            ya = ya.index_copy(1, flat, a.permute(0, 2, 3, 1, 4).reshape(1, flat.numel(), E))
+        ys.append(y)
+        yas.append(ya)
+    return torch.cat(ys), torch.cat(yas)
+
+
+def net_forward_indexed(x, xa, weights, alpha, n, C, tables, ctx_len=None, m=M_DEFAULT, activation=ACT_TANH):
+    for W, table in zip(weights, tables):
+        x, xa = stage_forward_indexed(x, xa, W, alpha, n, C, table, ctx_len, m, activation)
+    return x, xa
+
+
+def net_inverse_indexed(y, ya, weights, alpha, n, C, tables, ctx_len=None, m=M_DEFAULT, activation=ACT_TANH):
+    for W, table in zip(reversed(weights), reversed(tables)):
+        y, ya = stage_forward_indexed(y, ya, W, alpha, n, C, table, ctx_len, m, activation, inverse=True)
+    return y, ya
+
+
+def net_autograd_indexed(x, xa, weights, dy, dya, alpha, n, C, tables, ctx_len=None, m=M_DEFAULT,
+                         activation=ACT_TANH):
+    """Forward + autograd backward through net_forward_indexed.  Returns yi, ya, dx, dxa, [dW_l]."""
+    x = x.detach().clone().requires_grad_()
+    xa = xa.detach().clone().requires_grad_()
+    ws = [w.detach().clone().requires_grad_() for w in weights]
+    yi, ya = net_forward_indexed(x, xa, ws, alpha, n, C, tables, ctx_len, m, activation)
+    torch.autograd.backward([yi, ya], [dy, dya])
+    return yi.detach(), ya.detach(), x.grad, xa.grad, [w.grad if w.grad is not None else torch.zeros_like(w) for w in ws]
 
 
 # ----------------------------------------------------------------------------------------------
