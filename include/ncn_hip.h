@@ -148,7 +148,7 @@ int ncn_inverse(const void* y, const void* ya, int in_dtype,
  *                 order of the table): groups wholly below the length run as usual; the group the length cuts runs
  *                 on its live rows only, with as many steps as it has live rows; rows past the length pass through
  *                 (forward, inverse: out = in; backward: dx = dy, dxa = dya, x_rec = y, no share in dW).  Values are
- *                 clamped to [0, N].  Needs a head width <= 64 (NCN_ERR_UNSUPPORTED otherwise).
+ *                 clamped to [0, N].
  * Everything else as in ncn_forward / ncn_backward / ncn_inverse, except that these always run stage by stage (no
  * multi-stage passes, so forward takes no workspace) and ncn_backward_indexed needs ncn_workspace_bytes(shape).
  */

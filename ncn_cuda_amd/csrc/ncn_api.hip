@@ -124,8 +124,7 @@ struct Grouping {
 
 int check_grouping(const Grouping& g, const ncn_shape* sh) {
     if ((reinterpret_cast<uintptr_t>(g.table) & 3u) || (reinterpret_cast<uintptr_t>(g.ctx_len) & 3u)) return NCN_ERR_ALIGN;
-    // the partly live group of a batch entry runs on the generic kernel
-    if (g.ctx_len && sh->E / sh->n_head > kGenericMaxHeadDim) return NCN_ERR_UNSUPPORTED;
+    (void)sh;
     return NCN_OK;
 }
 
@@ -148,17 +147,21 @@ void fill_common(StageArgs& a, const ncn_shape* sh, const Plan& p, int stage, fl
     fill_step_table(a.tab, sh->n_cache, alpha, m, activation);
 }
 
-// With context lengths: the partly live group of every batch entry (generic kernel, one tile per batch entry),
-// then the rows past the lengths.  `a` is the stage's argument block as the main launch used it.
-hipError_t launch_ragged_rest(Pass pass, StageArgs a, const ncn_shape* sh, int partial_rows_used, hipStream_t s) {
-    StageArgs e = a;
-    e.edge = 1;
-    e.total_tiles = (uint32_t)sh->batch;
-    e.tiles_per_inst = 1;
-    if (pass == kBackward) e.dw_partials = a.dw_partials + (int64_t)partial_rows_used * 2 * sh->E;
-    const int grid = (int)(sh->batch < kEdgeGridX ? sh->batch : kEdgeGridX);
-    hipError_t err = launch_generic(pass, e, sh->n_head, grid, s);
-    if (err != hipSuccess) return err;
+// With context lengths, after the main launch: the rows past the lengths pass through.  The register kernels run
+// the group a length cuts themselves (masked steps); the generic kernel leaves it to a second launch of its own,
+// one tile per batch entry.  `a` is the stage's argument block as the main launch used it.
+hipError_t launch_ragged_rest(Pass pass, StageArgs a, const ncn_shape* sh, int path, int partial_rows_used,
+                              hipStream_t s) {
+    if (path != 2) {
+        StageArgs e = a;
+        e.edge = 1;
+        e.total_tiles = (uint32_t)sh->batch;
+        e.tiles_per_inst = 1;
+        if (pass == kBackward) e.dw_partials = a.dw_partials + (int64_t)partial_rows_used * 2 * sh->E;
+        const int grid = (int)(sh->batch < kEdgeGridX ? sh->batch : kEdgeGridX);
+        hipError_t err = launch_generic(pass, e, sh->n_head, grid, s);
+        if (err != hipSuccess) return err;
+    }
     return launch_pass_through(pass, a, sh->batch, s);
 }
 int edge_rows(const ncn_shape* sh) { return (int)(sh->batch < kEdgeGridX ? sh->batch : kEdgeGridX); }
@@ -187,7 +190,7 @@ size_t temp_bytes(const ncn_shape* sh, bool backward) {
 
 extern "C" {
 
-const char* ncn_version(void) { return "0.2"; }
+const char* ncn_version(void) { return "0.3"; }
 
 int ncn_plan_passes(const ncn_shape* shape, int first_stage, int n_stages, int activation, int backward, int32_t* out,
                     int max_passes) {
@@ -328,7 +331,7 @@ static int forward_impl(const void* x, const void* xa, int in_dtype, void* y, vo
         hipError_t err = (p.path != 2)      ? launch_generic(kForward, a, shape->n_head, p.grid_fwd, s)
                          : grouping.plain() ? launch_fast_forward(kForward, a, shape->n_head, p.grid_fwd, s)
                                             : launch_fast_forward_indexed(kForward, a, shape->n_head, p.grid_fwd, s);
-        if (err == hipSuccess && grouping.ctx_len) err = launch_ragged_rest(kForward, a, shape, 0, s);
+        if (err == hipSuccess && grouping.ctx_len) err = launch_ragged_rest(kForward, a, shape, p.path, 0, s);
         if (err != hipSuccess) return (int)err;
     }
     return NCN_OK;
@@ -360,7 +363,7 @@ static int inverse_impl(const void* y, const void* ya, int in_dtype, void* x, vo
         hipError_t err = (p.path != 2)      ? launch_generic(kInverse, a, shape->n_head, p.grid_fwd, s)
                          : grouping.plain() ? launch_fast_forward(kInverse, a, shape->n_head, p.grid_fwd, s)
                                             : launch_fast_forward_indexed(kInverse, a, shape->n_head, p.grid_fwd, s);
-        if (err == hipSuccess && grouping.ctx_len) err = launch_ragged_rest(kInverse, a, shape, 0, s);
+        if (err == hipSuccess && grouping.ctx_len) err = launch_ragged_rest(kInverse, a, shape, p.path, 0, s);
         if (err != hipSuccess) return (int)err;
     }
     return NCN_OK;
@@ -382,7 +385,8 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
     if (!aligned16(y) || !aligned16(ya) || !aligned16(dy) || !aligned16(dya) || !aligned16(dx) || !aligned16(dxa) ||
         !aligned16(x_rec) || !aligned16(xa_rec) || !aligned16(W) || !aligned16(dW) || !aligned16(workspace))
         return NCN_ERR_ALIGN;
-    const int extra_rows = grouping.ctx_len ? edge_rows(shape) : 0;  // partial rows of the edge launch
+    // partial rows of the generic kernel's second launch
+    const int extra_rows = (grouping.ctx_len && kernel_path(shape, activation) != 2) ? edge_rows(shape) : 0;
     const Plan p = make_plan(shape, activation, extra_rows);
     hipStream_t s = static_cast<hipStream_t>(stream);
     float* partials = static_cast<float*>(workspace);
@@ -470,7 +474,7 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
         hipError_t err = (p.path != 2)      ? launch_generic(kBackward, a, shape->n_head, p.grid_x, s)
                          : grouping.plain() ? launch_fast_backward(a, shape->n_head, p.grid_x, s)
                                             : launch_fast_backward_indexed(a, shape->n_head, p.grid_x, s);
-        if (err == hipSuccess && grouping.ctx_len) err = launch_ragged_rest(kBackward, a, shape, p.partial_rows, s);
+        if (err == hipSuccess && grouping.ctx_len) err = launch_ragged_rest(kBackward, a, shape, p.path, p.partial_rows, s);
         if (err != hipSuccess) return (int)err;
         err = launch_reduce_dw(partials, p.partial_rows + extra_rows, wstride, wstride, level1, dW + k * wstride, s);
         if (err != hipSuccess) return (int)err;

@@ -208,13 +208,13 @@ __global__ void __launch_bounds__(256) reduce_rows_kernel(const float* __restric
 
 // Rows past a batch entry's context length take no part in the stage: they pass through.
 //   forward / inverse: out = in (and the float32 copies)     backward: dx = dy, dxa = dya (0 when null), x_rec = y.
-// One wavefront per slot k = 0 .. N-1 of a batch entry, in group order.
-__global__ void __launch_bounds__(256) pass_through_kernel(const StageArgs A, const int backward, const int64_t slots) {
+// Block (x, y) walks the dead slots live .. N-1 of batch entries y, y + gridDim.y, .., one wavefront per slot.
+__global__ void __launch_bounds__(256) pass_through_kernel(const StageArgs A, const int backward, const int64_t batch) {
     const int lane = threadIdx.x & 63;
-    for (int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); r < slots; r += (int64_t)gridDim.x * 4) {
-        const uint32_t b = (uint32_t)(r / A.N);
-        const int64_t k = r - (int64_t)b * A.N;
-        if (k < live_slots(A, b)) continue;
+    for (int64_t bb = blockIdx.y; bb < batch; bb += gridDim.y)
+    for (int64_t k = live_slots(A, (uint32_t)bb) + (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); k < A.N;
+         k += (int64_t)gridDim.x * 4) {
+        const uint32_t b = (uint32_t)bb;
         const int64_t pos = slot_position(A, (uint32_t)(k / A.n_cache), (uint32_t)(k % A.n_cache));
         const int64_t off = ((int64_t)b * A.N + pos) * A.E;
         for (int64_t e = lane; e < A.E; e += 64) {
@@ -237,10 +237,10 @@ __global__ void __launch_bounds__(256) pass_through_kernel(const StageArgs A, co
 }  // namespace
 
 hipError_t launch_pass_through(Pass pass, const StageArgs& a, int64_t batch, hipStream_t s) {
-    const int64_t slots = batch * a.N;
-    const int64_t blocks = (slots + 3) / 4;
-    const unsigned grid = (unsigned)(blocks < 65536 ? blocks : 65536);
-    hipLaunchKernelGGL(pass_through_kernel, dim3(grid), dim3(256), 0, s, a, pass == kBackward ? 1 : 0, slots);
+    const int64_t per_entry = (a.N + 3) / 4;
+    const unsigned gx = (unsigned)(per_entry < 64 ? per_entry : 64);
+    const unsigned gy = (unsigned)(batch < 1024 ? batch : 1024);
+    hipLaunchKernelGGL(pass_through_kernel, dim3(gx, gy), dim3(256), 0, s, a, pass == kBackward ? 1 : 0, batch);
     return hipGetLastError();
 }
 

@@ -44,11 +44,12 @@ struct Tile {
     static constexpr int RLMASK = (LR - 1) * LF;
 };
 
-// Element offsets of this lane's R row fragments for wave tile `t`; false when the lane's group is past the end.
-// INDEXED builds read the grouping table and the context lengths when the launch has them; the plain builds only
-// know the stride permutation (and are what every launch without table and lengths uses).
+// Element offsets of this lane's R row fragments for wave tile `t`; returns the live rows of the lane's group:
+// NC, or 0 when the group is past the end.  INDEXED builds read the grouping table and the context lengths when
+// the launch has them (a group that a length cuts has 0 < live < NC); the plain builds only know the stride
+// permutation (and are what every launch without table and lengths uses).
 template <int NC, int EC, int R, int F, bool INDEXED>
-__device__ __forceinline__ bool tile_offsets(const StageArgs& A, uint32_t t, int lane, int head, int64_t (&off)[R]) {
+__device__ __forceinline__ int tile_offsets(const StageArgs& A, uint32_t t, int lane, int head, int64_t (&off)[R]) {
     using T = Tile<NC, EC, R, F>;
     const int fl = lane % T::LF;
     const int rl = (lane / T::LF) % T::LR;
@@ -56,8 +57,8 @@ __device__ __forceinline__ bool tile_offsets(const StageArgs& A, uint32_t t, int
     const uint32_t b = t / A.tiles_per_inst;
     const uint32_t tile = t - b * A.tiles_per_inst;
     const uint32_t group = tile * T::GPW + gw;
-    bool valid = group < A.groups;
-    if (INDEXED) valid = valid && live_rows(A, b, group) == NC;  // partly live groups: generic kernel
+    const bool valid = group < A.groups;
+    const int live = !valid ? 0 : (INDEXED ? live_rows(A, b, group) : NC);
     const int64_t base = (int64_t)b * A.N * A.E + (int64_t)head * EC + fl * F;
 #pragma unroll
     for (int rr = 0; rr < R; ++rr) {
@@ -66,7 +67,7 @@ __device__ __forceinline__ bool tile_offsets(const StageArgs& A, uint32_t t, int
                                     : (int64_t)stage_block(A, valid ? group : 0u, i) * NC + i;
         off[rr] = base + pos * A.E;
     }
-    return valid;
+    return live;
 }
 
 template <int F>
@@ -128,16 +129,20 @@ __device__ __forceinline__ float dot_frag(const float (&a)[F], const float (&b)[
 // ---------------------------------------------------------------------------------------------
 // forward_core runs the n_cache steps of one stage on registers that already hold x / m^t0, xa / m^t0 with
 // t0 = step_base steps done before (several stages in a row just keep counting) and leaves them scaled.
-template <int NC, int EC, int R, int F, bool TANH_ONLY = true>
+// STEP_MASK builds take `live`, the live rows of the lane's group, and skip steps j >= live with the lanes of that
+// group switched off (a group that a context length cuts runs one step per live row,
+// ncn_triton/ncn_triton_old.py:93-96).  Every cross-lane exchange of a step stays inside one group.
+template <int NC, int EC, int R, int F, bool TANH_ONLY = true, bool STEP_MASK = false>
 __device__ __forceinline__ void forward_core(float (&x)[R][F], float (&a)[R][F], const float (&wi)[F],
                                              const float (&wj)[F], const StepTable& S, int step_base, int lane,
-                                             float4* slots) {
+                                             float4* slots, int live = NC) {
     using T = Tile<NC, EC, R, F>;
     const float om = 1.0f - S.m;
 #pragma unroll 1
     for (int jo = 0; jo < T::LR; ++jo) {
 #pragma unroll
         for (int jr = 0; jr < R; ++jr) {
+            if (STEP_MASK && jo * R + jr >= live) continue;  // the lanes of a group agree: no lane it needs is off
             const int ts = step_base + jo * R + jr;   // steps done so far
             const float lam = S.step[ts].flam;     // z = lam X_i + c_i Xj
             const float kc = S.step[ts].fkc;       // c_i = kc S_i
@@ -165,11 +170,20 @@ __device__ __forceinline__ void forward_core(float (&x)[R][F], float (&a)[R][F],
 }
 
 // one stage from true values to true values
-template <int NC, int EC, int R, int F, bool TANH_ONLY>
+// m^k by repeated multiplication (k <= 64; only groups cut by a context length come here)
+__device__ __forceinline__ float pow_steps(float base, int k) {
+    float p = 1.0f;
+    for (int i = 0; i < k; ++i) p *= base;
+    return p;
+}
+
+template <int NC, int EC, int R, int F, bool TANH_ONLY, bool STEP_MASK = false>
 __device__ __forceinline__ void forward_steps(float (&x)[R][F], float (&a)[R][F], const float (&wi)[F],
-                                              const float (&wj)[F], const StepTable& S, int lane, float4* slots) {
-    forward_core<NC, EC, R, F, TANH_ONLY>(x, a, wi, wj, S, 0, lane, slots);
-    const float dn = S.m_pow_n;
+                                              const float (&wj)[F], const StepTable& S, int lane, float4* slots,
+                                              int live = NC) {
+    forward_core<NC, EC, R, F, TANH_ONLY, STEP_MASK>(x, a, wi, wj, S, 0, lane, slots, live);
+    // `live` steps were done: the registers hold x / m^live
+    const float dn = (!STEP_MASK || live == NC) ? S.m_pow_n : pow_steps(S.m, live);
 #pragma unroll
     for (int rr = 0; rr < R; ++rr)
 #pragma unroll
@@ -184,15 +198,30 @@ __device__ __forceinline__ void forward_steps(float (&x)[R][F], float (&a)[R][F]
 //   x = (y - (1-m) b)/m       recompute r from x        a = (b - (1-m) F)/m
 // with the same m^t scaling of the registers as the backward below (Y = m^t x, B = m^t xa).
 // ---------------------------------------------------------------------------------------------
-template <int NC, int EC, int R, int F, bool TANH_ONLY>
+// STEP_MASK: a group with `live` < NC live rows only undoes its steps live-1 .. 0.  The skipped steps come first in
+// the loop, so the registers are first scaled as if they had been done (m^(NC-live)): every later step then
+// finds the scaling its table entry assumes, and the final factor is the same for all groups.
+template <int NC, int EC, int R, int F, bool TANH_ONLY, bool STEP_MASK = false>
 __device__ __forceinline__ void inverse_steps(float (&y)[R][F], float (&b)[R][F], const float (&wi)[F],
-                                              const float (&wj)[F], const StepTable& S, int lane, float4* slots) {
+                                              const float (&wj)[F], const StepTable& S, int lane, float4* slots,
+                                              int live = NC) {
     using T = Tile<NC, EC, R, F>;
     const float nom = S.m - 1.0f;
+    if (STEP_MASK && live != NC) {
+        const float sc = pow_steps(S.m, NC - live);
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr)
+#pragma unroll
+            for (int f = 0; f < F; ++f) {
+                y[rr][f] *= sc;
+                b[rr][f] *= sc;
+            }
+    }
 #pragma unroll 1
     for (int jo = T::LR - 1; jo >= 0; --jo) {
 #pragma unroll
         for (int jr = R - 1; jr >= 0; --jr) {
+            if (STEP_MASK && jo * R + jr >= live) continue;
             const int ts = (T::LR - 1 - jo) * R + (R - 1 - jr);   // inversion steps done so far
             const float lam = S.step[ts].lam, kc2 = S.step[ts].kc2, kap = S.step[ts].kap;
 #pragma unroll
@@ -248,11 +277,12 @@ __device__ __forceinline__ void inverse_steps(float (&y)[R][F], float (&b)[R][F]
 // ---------------------------------------------------------------------------------------------
 // backward_core: the n_cache steps of one stage on registers in the scaled form above with t0 = step_base
 // inversion steps done before (P holds p / m^t0, not h); leaves them scaled by t0 + n_cache steps.
-template <int NC, int EC, int R, int F, bool MASKED, bool TANH_ONLY = true>
+// STEP_MASK: steps j >= live leave the registers as they are (see inverse_steps for the scaling).
+template <int NC, int EC, int R, int F, bool MASKED, bool TANH_ONLY = true, bool STEP_MASK = false>
 __device__ __forceinline__ void backward_core(float (&Y)[R][F], float (&B)[R][F], float (&G)[R][F], float (&P)[R][F],
                                               const float (&wi)[F], const float (&wj)[F], float (&dwi)[F],
                                               float (&dwj)[F], float own, const StepTable& S, int step_base, int lane,
-                                              float4* slots) {
+                                              float4* slots, int live = NC) {
     using T = Tile<NC, EC, R, F>;
     const int rl = (lane / T::LF) % T::LR;
     const float om = 1.0f - S.m;
@@ -263,6 +293,7 @@ __device__ __forceinline__ void backward_core(float (&Y)[R][F], float (&B)[R][F]
         const float sel = (T::LR == 1 || rl == jo) ? 1.0f : 0.0f;  // this lane holds the pivot row
 #pragma unroll
         for (int jr = R - 1; jr >= 0; --jr) {
+            if (STEP_MASK && jo * R + jr >= live) continue;  // lanes of a group agree: no lane it needs is off
             const int ts = step_base + (T::LR - 1 - jo) * R + (R - 1 - jr);   // inversion steps done so far
             const float lam = S.step[ts].lam;     // z = lam Y_i + chat_i Yj
             const float kc2 = S.step[ts].kc2;     // chat_i = kc2 S_i
@@ -320,18 +351,32 @@ __device__ __forceinline__ void backward_core(float (&Y)[R][F], float (&B)[R][F]
 }
 
 // one stage: G, H true gradients in and out; Y, B true outputs in, m^n_cache times the stage inputs out
-template <int NC, int EC, int R, int F, bool MASKED, bool TANH_ONLY>
+template <int NC, int EC, int R, int F, bool MASKED, bool TANH_ONLY, bool STEP_MASK = false>
 __device__ __forceinline__ void backward_steps(float (&Y)[R][F], float (&B)[R][F], float (&G)[R][F], float (&P)[R][F],
                                                const float (&wi)[F], const float (&wj)[F], float (&dwi)[F],
                                                float (&dwj)[F], float own, const StepTable& S, int lane,
-                                               float4* slots) {
+                                               float4* slots, int live = NC) {
     const float om = 1.0f - S.m;
     const float nom = -om;
 #pragma unroll
     for (int rr = 0; rr < R; ++rr)
 #pragma unroll
         for (int f = 0; f < F; ++f) P[rr][f] = fmaf(om, G[rr][f], P[rr][f]);  // h -> p
-    backward_core<NC, EC, R, F, MASKED, TANH_ONLY>(Y, B, G, P, wi, wj, dwi, dwj, own, S, 0, lane, slots);
+    if (STEP_MASK && live != NC) {
+        // as if the NC - live skipped steps had been done: Y, B carry m^t, G, P carry m^-t
+        const float sc = pow_steps(S.m, NC - live), isc = pow_steps(1.0f / S.m, NC - live);
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr)
+#pragma unroll
+            for (int f = 0; f < F; ++f) {
+                Y[rr][f] *= sc;
+                B[rr][f] *= sc;
+                G[rr][f] *= isc;
+                P[rr][f] *= isc;
+            }
+    }
+    backward_core<NC, EC, R, F, MASKED, TANH_ONLY, STEP_MASK>(Y, B, G, P, wi, wj, dwi, dwj, own, S, 0, lane, slots,
+                                                             live);
     // undo the scaling of the gradients: NC steps done
     const float dn = S.m_pow_n;       // m^NC
 #pragma unroll
@@ -360,21 +405,26 @@ __device__ __forceinline__ void backward_steps(float (&Y)[R][F], float (&B)[R][F
     float wi[F], wj[F];                                                                         \
     load_w<F>(A.W, A.E, head, EC, fl, wi, wj);
 
+// Row rr of this lane is live when its slot is below the group's live rows (always, or never, without lengths).
+#define NCN_ROW_LIVE(rr) ((int)(((lane / T::LF) % T::LR) * R + (rr)) < live)
+
 template <int NC, int EC, int R, int F, bool TANH_ONLY = true, bool INDEXED = false>
 __global__ void __launch_bounds__(kBlockThreads) stage_forward_kernel(const StageArgs A) {
     NCN_WAVE_PROLOGUE
     for (uint32_t t = gwave / A.n_head; t < A.total_tiles; t += tile_step) {
         int64_t off[R];
-        const bool valid = tile_offsets<NC, EC, R, F, INDEXED>(A, t, lane, head, off);
+        const int live = tile_offsets<NC, EC, R, F, INDEXED>(A, t, lane, head, off);
         float x[R][F], a[R][F];
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) {
+            const bool valid = INDEXED ? NCN_ROW_LIVE(rr) : live != 0;
             load_frag<F>(A.in0, A.in_dtype, off[rr], valid, x[rr]);
             load_frag<F>(A.in1, A.in_dtype, off[rr], valid, a[rr]);
         }
-        forward_steps<NC, EC, R, F, TANH_ONLY>(x, a, wi, wj, A.tab, lane, slots);
+        forward_steps<NC, EC, R, F, TANH_ONLY, INDEXED>(x, a, wi, wj, A.tab, lane, slots, live);
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) {
+            const bool valid = INDEXED ? NCN_ROW_LIVE(rr) : live != 0;
             store_frag<F>(A.out0, A.out_dtype, off[rr], valid, x[rr]);
             store_frag<F>(A.out1, A.out_dtype, off[rr], valid, a[rr]);
             if (A.aux0) {
@@ -390,16 +440,18 @@ __global__ void __launch_bounds__(kBlockThreads) stage_inverse_kernel(const Stag
     NCN_WAVE_PROLOGUE
     for (uint32_t t = gwave / A.n_head; t < A.total_tiles; t += tile_step) {
         int64_t off[R];
-        const bool valid = tile_offsets<NC, EC, R, F, INDEXED>(A, t, lane, head, off);
+        const int live = tile_offsets<NC, EC, R, F, INDEXED>(A, t, lane, head, off);
         float y[R][F], b[R][F];
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) {
+            const bool valid = INDEXED ? NCN_ROW_LIVE(rr) : live != 0;
             load_frag<F>(A.in0, A.in_dtype, off[rr], valid, y[rr]);
             load_frag<F>(A.in1, A.in_dtype, off[rr], valid, b[rr]);
         }
-        inverse_steps<NC, EC, R, F, TANH_ONLY>(y, b, wi, wj, A.tab, lane, slots);
+        inverse_steps<NC, EC, R, F, TANH_ONLY, INDEXED>(y, b, wi, wj, A.tab, lane, slots, live);
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) {
+            const bool valid = INDEXED ? NCN_ROW_LIVE(rr) : live != 0;
             store_frag<F>(A.out0, A.out_dtype, off[rr], valid, y[rr]);
             store_frag<F>(A.out1, A.out_dtype, off[rr], valid, b[rr]);
         }
@@ -407,7 +459,8 @@ __global__ void __launch_bounds__(kBlockThreads) stage_inverse_kernel(const Stag
 }
 
 // Tiles of up to 16 elements per lane fit 128 VGPRs (4 waves per SIMD) when the compiler is asked to; measured 3-4 %
-// faster than the 136 it picks by itself.  Larger tiles and the multi-activation build would spill, so they are left alone.
+// faster than the 136 it picks by itself.  Larger tiles, the multi-activation build and the builds that mask steps
+// would spill, so they are left alone.
 template <int NC, int EC, int R, int F, bool TANH_ONLY = true, bool INDEXED = false>
 __global__ void __launch_bounds__(kBlockThreads, (TANH_ONLY && R * F <= 16 && F == 4) ? 4 : 1) stage_backward_kernel(const StageArgs A) {
     NCN_WAVE_PROLOGUE
@@ -417,18 +470,21 @@ __global__ void __launch_bounds__(kBlockThreads, (TANH_ONLY && R * F <= 16 && F 
 
     for (uint32_t t = gwave / A.n_head; t < A.total_tiles; t += tile_step) {
         int64_t off[R];
-        const bool valid = tile_offsets<NC, EC, R, F, INDEXED>(A, t, lane, head, off);
+        const int live = tile_offsets<NC, EC, R, F, INDEXED>(A, t, lane, head, off);
         float Y[R][F], B[R][F], G[R][F], H[R][F];
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) {
+            const bool valid = INDEXED ? NCN_ROW_LIVE(rr) : live != 0;
             load_frag<F>(A.in0, A.in_dtype, off[rr], valid, Y[rr]);
             load_frag<F>(A.in1, A.in_dtype, off[rr], valid, B[rr]);
             load_frag<F>(A.g0, A.g_dtype, off[rr], valid, G[rr]);
             load_frag<F>(A.g1, A.g_dtype, off[rr], valid && A.g1 != nullptr, H[rr]);
         }
-        backward_steps<NC, EC, R, F, false, TANH_ONLY>(Y, B, G, H, wi, wj, dwi, dwj, 1.0f, A.tab, lane, slots);
+        backward_steps<NC, EC, R, F, false, TANH_ONLY, INDEXED>(Y, B, G, H, wi, wj, dwi, dwj, 1.0f, A.tab, lane, slots,
+                                                               live);
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) {
+            const bool valid = INDEXED ? NCN_ROW_LIVE(rr) : live != 0;
             store_frag<F>(A.out0, A.out_dtype, off[rr], valid, G[rr]);
             store_frag<F>(A.out1, A.out_dtype, off[rr], valid, H[rr]);
             if (A.aux0) {
@@ -458,6 +514,7 @@ __global__ void __launch_bounds__(kBlockThreads, (TANH_ONLY && R * F <= 16 && F 
         }
     }
 }
+#undef NCN_ROW_LIVE
 #undef NCN_WAVE_PROLOGUE
 
 }  // namespace ncn

@@ -59,19 +59,24 @@ def _run_gpu(M, x, xa, Ws, dy, dya, alpha, n, C, tables, lens, act=0, one_call=F
     return outs[-1][0], outs[-1][1], xr, xar, g, h, dWs
 
 
-def _check(got, ref, x, xa, tol=TOL):
+def _check(got, ref, x, xa, tol=TOL, n=4):
+    """Forward at `tol`; what goes through the inversion is allowed its rounding growth (1/m)^n per stage."""
     y, ya, xr, xar, dx, dxa, dWs = got
     ryi, rya, rdx, rdxa, rdWs = ref
     assert O.rel_err(y, ryi) < tol and O.rel_err(ya, rya) < tol
-    assert O.rel_err(dx, rdx) < tol and O.rel_err(dxa, rdxa) < tol
+    gtol = max(tol, 1e-6 * (1 / 0.9) ** n)
+    assert O.rel_err(dx, rdx) < gtol and O.rel_err(dxa, rdxa) < gtol
     for a, b in zip(dWs, rdWs):
-        assert O.rel_err(a, b) < tol
+        assert O.rel_err(a, b) < gtol
     if xr is not None:
-        assert O.rel_err(xr, x) < 3e-5 and O.rel_err(xar, xa) < 3e-5
+        rtol = max(3e-5, 3e-6 * (1 / 0.9) ** n)
+        assert O.rel_err(xr, x) < rtol and O.rel_err(xar, xa) < rtol
 
 
-SHAPES = [(3, 64, 32, 2, 4, 3), (2, 256, 128, 4, 16, 2), (3, 36, 20, 2, 3, 3), (5, 128, 64, 2, 8, 2)]
-IDS = ["register_n4_Ec16", "register_n16_Ec32", "generic_n3_Ec10", "register_n8_Ec32"]
+SHAPES = [(3, 64, 32, 2, 4, 3), (2, 256, 128, 4, 16, 2), (3, 36, 20, 2, 3, 3), (5, 128, 64, 2, 8, 2),
+          (2, 64, 256, 2, 8, 2), (2, 128, 8, 2, 32, 1)]
+IDS = ["register_n4_Ec16", "register_n16_Ec32", "generic_n3_Ec10", "register_n8_Ec32", "register_n8_Ec128",
+       "register_n32_Ec4"]
 
 
 @pytest.mark.parametrize("kind", ["stride", "radix", "random"])
@@ -82,7 +87,7 @@ def test_table_grouping_vs_oracle(M, shape, kind):
     tables = _tables(kind, N, n, L)
     d = torch.float64
     ref = O.net_autograd_indexed(x.to(d), xa.to(d), [w.to(d) for w in Ws], dy.to(d), dya.to(d), 0.9, n, C, tables)
-    _check(_run_gpu(M, x, xa, Ws, dy, dya, 0.9, n, C, tables, None), ref, x, xa)
+    _check(_run_gpu(M, x, xa, Ws, dy, dya, 0.9, n, C, tables, None), ref, x, xa, n=n)
 
 
 @pytest.mark.parametrize("shape", SHAPES[:2], ids=IDS[:2])
@@ -119,7 +124,7 @@ def test_context_lengths_vs_oracle(M, shape, kind, one_call):
     ref = O.net_autograd_indexed(x.to(d), xa.to(d), [w.to(d) for w in Ws], dy.to(d), dya.to(d), 0.9, n, C, tables,
                                  lens)
     got = _run_gpu(M, x, xa, Ws, dy, dya, 0.9, n, C, tables, lens, one_call=one_call)
-    _check(got, ref, x, xa, tol=TOL if not one_call else 3e-5)
+    _check(got, ref, x, xa, tol=TOL if not one_call else 3e-5, n=n)
 
 
 def test_context_lengths_without_table_and_inverse(M):
