@@ -30,6 +30,7 @@
 namespace ncn {
 
 constexpr int kFusedMaxStages = 8;
+constexpr size_t kFusedStateBytes = 64 * 1024;  // LDS for the row arrays of one workgroup (2 forward, 4 backward)
 constexpr int kFusedWavesFwd = 8;   // (16 waves per workgroup measured slower: all waves of a workgroup share its phases)
 constexpr int kFusedWavesBwd = 8;   // backward runs at 128 VGPRs: 4 waves per SIMD in all
 
@@ -139,6 +140,63 @@ __device__ __forceinline__ void fused_load_rows(const FusedArgs& A, const FusedI
     }
 }
 
+// Window rows on their way from global memory to LDS: 4 features per thread and trip, kept as raw bits so that
+// nothing waits for the loads until fused_commit_rows turns them into floats.  A workgroup fetches the window of
+// its next item while it computes the current one.
+template <int NC, int EC, int NW, int K>
+__device__ __forceinline__ void fused_window_offsets(const FusedArgs& A, const FusedItem& it, uint32_t rows,
+                                                     int64_t (&off)[K]) {
+    constexpr uint32_t CPR = EC / 4;
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        // a trip past the end re-reads the last chunk, which fused_commit_rows ignores
+        const uint32_t c = min(threadIdx.x + k * 64 * NW, rows * CPR - 1u);
+        const uint32_t lr = c / CPR, c4 = c - lr * CPR;
+        off[k] = fused_row_offset<NC>(A, it, lr) + c4 * 4;
+    }
+}
+
+// one wave-uniform branch around straight runs of loads: nothing between the loads makes one wait for another
+template <int K>
+__device__ __forceinline__ void fused_fetch_rows(const void* src, int dtype, const int64_t (&off)[K], uint4 (&raw)[K]) {
+    if (!src) {
+#pragma unroll
+        for (int k = 0; k < K; ++k) raw[k] = make_uint4(0u, 0u, 0u, 0u);
+    } else if (dtype == NCN_F32) {
+#pragma unroll
+        for (int k = 0; k < K; ++k) raw[k] = *reinterpret_cast<const uint4*>(static_cast<const float*>(src) + off[k]);
+    } else {
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            const uint2 t = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(src) + off[k]);
+            raw[k] = make_uint4(t.x, t.y, 0u, 0u);
+        }
+    }
+}
+
+__device__ __forceinline__ void fused_raw_to_float(const uint4& r, int dtype, float (&v)[4]) {
+    if (dtype == NCN_F32) {
+        v[0] = __uint_as_float(r.x); v[1] = __uint_as_float(r.y); v[2] = __uint_as_float(r.z); v[3] = __uint_as_float(r.w);
+    } else {
+        v[0] = bf16_to_f32(r.x & 0xffffu); v[1] = bf16_to_f32(r.x >> 16);
+        v[2] = bf16_to_f32(r.y & 0xffffu); v[3] = bf16_to_f32(r.y >> 16);
+    }
+}
+
+template <int EC, int NW, int K>
+__device__ __forceinline__ void fused_commit_rows(const uint4 (&raw)[K], int dtype, float* dst, uint32_t rows) {
+    constexpr uint32_t CPR = EC / 4;
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const uint32_t c = threadIdx.x + k * 64 * NW;
+        if (c < rows * CPR) {
+            float v[4];
+            fused_raw_to_float(raw[k], dtype, v);
+            lds_store_frag<4>(dst + c * 4, v);   // c * 4 == lr * EC + c4 * 4
+        }
+    }
+}
+
 // LDS -> global for the owned rows, each value times `scale`
 template <int NC, int EC, int NW>
 __device__ __forceinline__ void fused_store_rows_scaled(const FusedArgs& A, const FusedItem& it, const float* src,
@@ -181,11 +239,26 @@ __global__ void __launch_bounds__(64 * kFusedWavesFwd) fused_forward_kernel(cons
     float4* slots = reinterpret_cast<float4*>(w_lds + kFusedMaxStages * 2 * EC) + wave * (F / 4) * 64;
     fused_load_weights<EC, NW>(A, blockIdx.x % A.n_head, w_lds);   // every item of this workgroup has this head
 
+    // trips of 64 * NW threads over the float4 chunks of the largest window the LDS budget allows
+    constexpr int K = (int)((kFusedStateBytes / 2 / sizeof(float4) + 64 * NW - 1) / (64 * NW));
+    uint4 rx[K], ra[K];
+    if (blockIdx.x < A.total_items) {
+        int64_t off[K];
+        fused_window_offsets<NC, EC, NW, K>(A, fused_item<EC>(A, blockIdx.x), rows, off);
+        fused_fetch_rows<K>(A.in0, A.in_dtype, off, rx);
+        fused_fetch_rows<K>(A.in1, A.in_dtype, off, ra);
+    }
     for (uint32_t item = blockIdx.x; item < A.total_items; item += gridDim.x) {
         const FusedItem it = fused_item<EC>(A, item);
-        fused_load_rows<NC, EC, NW>(A, it, A.in0, A.in_dtype, xs, rows);
-        fused_load_rows<NC, EC, NW>(A, it, A.in1, A.in_dtype, as, rows);
+        fused_commit_rows<EC, NW, K>(rx, A.in_dtype, xs, rows);
+        fused_commit_rows<EC, NW, K>(ra, A.in_dtype, as, rows);
         __syncthreads();
+        if (item + gridDim.x < A.total_items) {   // the next window travels while this one is computed
+            int64_t off[K];
+            fused_window_offsets<NC, EC, NW, K>(A, fused_item<EC>(A, item + gridDim.x), rows, off);
+            fused_fetch_rows<K>(A.in0, A.in_dtype, off, rx);
+            fused_fetch_rows<K>(A.in1, A.in_dtype, off, ra);
+        }
         for (int st = 0; st < A.n_stages; ++st) {
             const uint32_t ss = A.sub_stride[st];
             const uint32_t ngroups = A.closed ? A.window : A.window - (NC - 1) * ss;
@@ -221,7 +294,7 @@ __global__ void __launch_bounds__(64 * kFusedWavesFwd) fused_forward_kernel(cons
 }
 
 template <int NC, int EC, int R, int F>
-__global__ void __launch_bounds__(64 * kFusedWavesBwd) fused_backward_kernel(const FusedArgs A) {
+__global__ void __launch_bounds__(64 * kFusedWavesBwd, 4) fused_backward_kernel(const FusedArgs A) {
     constexpr int NW = kFusedWavesBwd;
     using T = Tile<NC, EC, R, F>;
     extern __shared__ float4 fused_lds4[];
@@ -244,6 +317,10 @@ __global__ void __launch_bounds__(64 * kFusedWavesBwd) fused_backward_kernel(con
     const int head = blockIdx.x % A.n_head;   // == head of every item of this workgroup (gridDim.x % n_head == 0)
     fused_load_weights<EC, NW>(A, head, w_lds);
 
+    // The backward step code leaves no registers to carry the next window, so a workgroup only pulls it towards the
+    // caches: each thread reads one word of one row of the next item (one 128-byte line per float32 row) into a word
+    // that nothing needs before the next item, then loads the window as usual and finds it close.
+    uint32_t warm = 0;
     for (uint32_t item = blockIdx.x; item < A.total_items; item += gridDim.x) {
         const FusedItem it = fused_item<EC>(A, item);
         fused_load_rows<NC, EC, NW>(A, it, A.in0, A.in_dtype, ys, rows);
@@ -263,6 +340,17 @@ __global__ void __launch_bounds__(64 * kFusedWavesBwd) fused_backward_kernel(con
             }
         }
         __syncthreads();
+        if (item + gridDim.x < A.total_items) {
+            const FusedItem itn = fused_item<EC>(A, item + gridDim.x);
+            const uint32_t lr = threadIdx.x % rows, arr = threadIdx.x / rows;   // rows <= 64 * NW / 4 for 4 arrays
+            const int64_t off = fused_row_offset<NC>(A, itn, lr);
+            const void* src = arr == 0 ? A.in0 : arr == 1 ? A.in1 : arr == 2 ? A.g0 : A.g1;
+            const int dt = arr < 2 ? A.in_dtype : A.g_dtype;
+            if (arr < 4 && src) {
+                if (dt == NCN_F32) warm ^= *reinterpret_cast<const uint32_t*>(static_cast<const float*>(src) + off);
+                else warm ^= *reinterpret_cast<const uint32_t*>(static_cast<const uint16_t*>(src) + off);
+            }
+        }
         for (int st = A.n_stages - 1; st >= 0; --st) {
             const uint32_t ss = A.sub_stride[st];
             const uint32_t ngroups = A.closed ? A.window : A.window - (NC - 1) * ss;
@@ -338,6 +426,7 @@ __global__ void __launch_bounds__(64 * kFusedWavesBwd) fused_backward_kernel(con
         __syncthreads();
     }
     __syncthreads();
+    if (warm == 0x7fc12345u && A.n_stages < 0) A.dw_partials[0] = 0.f;   // never true: keeps the cache-warming reads
     // one partial row per workgroup and stage; workgroup b owns slot (b / n_head, head b % n_head)
     float* prow = A.dw_partials + (int64_t)(blockIdx.x / A.n_head) * A.n_stages * (2 * A.E);
     for (int k = threadIdx.x; k < A.n_stages * 2 * EC; k += 64 * NW) {
