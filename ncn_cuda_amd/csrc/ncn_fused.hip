@@ -14,7 +14,7 @@ namespace {
 #define NCN_FOR_EACH_FUSED_CONFIG(X) \
     X(2, 16) X(4, 16) X(2, 32) X(4, 32)
 
-constexpr int kFusedMaxGridFwd = 4096;           // forward: no partial rows to pay for, let retiring workgroups balance
+constexpr int kFusedMaxGridFwd = 4096;           // forward: a few windows per workgroup, so that each can fetch its next one early
 constexpr int kFusedMaxGridBwd = 2048;           // backward: one dW partial row per n_head workgroups and stage
 
 size_t fused_lds_bytes(int nc, int ec, bool backward, uint32_t window, int n_stages) {
