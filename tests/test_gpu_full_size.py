@@ -1,0 +1,104 @@
+"""The BASELINE configurations at their full sizes.  The oracle cannot run them whole, so parity is carried by what
+does not depend on size: (batch, head) instances are independent, hence the first batch entries of a full-size run
+must equal the oracle on just those entries; dW is a sum over batch entries, hence the full-size dW must equal the
+sum of the dW of batch chunks; inverse(forward(x)) must give x back; two runs must agree bit for bit."""
+import pytest
+import torch
+
+from oracle import ncn_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+# name: batch, N, E, heads, n_cache, stages, storage dtype, W scale   (the shapes bench.py runs)
+CONFIGS = {
+    "cfg2": (32, 1024, 128, 4, 4, 5, torch.float32, 1.0),
+    "cfg3": (128, 4096, 128, 4, 16, 3, torch.bfloat16, 1.0),
+    "cfg4": (128, 8192, 128, 4, 2, 13, torch.float32, 1.0),
+    "cfg5": (64, 2048, 128, 4, 8, 4, torch.float32, 0.1),
+}
+
+
+@pytest.fixture(scope="module")
+def M():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from ncn_cuda_amd import ncn_cuda_module
+    return ncn_cuda_module
+
+
+def _inputs(name):
+    batch, N, E, C, n, L, dtype, wscale = CONFIGS[name]
+    g = torch.Generator(device="cuda").manual_seed(7)
+    x = torch.randn(batch, N, E, device="cuda", generator=g).to(dtype)
+    xa = (0.5 * torch.randn(batch, N, E, device="cuda", generator=g)).to(dtype)
+    dy = torch.randn(batch, N, E, device="cuda", generator=g).to(dtype)
+    W = (torch.randn(L, 2 * E, device="cuda", generator=g) * wscale / n ** 0.5).to(dtype).float()
+    return x, xa, dy, W
+
+
+def _run(M, x, xa, dy, W, C, n, L, dtype):
+    """Forward + reversible backward the way bench.py runs the configuration: segments of 26 // n stages."""
+    seg = max(1, 26 // n)
+    saved, spans = [], []
+    cx, cxa = x, xa
+    for a in range(0, L, seg):
+        cnt = min(seg, L - a)
+        if cnt == 1:
+            cx, cxa, y32, ya32 = M.forward_stages(cx, cxa, W[a], 0.9, 0, n, C, a, 1, save_fp32=True)
+            saved.append((y32, ya32))
+        else:
+            cx, cxa = M.forward_stages(cx, cxa, W[a:a + cnt], 0.9, 0, n, C, a, cnt, out_dtype=torch.float32)
+            saved.append((cx, cxa))
+        spans.append((a, cnt))
+    g, h = dy, None
+    dWs = [None] * len(spans)
+    for k in range(len(spans) - 1, -1, -1):
+        a, cnt = spans[k]
+        _, _, g, h, dWs[k] = M.backward_stages(saved[k][0], saved[k][1], g, h, W[a:a + cnt], 0.9, 0, n, C, a, cnt,
+                                               grad_dtype=dtype if cnt == 1 else torch.float32, want_inputs=cnt > 1)
+    return cx, cxa, g, h, torch.cat(dWs)
+
+
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_full_size_slice_parity_and_dw_additivity(M, name):
+    batch, N, E, C, n, L, dtype, _ = CONFIGS[name]
+    x, xa, dy, W = _inputs(name)
+    tol = 2e-2 if dtype == torch.bfloat16 else 1e-5
+    y, ya, dx, dxa, dW = _run(M, x, xa, dy, W, C, n, L, dtype)
+    again = _run(M, x, xa, dy, W, C, n, L, dtype)
+    for a, b in zip((y, ya, dx, dxa, dW), again):
+        assert torch.equal(a, b)                                   # deterministic, dW included
+    # the first two batch entries against the oracle (float64 on the same stored values)
+    k = 2
+    d = torch.float64
+    ref = O.net_autograd(x[:k].cpu().to(d), xa[:k].cpu().to(d), [w.cpu().to(d) for w in W], dy[:k].cpu().to(d),
+                         torch.zeros(k, N, E, dtype=d), 0.9, n, C)
+    gtol = max(tol, 1e-6 * (1 / 0.9) ** (n * max(1, 26 // n)))     # rounding growth of the reversal per segment
+    assert O.rel_err(y[:k], ref[0]) < tol and O.rel_err(ya[:k], ref[1]) < tol
+    assert O.rel_err(dx[:k], ref[2]) < gtol and O.rel_err(dxa[:k], ref[3]) < gtol
+    # dW of the two entries alone (GPU) against the oracle, then additivity over batch chunks for the rest
+    part = _run(M, x[:k].contiguous(), xa[:k].contiguous(), dy[:k].contiguous(), W, C, n, L, dtype)[4]
+    for l in range(L):
+        assert O.rel_err(part[l], ref[4][l]) < gtol
+    chunks = 4
+    step = batch // chunks
+    total = torch.zeros_like(dW, dtype=torch.float64)
+    for c in range(chunks):
+        s = slice(c * step, (c + 1) * step)
+        total += _run(M, x[s].contiguous(), xa[s].contiguous(), dy[s].contiguous(), W, C, n, L, dtype)[4].double()
+    assert O.rel_err(dW, total) < 1e-5                             # float32 sums in a different order
+
+
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_full_size_inverse_round_trip(M, name):
+    """inverse(forward(x, xa)) == (x, xa); BASELINE quotes 1e-4 for the reconstruction of configuration 5."""
+    batch, N, E, C, n, L, dtype, _ = CONFIGS[name]
+    x, xa, _, W = _inputs(name)
+    x, xa = x.float(), xa.float()
+    seg = max(1, 26 // n)
+    for a in range(0, L, seg):            # reversal is only asked over what one saved checkpoint covers
+        cnt = min(seg, L - a)
+        y, ya = M.forward_stages(x, xa, W[a:a + cnt], 0.9, 0, n, C, a, cnt)
+        xi, xai = M.inverse_stages(y, ya, W[a:a + cnt], 0.9, 0, n, C, a, cnt)
+        assert O.rel_err(xi, x) < 1e-4 and O.rel_err(xai, xa) < 1e-4
+        x, xa = y, ya
