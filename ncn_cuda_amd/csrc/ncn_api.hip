@@ -306,7 +306,7 @@ static int forward_impl(const void* x, const void* xa, int in_dtype, void* y, vo
                 a.out0 = d0; a.out1 = d1; a.out_dtype = d_dtype;
                 a.aux0 = last ? y32 : nullptr; a.aux1 = last ? ya32 : nullptr;
                 a.W = W + ps.first * wstride;
-                fill_step_table(a.tab, shape->n_cache, alpha, m);
+                fill_step_table(a.tab, shape->n_cache, alpha, m, activation);
                 err = launch_fused(false, a, shape, ps, s);
             }
             if (err != hipSuccess) return (int)err;
@@ -439,7 +439,7 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
                 a.aux0 = dxr; a.aux1 = dxar;
                 a.W = W + ps.first * wstride;
                 a.dw_partials = partials;
-                fill_step_table(a.tab, shape->n_cache, alpha, m);
+                fill_step_table(a.tab, shape->n_cache, alpha, m, activation);
                 err = launch_fused(true, a, shape, ps, s);
                 if (err != hipSuccess) return (int)err;
                 const int rows = fused_grid(shape, ps, true) / shape->n_head;

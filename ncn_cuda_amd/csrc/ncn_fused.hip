@@ -44,7 +44,7 @@ uint32_t floor_pow2(uint32_t v) {
 }  // namespace
 
 bool fused_supported(const ncn_shape* sh, int activation) {
-    if (activation != NCN_ACT_TANH) return false;
+    (void)activation;  // every activation has a build (tanh its own, without the branch on the code)
     const int64_t ec = sh->E / sh->n_head;
     const uint32_t groups = (uint32_t)(sh->N / sh->n_cache);
     if ((groups & (groups - 1)) != 0 || groups < 2) return false;
@@ -141,13 +141,14 @@ static hipError_t launch_fused_t(bool backward, const FusedArgs& a, int grid, si
     constexpr TileShape t = fast_tile(NC, EC);
     static_assert(t.r != 0, "multi-stage shapes must be one-stage shapes too");
     hipError_t err;
+    const bool tanh_only = a.tab.activation == NCN_ACT_TANH;
     if (backward) {
-        auto k = fused_backward_kernel<NC, EC, t.r, t.f>;
+        auto k = tanh_only ? fused_backward_kernel<NC, EC, t.r, t.f, true> : fused_backward_kernel<NC, EC, t.r, t.f, false>;
         err = hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (err != hipSuccess) return err;
         hipLaunchKernelGGL(k, dim3(grid), dim3(64 * kFusedWavesBwd), lds, s, a);
     } else {
-        auto k = fused_forward_kernel<NC, EC, t.r, t.f>;
+        auto k = tanh_only ? fused_forward_kernel<NC, EC, t.r, t.f, true> : fused_forward_kernel<NC, EC, t.r, t.f, false>;
         err = hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (err != hipSuccess) return err;
         hipLaunchKernelGGL(k, dim3(grid), dim3(64 * kFusedWavesFwd), lds, s, a);

@@ -224,7 +224,8 @@ __device__ __forceinline__ void fused_load_weights(const FusedArgs& A, int head,
     }
 }
 
-template <int NC, int EC, int R, int F>
+// TANH_ONLY as in the one-stage kernels: the tanh build has no branch on the activation code.
+template <int NC, int EC, int R, int F, bool TANH_ONLY>
 __global__ void __launch_bounds__(64 * kFusedWavesFwd) fused_forward_kernel(const FusedArgs A) {
     constexpr int NW = kFusedWavesFwd;
     using T = Tile<NC, EC, R, F>;
@@ -276,7 +277,7 @@ __global__ void __launch_bounds__(64 * kFusedWavesFwd) fused_forward_kernel(cons
                     lds_load_frag<F>(xs + row[rr], x[rr]);
                     lds_load_frag<F>(as + row[rr], a[rr]);
                 }
-                forward_core<NC, EC, R, F>(x, a, wi, wj, A.tab, st * NC, lane, slots);
+                forward_core<NC, EC, R, F, TANH_ONLY>(x, a, wi, wj, A.tab, st * NC, lane, slots);
                 if (valid) {
 #pragma unroll
                     for (int rr = 0; rr < R; ++rr) {
@@ -293,8 +294,8 @@ __global__ void __launch_bounds__(64 * kFusedWavesFwd) fused_forward_kernel(cons
     }
 }
 
-template <int NC, int EC, int R, int F>
-__global__ void __launch_bounds__(64 * kFusedWavesBwd, 4) fused_backward_kernel(const FusedArgs A) {
+template <int NC, int EC, int R, int F, bool TANH_ONLY>
+__global__ void __launch_bounds__(64 * kFusedWavesBwd, TANH_ONLY ? 4 : 1) fused_backward_kernel(const FusedArgs A) {
     constexpr int NW = kFusedWavesBwd;
     using T = Tile<NC, EC, R, F>;
     extern __shared__ float4 fused_lds4[];
@@ -373,7 +374,7 @@ __global__ void __launch_bounds__(64 * kFusedWavesBwd, 4) fused_backward_kernel(
                     lds_load_frag<F>(gs + row[rr], G[rr]);
                     lds_load_frag<F>(ps + row[rr], P[rr]);
                 }
-                backward_core<NC, EC, R, F, true>(Y, B, G, P, wi, wj, dwi, dwj, own, A.tab, (A.n_stages - 1 - st) * NC,
+                backward_core<NC, EC, R, F, true, TANH_ONLY>(Y, B, G, P, wi, wj, dwi, dwj, own, A.tab, (A.n_stages - 1 - st) * NC,
                                                   lane, slots);
                 if (valid) {
 #pragma unroll

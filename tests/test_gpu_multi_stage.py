@@ -87,3 +87,41 @@ def test_multi_stage_dya_none_and_bf16_input(M):
     assert O.rel_err(a[2], ref[2]) < 1e-4
     for l in range(L):
         assert O.rel_err(a[4][l], ref[4][l]) < 1e-4
+
+
+@pytest.mark.parametrize("act", [2, -1, 3], ids=["sigmoid", "linear", "leaky_relu"])
+@pytest.mark.parametrize("case", [(2, 1024, 64, 2, 2, 0, 9), (2, 512, 128, 4, 4, 1, 4)],
+                         ids=["n2_halo_and_closed", "n4_from_stage1"])
+def test_multi_stage_other_activations(M, case, act):
+    """The LDS passes in their runtime-activation build (relu is left out as in the one-stage test: its kink makes
+    the reversible recomputation flip F' for |T| ~ eps)."""
+    batch, N, E, C, n, first, L = case
+    alpha = 0.9
+    x, xa, Ws, dyi, dya = O.make_inputs(batch, N, E, L, n, seed=23, xa_zero=False)
+    gx, gxa, gdy, gdya = x.cuda(), xa.cuda(), dyi.cuda(), dya.cuda()
+    Wst = torch.stack(Ws).cuda()
+    import ctypes
+    from ncn_cuda_amd import _lib
+    shape = _lib.NcnShape(batch, N, E, C, n)
+    assert _lib.load().ncn_plan_passes(ctypes.byref(shape), first, L, act, 0, None, 0) >= 1   # LDS passes are used
+    y, ya = M.forward_stages(gx, gxa, Wst, alpha, act, n, C, first, L)
+    d = torch.float64
+    ref = O.net_autograd(x.to(d), xa.to(d), [w.to(d) for w in Ws], dyi.to(d), dya.to(d), alpha, n, C, activation=act,
+                         first_stage=first)
+    assert O.rel_err(y, ref[0]) < 1e-5 and O.rel_err(ya, ref[1]) < 1e-5
+    xr, xar, dx, dxa, dW = M.backward_stages(y, ya, gdy, gdya, Wst, alpha, act, n, C, first, L)
+    tol = max(1e-5, 5e-7 * (1 / 0.9) ** (n * L))
+    assert O.rel_err(xr, x) < tol and O.rel_err(xar, xa) < tol
+    if act == 3:
+        # a kink: where |T| is within rounding of 0 the recomputed slope flips between 1 and 0.01, which moves a
+        # handful of gradient entries (and, through them, dW a little); everything else must agree
+        def q999(a, b):
+            e = (a.detach().double().cpu() - b).abs().flatten() / b.abs().max()
+            return e.kthvalue(int(0.999 * e.numel())).values.item()
+        assert q999(dx, ref[2]) < tol and q999(dxa, ref[3]) < tol
+        for l in range(L):
+            assert O.rel_err(dW[l], ref[4][l]) < 1e-3
+        return
+    assert O.rel_err(dx, ref[2]) < tol and O.rel_err(dxa, ref[3]) < tol
+    for l in range(L):
+        assert O.rel_err(dW[l], ref[4][l]) < tol
