@@ -96,6 +96,15 @@ Plan make_plan(const ncn_shape* sh, int activation, int reserve_rows = 0) {
 }
 
 void fill_step_table(StepTable& t, int n_cache, float alpha, float m, int activation = NCN_ACT_TANH) {
+    // a call fills the same table for every stage it launches, and callers repeat (alpha, m) step after step:
+    // keep the last one per thread (some 450 pow() otherwise)
+    thread_local StepTable cached;
+    thread_local int cached_n = -1;
+    if (cached_n == n_cache && cached.alpha == alpha && cached.m == m) {
+        t = cached;
+        t.activation = activation;
+        return;
+    }
     const double md = m, al = alpha, k2l = 2.8853900817779268;
     t.alpha = alpha;
     t.m = m;
@@ -113,6 +122,8 @@ void fill_step_table(StepTable& t, int n_cache, float alpha, float m, int activa
         t.step[k].fkc = (float)(k2l * (1.0 - al) * mt * mt);
         t.step[k].fkap = (float)((1.0 - md) * im);
     }
+    cached = t;
+    cached_n = n_cache;
 }
 
 // How the rows are grouped and which of them are live: caller's tables of the *_indexed entry points, or nothing.

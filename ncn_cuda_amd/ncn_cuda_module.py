@@ -17,6 +17,7 @@ Deviations from the reference module, all visible in the signatures or return va
   * invalid arguments raise ValueError/TypeError instead of reading out of bounds.
 """
 import ctypes
+import weakref
 
 import torch
 
@@ -113,13 +114,23 @@ def validate_grouping(group_index, ctx_len, batch, N, n_stages):
         raise ValueError(f"ctx_len must hold one length per batch entry ({batch}), got {ctx_len.numel()}")
 
 
+_checked_tables = {}   # id(tensor) -> (weak reference, version counter, N) of tables found good; dies with the tensor
+
+
 def check_group_table(group_index, N):
     """Raises ValueError unless every row of the table is a permutation of 0 .. N-1 (the kernels clamp bad entries
-    but cannot repair a table).  Works on CPU or GPU tensors; on the GPU it synchronises."""
+    but cannot repair a table).  Works on CPU or GPU tensors; on the GPU it synchronises, so a table that passed is
+    remembered (the tensor object with its version counter) and not sorted again while it stays unchanged."""
+    key = id(group_index)
+    seen = _checked_tables.get(key)
+    if seen is not None and seen[0]() is group_index and seen[1:] == (group_index._version, int(N)):
+        return
     t = group_index.reshape(-1, N).to(torch.int64)
     want = torch.arange(N, dtype=torch.int64, device=t.device).expand_as(t)
     if not torch.equal(torch.sort(t, dim=1).values, want):
         raise ValueError("group_index: every stage's row must be a permutation of 0 .. N-1")
+    _checked_tables[key] = (weakref.ref(group_index, lambda _, k=key: _checked_tables.pop(k, None)),
+                            group_index._version, int(N))
 
 
 def _grouping(group_index, ctx_len, batch, N, n_stages, dev, check_tables):
