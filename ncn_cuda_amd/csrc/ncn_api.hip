@@ -453,10 +453,11 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
                 fill_step_table(a.tab, shape->n_cache, alpha, m, activation);
                 err = launch_fused(true, a, shape, ps, s);
                 if (err != hipSuccess) return (int)err;
+                // a partial row holds the pass's stages side by side, as dW does: one reduction for all of them
+                // (rows * count <= kMaxGridX: the chunk sums take at most kMaxGridX / 32 + count rows of 2E)
                 const int rows = fused_grid(shape, ps, true) / shape->n_head;
-                for (int k = 0; k < ps.count && err == hipSuccess; ++k)
-                    err = launch_reduce_dw(partials + k * wstride, rows, (int64_t)ps.count * wstride, wstride, level1,
-                                           dW + (ps.first + k) * wstride, s);
+                err = launch_reduce_dw(partials, rows, (int64_t)ps.count * wstride, (int64_t)ps.count * wstride, level1,
+                                       dW + ps.first * wstride, s);
             }
             if (err != hipSuccess) return (int)err;
             cy = dxr; cya = dxar; cy_dtype = NCN_F32;

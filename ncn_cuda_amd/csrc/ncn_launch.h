@@ -40,7 +40,9 @@ constexpr int kMaxGridX = 4096;
 constexpr int kMaxForwardGridX = 1 << 18;
 // dW partial rows are summed in two levels: chunks of kReduceRowsPerBlock rows, then the chunk sums.
 constexpr int kReduceRowsPerBlock = 32;
-constexpr int kReduceLevel1Rows = kMaxGridX / kReduceRowsPerBlock;
+// (+ 8: a multi-stage pass reduces its up to 8 stages at once, ceil(rows / 32) chunks of `stages` rows each, where
+// rows * stages <= kMaxGridX)
+constexpr int kReduceLevel1Rows = kMaxGridX / kReduceRowsPerBlock + 8;
 
 hipError_t launch_fast_forward(Pass pass, const StageArgs& a, int n_head, int grid_x, hipStream_t s);
 hipError_t launch_fast_backward(const StageArgs& a, int n_head, int grid_x, hipStream_t s);
