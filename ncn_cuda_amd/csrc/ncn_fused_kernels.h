@@ -318,40 +318,47 @@ __global__ void __launch_bounds__(64 * kFusedWavesBwd, TANH_ONLY ? 4 : 1) fused_
     const int head = blockIdx.x % A.n_head;   // == head of every item of this workgroup (gridDim.x % n_head == 0)
     fused_load_weights<EC, NW>(A, head, w_lds);
 
-    // The backward step code leaves no registers to carry the next window, so a workgroup only pulls it towards the
-    // caches: each thread reads one word of one row of the next item (one 128-byte line per float32 row) into a word
-    // that nothing needs before the next item, then loads the window as usual and finds it close.
-    uint32_t warm = 0;
+    // The step code leaves no registers to carry a window across the stages, but between two items they are free:
+    // the window of the next item is requested (all loads of a thread back to back) before the owned rows of this one
+    // are written out, and lands in LDS after them.
+    constexpr int K = (int)((kFusedStateBytes / 4 / sizeof(float4) + 64 * NW - 1) / (64 * NW));
+    struct Raw {
+        uint4 y[K], b[K], g[K], h[K];
+    };
+    auto fetch = [&](uint32_t item, Raw& r) {
+        int64_t off[K];
+        fused_window_offsets<NC, EC, NW, K>(A, fused_item<EC>(A, item), rows, off);
+        fused_fetch_rows<K>(A.in0, A.in_dtype, off, r.y);
+        fused_fetch_rows<K>(A.in1, A.in_dtype, off, r.b);
+        fused_fetch_rows<K>(A.g0, A.g_dtype, off, r.g);
+        fused_fetch_rows<K>(A.g1, A.g_dtype, off, r.h);
+    };
+    auto commit = [&](const Raw& r) {
+        fused_commit_rows<EC, NW, K>(r.y, A.in_dtype, ys, rows);
+        fused_commit_rows<EC, NW, K>(r.b, A.in_dtype, bs, rows);
+        fused_commit_rows<EC, NW, K>(r.g, A.g_dtype, gs, rows);
+        constexpr uint32_t CPR = EC / 4;   // p = (1-m) g + h  (h = 0 when dya is null: the fetch left zeros)
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            const uint32_t c = threadIdx.x + k * 64 * NW;
+            if (c < rows * CPR) {
+                float g[4], h[4];
+                fused_raw_to_float(r.g[k], A.g_dtype, g);
+                fused_raw_to_float(r.h[k], A.g_dtype, h);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) h[e] = fmaf(om, g[e], h[e]);
+                lds_store_frag<4>(ps + c * 4, h);
+            }
+        }
+    };
+    if (blockIdx.x < A.total_items) {
+        Raw first;
+        fetch(blockIdx.x, first);
+        commit(first);
+    }
+    __syncthreads();
     for (uint32_t item = blockIdx.x; item < A.total_items; item += gridDim.x) {
         const FusedItem it = fused_item<EC>(A, item);
-        fused_load_rows<NC, EC, NW>(A, it, A.in0, A.in_dtype, ys, rows);
-        fused_load_rows<NC, EC, NW>(A, it, A.in1, A.in_dtype, bs, rows);
-        {   // g and p = (1-m) g + h
-            constexpr uint32_t CPR = EC / 4;
-            for (uint32_t c = threadIdx.x; c < rows * CPR; c += 64 * NW) {
-                const uint32_t lr = c / CPR, c4 = c - lr * CPR;
-                const int64_t off = fused_row_offset<NC>(A, it, lr) + c4 * 4;
-                float g[4], h[4];
-                load_frag<4>(A.g0, A.g_dtype, off, true, g);
-                load_frag<4>(A.g1, A.g_dtype, off, A.g1 != nullptr, h);
-#pragma unroll
-                for (int k = 0; k < 4; ++k) h[k] = fmaf(om, g[k], h[k]);
-                lds_store_frag<4>(gs + lr * EC + c4 * 4, g);
-                lds_store_frag<4>(ps + lr * EC + c4 * 4, h);
-            }
-        }
-        __syncthreads();
-        if (item + gridDim.x < A.total_items) {
-            const FusedItem itn = fused_item<EC>(A, item + gridDim.x);
-            const uint32_t lr = threadIdx.x % rows, arr = threadIdx.x / rows;   // rows <= 64 * NW / 4 for 4 arrays
-            const int64_t off = fused_row_offset<NC>(A, itn, lr);
-            const void* src = arr == 0 ? A.in0 : arr == 1 ? A.in1 : arr == 2 ? A.g0 : A.g1;
-            const int dt = arr < 2 ? A.in_dtype : A.g_dtype;
-            if (arr < 4 && src) {
-                if (dt == NCN_F32) warm ^= *reinterpret_cast<const uint32_t*>(static_cast<const float*>(src) + off);
-                else warm ^= *reinterpret_cast<const uint32_t*>(static_cast<const uint16_t*>(src) + off);
-            }
-        }
         for (int st = A.n_stages - 1; st >= 0; --st) {
             const uint32_t ss = A.sub_stride[st];
             const uint32_t ngroups = A.closed ? A.window : A.window - (NC - 1) * ss;
@@ -402,7 +409,7 @@ __global__ void __launch_bounds__(64 * kFusedWavesBwd, TANH_ONLY ? 4 : 1) fused_
             }
             __syncthreads();
         }
-        {   // owned rows back to true values: g = G m^T, h = P m^T - (1-m) g, x = Y / m^T, xa = B / m^T
+        auto write_out = [&]() {   // owned rows back to true values: g = G m^T, h = P m^T - (1-m) g, x = Y / m^T, xa = B / m^T
             constexpr uint32_t CPR = EC / 4;
             const uint32_t r0 = it.own_lo * NC, nrows = it.own_cnt * NC;
             for (uint32_t c = threadIdx.x; c < nrows * CPR; c += 64 * NW) {
@@ -419,15 +426,22 @@ __global__ void __launch_bounds__(64 * kFusedWavesBwd, TANH_ONLY ? 4 : 1) fused_
                 store_frag<4>(A.out0, A.out_dtype, off, true, g);
                 store_frag<4>(A.out1, A.out_dtype, off, true, h);
             }
-        }
-        if (A.aux0) {
-            fused_store_rows_scaled<NC, EC, NW>(A, it, ys, A.scale_up, A.aux0, NCN_F32, nullptr);
-            fused_store_rows_scaled<NC, EC, NW>(A, it, bs, A.scale_up, A.aux1, NCN_F32, nullptr);
+            if (A.aux0) {
+                fused_store_rows_scaled<NC, EC, NW>(A, it, ys, A.scale_up, A.aux0, NCN_F32, nullptr);
+                fused_store_rows_scaled<NC, EC, NW>(A, it, bs, A.scale_up, A.aux1, NCN_F32, nullptr);
+            }
+        };
+        if (item + gridDim.x < A.total_items) {   // the same for the whole workgroup
+            Raw next;
+            fetch(item + gridDim.x, next);
+            write_out();
+            __syncthreads();   // every thread has read what it writes out: the window may be overwritten
+            commit(next);
+        } else {
+            write_out();
         }
         __syncthreads();
     }
-    __syncthreads();
-    if (warm == 0x7fc12345u && A.n_stages < 0) A.dw_partials[0] = 0.f;   // never true: keeps the cache-warming reads
     // one partial row per workgroup and stage; workgroup b owns slot (b / n_head, head b % n_head)
     float* prow = A.dw_partials + (int64_t)(blockIdx.x / A.n_head) * A.n_stages * (2 * A.E);
     for (int k = threadIdx.x; k < A.n_stages * 2 * EC; k += 64 * NW) {
