@@ -393,18 +393,23 @@ __global__ void __launch_bounds__(64 * kFusedWavesBwd, TANH_ONLY ? 4 : 1) fused_
                     }
                 }
             }
-            // this wave's dW share of the stage: sum the lanes that hold the same features, add to the wave's slot
+            // this wave's dW share of the stage: sum the lanes of each half of the wave that hold the same features,
+            // then the two halves add to the wave's slot one after the other (a wave's LDS operations keep their
+            // order: the sum is the same in every run, and the costly exchange across the halves is not needed)
 #pragma unroll
             for (int f = 0; f < F; ++f) {
-                dwi[f] = lane_sum<T::LF, 64>(dwi[f]);
-                dwj[f] = lane_sum<T::LF, 64>(dwj[f]);
+                dwi[f] = lane_sum<T::LF, 32>(dwi[f]);
+                dwj[f] = lane_sum<T::LF, 32>(dwj[f]);
             }
-            if (lane < T::LF) {
-                float* d = dw_mine + st * (2 * EC) + fl * F;
 #pragma unroll
-                for (int f = 0; f < F; ++f) {
-                    d[f] += dwi[f];
-                    d[EC + f] += dwj[f];
+            for (int half = 0; half < 2; ++half) {
+                if (lane == fl + 32 * half) {
+                    float* d = dw_mine + st * (2 * EC) + fl * F;
+#pragma unroll
+                    for (int f = 0; f < F; ++f) {
+                        d[f] += dwi[f];
+                        d[EC + f] += dwj[f];
+                    }
                 }
             }
             __syncthreads();
