@@ -126,20 +126,6 @@ __device__ __forceinline__ void lds_store_frag(float* row, const float (&v)[F]) 
         reinterpret_cast<float4*>(row)[k] = make_float4(v[4 * k], v[4 * k + 1], v[4 * k + 2], v[4 * k + 3]);
 }
 
-// global -> LDS for every row of the window (4 features per thread and trip)
-template <int NC, int EC, int NW>
-__device__ __forceinline__ void fused_load_rows(const FusedArgs& A, const FusedItem& it, const void* src, int dtype,
-                                                float* dst, uint32_t rows) {
-    constexpr uint32_t CPR = EC / 4;
-    for (uint32_t c = threadIdx.x; c < rows * CPR; c += 64 * NW) {
-        const uint32_t lr = c / CPR, c4 = c - lr * CPR;
-        float v[4];
-        if (src) load_frag<4>(src, dtype, fused_row_offset<NC>(A, it, lr) + c4 * 4, true, v);
-        else v[0] = v[1] = v[2] = v[3] = 0.f;
-        lds_store_frag<4>(dst + lr * EC + c4 * 4, v);
-    }
-}
-
 // Window rows on their way from global memory to LDS: 4 features per thread and trip, kept as raw bits so that
 // nothing waits for the loads until fused_commit_rows turns them into floats.  A workgroup fetches the window of
 // its next item while it computes the current one.
