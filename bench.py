@@ -206,12 +206,21 @@ def main():
         sample_b = int(max(probe_b, min(batch, round(6.0 / max(tp / probe_b, 1e-6)))))
         ts = cpu_run(sample_b)
         cpu_tokens_s = sample_b * E / ts
+        # the literal restatement of torch_ref's Python loops, on the one configuration where it is feasible
+        # (configuration 1: x[1,256,32], n_cache 2, 8 stages, one head, forward only)
+        lx, lxa, lWs, _, _ = O.make_inputs(1, 256, 32, 8, 2, seed=0, xa_zero=True)
+        tl = time.perf_counter()
+        O.literal_net_forward(lx, lxa, lWs, alpha, 2, 1)
+        literal_s = time.perf_counter() - tl
         result["cpu_baseline"] = {"value": cpu_tokens_s, "unit": "tokens/s", "cores": threads, "kind": "port",
                                   "sample": f"first {sample_b} of {batch} batch entries of the same workload "
                                             f"({sample_b * E} of {tokens} tokens), float32, vectorised PyTorch "
                                             f"restatement of torch_ref (forward + reversible backward), "
                                             f"{ts:.1f} s wall",
-                                  "host_cpus_visible": ncores}
+                                  "host_cpus_visible": ncores,
+                                  "literal_loops_cfg1": {"value": 32 / literal_s, "unit": "tokens/s", "cores": 1,
+                                                         "sample": "configuration 1 (B=32 D=256 g=2, 8 stages), forward "
+                                                                   "only, per-row Python loops as in torch_ref"}}
     print(json.dumps(result))
 
 
