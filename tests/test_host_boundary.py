@@ -100,6 +100,52 @@ def test_entry_points_reject_bad_arguments_before_touching_the_gpu(lib):
     assert h.ncn_backward(*args, p, ctypes.c_size_t(ws), ctypes.byref(sh), 0, 2, 0.9, 0.9, 0, z) == -8  # needs x_rec
 
 
+def test_indexed_entry_points_reject_bad_arguments_before_touching_the_gpu(lib):
+    h = lib.load()
+    sh = _shape(lib, 2, 64, 32, 4, 4)
+    p = ctypes.c_void_p(4096)       # never dereferenced: every call below fails validation first
+    z = ctypes.c_void_p(0)
+    odd4 = ctypes.c_void_p(4098)    # an int32 table must be 4-byte aligned
+    fwd = lambda x, table, lens, act=0: h.ncn_forward_indexed(x, p, 0, p, p, 0, z, z, p, table, lens, ctypes.byref(sh),
+                                                             0, 1, 0.9, 0.9, act, z)
+    assert fwd(z, p, p) == -1
+    assert fwd(p, odd4, z) == -7
+    assert fwd(p, z, odd4) == -7
+    assert fwd(p, p, p, act=9) == -4
+    assert h.ncn_inverse_indexed(p, p, 0, z, p, 0, p, p, p, ctypes.byref(sh), 0, 1, 0.9, 0.9, 0, z) == -1
+    assert h.ncn_inverse_indexed(p, p, 0, p, p, 0, p, odd4, p, ctypes.byref(sh), 0, 1, 0.9, 0.9, 0, z) == -7
+    args = [p, p, 0, p, p, 0, p, p, 0, z, z, p, p]
+    ws = h.ncn_workspace_bytes(ctypes.byref(sh))
+    assert h.ncn_backward_indexed(*args, p, ctypes.c_size_t(ws - 1), p, p, ctypes.byref(sh), 0, 1, 0.9, 0.9, 0, z) == -5
+    assert h.ncn_backward_indexed(*args, p, ctypes.c_size_t(ws), odd4, p, ctypes.byref(sh), 0, 1, 0.9, 0.9, 0, z) == -7
+    bad = _shape(lib, 2, 66, 32, 4, 4)
+    assert h.ncn_backward_indexed(*args, p, ctypes.c_size_t(ws), p, p, ctypes.byref(bad), 0, 1, 0.9, 0.9, 0, z) == -2
+
+
+def test_python_grouping_validation():
+    from ncn_cuda_amd import ncn_cuda_module as M
+    good = torch.randperm(64)
+    M.validate_grouping(good, torch.tensor([3, 64]), batch=2, N=64, n_stages=1)
+    M.validate_grouping(None, None, batch=2, N=64, n_stages=1)
+    M.check_group_table(good, 64)
+    M.check_group_table(torch.stack([good, good.flip(0)]), 64)
+    with pytest.raises(ValueError, match="permutation"):
+        M.check_group_table(torch.zeros(64, dtype=torch.int64), 64)
+    with pytest.raises(ValueError, match="group_index"):
+        M.validate_grouping(good[:-1], None, batch=2, N=64, n_stages=1)
+    with pytest.raises(ValueError, match="group_index"):
+        M.validate_grouping(good, None, batch=2, N=64, n_stages=2)
+    with pytest.raises(ValueError, match="ctx_len"):
+        M.validate_grouping(None, torch.tensor([1, 2, 3]), batch=2, N=64, n_stages=1)
+    with pytest.raises(TypeError):
+        M.validate_grouping(good.float(), None, batch=2, N=64, n_stages=1)
+    with pytest.raises(TypeError):
+        M.validate_grouping([1, 2, 3], None, batch=2, N=64, n_stages=1)
+    x = torch.zeros(2, 64, 32)
+    with pytest.raises(RuntimeError, match="GPU"):      # tables do not open a CPU path either
+        M.forward_stages(x, x, torch.zeros(64), 0.9, 0, 4, 4, 0, 1, group_index=good)
+
+
 def test_python_validation_mirrors_reference_asserts():
     from ncn_cuda_amd import ncn_cuda_module as M
     x = torch.randn(2, 32, 16)
