@@ -2,6 +2,7 @@
 """Headline benchmark: NCN forward + backward of the full stage stack on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg3|cfg2|cfg4|cfg5] [--no-cpu]
+                    [--grouping closed|stride-table|radix-table|ragged]
 
 One step = forward of all L stages (each stage saving its outputs, like the reference's autograd
 node) + reversible backward of all L stages producing dx, dxa and every dW_l, on inputs that are
@@ -50,6 +51,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--config", default="cfg3", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--grouping", default="closed", choices=["closed", "stride-table", "radix-table", "ragged"],
+                    help="closed: the stride permutation in closed form (the headline path).  The others go through "
+                         "the *_indexed entry points, one call per stage: the same permutation as a table, the "
+                         "radix-n digit grouping as a table, or the stride table with one context length per batch "
+                         "entry (N - 1 - b mod n_cache live rows)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one plain 1 GiB device copy, so that a rocprofv3 --pmc run has a kernel of known "
                          "traffic to calibrate FETCH_SIZE / WRITE_SIZE against")
@@ -85,7 +91,19 @@ def main():
     # Stages per saved checkpoint: 1 for the headline shape (every stage saves its outputs, like the reference's
     # autograd node); small groups run whole segments per call (multi-stage LDS passes) and reverse them from the
     # segment's outputs: rounding grows like (1/m)^(n_cache * stages), kept below 16x.
-    save_every = max(1, 26 // n)
+    save_every = max(1, 26 // n) if args.grouping == "closed" else 1   # tables run stage by stage
+    tables = lens = None
+    if args.grouping != "closed":
+        from ncn_cuda_amd import chunk_linear as CL
+        if args.grouping == "radix-table":
+            levels = 1
+            while n ** (levels + 1) <= N and N % n ** (levels + 1) == 0:
+                levels += 1
+            tables = [CL.radix_group_table(N, n, l % levels, device=dev) for l in range(L)]
+        else:
+            tables = [CL.stride_group_table(N, n, l, device=dev) for l in range(L)]
+        if args.grouping == "ragged":
+            lens = (N - 1 - torch.arange(batch, device=dev) % n).to(torch.int32)
     segs = [(a, min(save_every, L - a)) for a in range(0, L, save_every)]
     Wst = torch.stack([w.to(torch.float32) for w in gWs])
 
@@ -93,7 +111,11 @@ def main():
         saved = []
         cx, cxa = gx, gxa
         for a, cnt in segs:
-            if bf16 and cnt == 1:
+            if tables is not None:
+                cx, cxa, y32, ya32 = M.forward_stages(cx, cxa, Wst[a], alpha, 0, n, C, a, 1, save_fp32=True,
+                                                      group_index=tables[a], ctx_len=lens, check_tables=False)
+                saved.append((y32, ya32))
+            elif bf16 and cnt == 1:
                 cx, cxa, y32, ya32 = M.forward_stages(cx, cxa, Wst[a], alpha, 0, n, C, a, 1, save_fp32=True)
                 saved.append((y32, ya32))
             else:
@@ -106,9 +128,10 @@ def main():
             if events is not None:
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 e0.record()
+            extra = {} if tables is None else dict(group_index=tables[a], ctx_len=lens, check_tables=False)
             _, _, dy, dya_, dWs[k] = M.backward_stages(saved[k][0], saved[k][1], dy, dya_, Wst[a:a + cnt], alpha, 0, n,
                                                        C, a, cnt, grad_dtype=io_dtype if cnt == 1 else torch.float32,
-                                                       want_inputs=cnt > 1)
+                                                       want_inputs=cnt > 1, **extra)
             if events is not None:
                 e1.record()
                 events.append((e0, e1, cnt))
@@ -168,10 +191,12 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"{args.config}: B={tokens} D={N} g={n} -> x[batch={batch},N={N},E={E}], "
                                f"{C} heads of {E // C}, n_cache={n}, {L} stages, alpha=0.9, m=0.9, tanh, "
-                               f"{cfg['dtype']} storage, outputs saved every {save_every} stage(s)", "positions_per_s": batch * N / (ms_per_step * 1e-3)},
+                               f"{cfg['dtype']} storage, outputs saved every {save_every} stage(s), "
+                               f"grouping {args.grouping}", "positions_per_s": batch * N / (ms_per_step * 1e-3)},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_BWD_TRAFFIC_BYTES.get(args.config),
-                     "kernel": (f"stage_backward_kernel<{n},{E // C}>" if save_every == 1 else
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_BWD_TRAFFIC_BYTES.get(args.config) if args.grouping == "closed" else None,
+                     "kernel": (f"stage_backward_kernel<{n},{E // C}>" + (" (indexed build)" if tables else "")
+                                if save_every == 1 else
                                 f"backward of {save_every}-stage segments (multi-stage passes), per stage"),
                      "avg_launch_ms": bwd_ms,
                      "attainable_copy_GBps": copy_gbps, "frac_of_attainable_copy": achieved / copy_gbps,
