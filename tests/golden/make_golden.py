@@ -127,7 +127,7 @@ def main():
     torch.set_num_threads(4)
     _index_fixture(ref)
     _invert_fixture(inv)
-    # BASELINE config 1: x [B=32, D=256], g=2, 8 stages  ->  [batch=1, N=256, E=32], 4 heads of 8
+    # benchmark configuration 1: x [B=32, D=256], g=2, 8 stages  ->  [batch=1, N=256, E=32], 4 heads of 8
     _case("cfg1_n2_L8", ref, inv, batch=1, N=256, E=32, C=4, n=2, L=8, alpha=0.9,
           w_std=(1 / 2) ** 0.5, seed=0, xa_zero=True, run_inv=False)
     # multi-batch, multi-head, n=4, 3 stages, xa != 0, alpha != 0.9, both heads differ in W

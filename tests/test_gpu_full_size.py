@@ -1,4 +1,4 @@
-"""The BASELINE configurations at their full sizes.  The oracle cannot run them whole, so parity is carried by what
+"""The four benchmark configurations at their full sizes.  The oracle cannot run them whole, so parity is carried by what
 does not depend on size: (batch, head) instances are independent, hence the first batch entries of a full-size run
 must equal the oracle on just those entries; dW is a sum over batch entries, hence the full-size dW must equal the
 sum of the dW of batch chunks; inverse(forward(x)) must give x back; two runs must agree bit for bit."""
@@ -91,7 +91,7 @@ def test_full_size_slice_parity_and_dw_additivity(M, name):
 
 @pytest.mark.parametrize("name", list(CONFIGS))
 def test_full_size_inverse_round_trip(M, name):
-    """inverse(forward(x, xa)) == (x, xa); BASELINE quotes 1e-4 for the reconstruction of configuration 5."""
+    """inverse(forward(x, xa)) == (x, xa); the target for the reconstruction of configuration 5 is 1e-4."""
     batch, N, E, C, n, L, dtype, _ = CONFIGS[name]
     x, xa, _, W = _inputs(name)
     x, xa = x.float(), xa.float()
