@@ -138,8 +138,10 @@ __device__ __forceinline__ void store_elem(void* base, int dtype, int64_t off, f
 // ---------------------------------------------------------------------------------------------
 // cross-lane moves inside one 64-wide wavefront
 // ---------------------------------------------------------------------------------------------
-// value of lane (lane ^ S)
-template <int S>
+// value of lane (lane ^ S).  ROWS: stride 8 as a DPP row rotation instead of a trip through the LDS crossbar
+// (costs the same issue slots, and on kernels that are bound by issue a little more through its wait states; pays
+// on kernels that wait on latency).
+template <int S, bool ROWS = false>
 __device__ __forceinline__ float lane_xor(float v) {
     static_assert(S == 1 || S == 2 || S == 4 || S == 8 || S == 16 || S == 32, "power of two below 64");
     int x = __float_as_int(v);
@@ -147,6 +149,8 @@ __device__ __forceinline__ float lane_xor(float v) {
         x = __builtin_amdgcn_mov_dpp(x, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
     } else if constexpr (S == 2) {
         x = __builtin_amdgcn_mov_dpp(x, 0x4E, 0xF, 0xF, true);  // quad_perm [2,3,0,1]
+    } else if constexpr (S == 8 && ROWS) {
+        x = __builtin_amdgcn_update_dpp(0, x, 0x128, 0xF, 0xF, true);  // row_ror:8 == lane ^ 8 inside a row of 16
     } else if constexpr (S < 32) {
         x = __builtin_amdgcn_ds_swizzle(x, (S << 10) | 0x1F);   // bit mode: lane' = lane ^ S inside 32
     } else {
@@ -156,12 +160,17 @@ __device__ __forceinline__ float lane_xor(float v) {
     return __int_as_float(x);
 }
 
-// sum over the lanes {lane ^ k*LO : k} for strides LO, 2*LO, .. < HI  (LO, HI powers of two)
-template <int LO, int HI>
+// sum over the lanes {lane ^ k*LO : k} for strides LO, 2*LO, .. < HI  (LO, HI powers of two).
+// ROWS (see lane_xor): when the recursion started at stride 1 (FROM1), the value is the same in the four lanes of a
+// quad from stride 4 on, and the partner quad is read through row_half_mirror (lane 7 - i of each 8).
+template <int LO, int HI, bool ROWS = false, bool FROM1 = (LO == 1)>
 __device__ __forceinline__ float lane_sum(float v) {
     if constexpr (LO < HI) {
-        v += lane_xor<LO>(v);
-        return lane_sum<LO * 2, HI>(v);
+        if constexpr (LO == 4 && FROM1 && ROWS)
+            v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true));
+        else
+            v += lane_xor<LO, ROWS>(v);
+        return lane_sum<LO * 2, HI, ROWS, FROM1>(v);
     } else {
         return v;
     }

@@ -132,7 +132,7 @@ __device__ __forceinline__ float dot_frag(const float (&a)[F], const float (&b)[
 // STEP_MASK builds take `live`, the live rows of the lane's group, and skip steps j >= live with the lanes of that
 // group switched off (a group that a context length cuts runs one step per live row,
 // ncn_triton/ncn_triton_old.py:93-96).  Every cross-lane exchange of a step stays inside one group.
-template <int NC, int EC, int R, int F, bool TANH_ONLY = true, bool STEP_MASK = false>
+template <int NC, int EC, int R, int F, bool TANH_ONLY = true, bool STEP_MASK = false, bool ROWS = false>
 __device__ __forceinline__ void forward_core(float (&x)[R][F], float (&a)[R][F], const float (&wi)[F],
                                              const float (&wj)[F], const StepTable& S, int step_base, int lane,
                                              float4* slots, int live = NC) {
@@ -154,7 +154,7 @@ __device__ __forceinline__ void forward_core(float (&x)[R][F], float (&a)[R][F],
 #pragma unroll
             for (int k = 1; k <= R; ++k) {
                 const int rr = (jr + k) % R;
-                const float s = lane_sum<1, T::LF>(dot_frag<F>(x[rr], wi) + e);
+                const float s = lane_sum<1, T::LF, ROWS>(dot_frag<F>(x[rr], wi) + e);
                 const float c = kc * s;
 #pragma unroll
                 for (int f = 0; f < F; ++f) {
@@ -278,7 +278,7 @@ __device__ __forceinline__ void inverse_steps(float (&y)[R][F], float (&b)[R][F]
 // backward_core: the n_cache steps of one stage on registers in the scaled form above with t0 = step_base
 // inversion steps done before (P holds p / m^t0, not h); leaves them scaled by t0 + n_cache steps.
 // STEP_MASK: steps j >= live leave the registers as they are (see inverse_steps for the scaling).
-template <int NC, int EC, int R, int F, bool MASKED, bool TANH_ONLY = true, bool STEP_MASK = false>
+template <int NC, int EC, int R, int F, bool MASKED, bool TANH_ONLY = true, bool STEP_MASK = false, bool ROWS = false>
 __device__ __forceinline__ void backward_core(float (&Y)[R][F], float (&B)[R][F], float (&G)[R][F], float (&P)[R][F],
                                               const float (&wi)[F], const float (&wj)[F], float (&dwi)[F],
                                               float (&dwj)[F], float own, const StepTable& S, int step_base, int lane,
@@ -311,7 +311,7 @@ __device__ __forceinline__ void backward_core(float (&Y)[R][F], float (&B)[R][F]
             float rhosum = 0.f;
 #pragma unroll
             for (int rr = 0; rr < R; ++rr) {
-                const float Ssum = lane_sum<1, T::LF>(dot_frag<F>(Y[rr], wi) + e);
+                const float Ssum = lane_sum<1, T::LF, ROWS>(dot_frag<F>(Y[rr], wi) + e);
                 const float chat = kc2 * Ssum;
                 float u[F];
                 float rh = 0.f;
@@ -324,7 +324,7 @@ __device__ __forceinline__ void backward_core(float (&Y)[R][F], float (&B)[R][F]
                     u[f] = P[rr][f] * w;
                     rh = fmaf(u[f], xj[f], rh);
                 }
-                rh = lane_sum<1, T::LF>(rh);
+                rh = lane_sum<1, T::LF, ROWS>(rh);
                 const float rho = krho * rh;       // (1-alpha) r_i / m^(t+1)
                 const float c4 = krho * Ssum;      // (1-alpha) s_i u-scale / m^(t+1)
                 const float rho_w = MASKED ? rho * own : rho;
@@ -341,7 +341,7 @@ __device__ __forceinline__ void backward_core(float (&Y)[R][F], float (&B)[R][F]
 #pragma unroll
             for (int f = 0; f < F; ++f) {
                 dwj[f] = fmaf(rhosum_w, xj[f], dwj[f]);
-                const float vt = lane_sum<T::LF, T::LPG>(fmaf(rhosum, wj[f], v[f]));  // over the group's row lanes
+                const float vt = lane_sum<T::LF, T::LPG, ROWS>(fmaf(rhosum, wj[f], v[f]));  // over the group's row lanes
                 G[jr][f] = fmaf(sel, vt, G[jr][f]);
                 P[jr][f] = fmaf(om, G[jr][f], P[jr][f]);
             }
