@@ -139,3 +139,24 @@ def test_net_cuda_fuse_stages_flag_keeps_parameters(pkg):
     assert O.rel_err(outs[1][1], outs[0][1]) < 1e-5
     for ga, gb in zip(outs[0][2], outs[1][2]):
         assert O.rel_err(gb, ga) < 1e-5
+
+
+def test_triton_named_surface_matches_cuda_named_surface(pkg):
+    """NCNNetTestTriton (activation by name) and NCNNetTestCuda give the same numbers: one set of kernels."""
+    from ncn_cuda_amd import ncn_triton as T
+    batch, N, E, C, n, L = 2, 128, 64, 2, 8, 3
+    x, xa, Ws, dy, dya = O.make_inputs(batch, N, E, L, n, seed=3, xa_zero=False)
+    for name in ("tanh", "leaky-relu", "identity"):
+        res = []
+        for make in (lambda w: T.NCNNetTestTriton(0.9, name, n, C, L, w),
+                     lambda w: pkg.NCNNetTestCuda(0.9, name if name in pkg.ACTIVATION_CODES else "linear", n, C, L, w)):
+            gx, gxa = x.cuda().requires_grad_(), xa.cuda().requires_grad_()
+            gw = [w.cuda().requires_grad_() for w in Ws]
+            yi, ya = make(gw)(gx, gxa)
+            torch.autograd.backward([yi, ya], [dy.cuda(), dya.cuda()])
+            res.append([yi, ya, gx.grad, gxa.grad] + [w.grad for w in gw])
+        for a, b in zip(*res):
+            assert torch.equal(a, b)
+    d = torch.float64
+    ref = O.net_autograd(x.to(d), xa.to(d), [w.to(d) for w in Ws], dy.to(d), dya.to(d), 0.9, n, C, activation=-1)
+    assert O.rel_err(res[0][0], ref[0]) < 1e-5 and O.rel_err(res[0][2], ref[2]) < 1e-5

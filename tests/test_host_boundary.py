@@ -191,6 +191,24 @@ def test_surface_matches_reference_names():
     assert pkg.ACTIVATION_CODES["leaky-relu"] == 3 and len(pkg.ACTIVATION_CODES) == 5
 
 
+def test_triton_surface_names_and_arguments():
+    """ncn_triton/ncn_triton.py:333-421 by name and positional arguments; activation names map to codes."""
+    import inspect
+    from ncn_cuda_amd import ncn_triton as T
+    assert list(inspect.signature(T.fused_ncn_triton).parameters) == [
+        "x", "xa", "W", "ALPHA", "ACTIVATION", "NHEAD", "CACHE", "MODULE_L"]
+    ctor = ["alpha", "activation", "n_cache", "n_head"]
+    assert list(inspect.signature(T.NCNModuleTriton.__init__).parameters)[1:] == ctor + ["module_nr", "embed_dim"]
+    assert list(inspect.signature(T.NCNNetTriton.__init__).parameters)[1:] == ctor + ["num_modules", "embed_dim"]
+    assert list(inspect.signature(T.NCNNetTestTriton.__init__).parameters)[1:] == ctor + ["num_modules", "weights"]
+    assert [T.activation_code(a) for a in ("tanh", "leaky-relu", "none", "relu", 2)] == [0, 3, -1, -1, 2]
+    net = T.NCNNetTriton(0.9, "tanh", 4, 2, 3, 16)
+    assert sorted(net.state_dict()) == [f"ncn_modules.{l}.weight" for l in range(3)]
+    assert net.ncn_modules[0].weight.shape == (32,) and net.ncn_modules[0].weight.std() < 0.1
+    net.ncn_modules[1].reset_parameters()
+    assert net.ncn_modules[1].weight.abs().max() <= 0.25
+
+
 def test_product_code_never_imports_the_oracle():
     pkg_dir = os.path.join(ROOT, "ncn_cuda_amd")
     for dirpath, _, files in os.walk(pkg_dir):
