@@ -35,7 +35,7 @@ constexpr int kGenericMaxHeadDim = 64;
 constexpr int kGenericArrays = 7;
 
 // Upper bound on gridDim.x of a stage launch == rows of the dW partial buffer.
-constexpr int kMaxGridX = 4096;
+constexpr int kMaxGridX = 16384;
 // Upper bound on gridDim.x of a forward / inverse launch (no partial rows to pay for).
 constexpr int kMaxForwardGridX = 1 << 18;
 // dW partial rows are summed in two levels: chunks of kReduceRowsPerBlock rows, then the chunk sums.
