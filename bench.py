@@ -39,7 +39,7 @@ VALU_PEAK_TFLOPS = 157.3   # MI355X FP32 vector peak (packed); 78.6 without pack
 # + 2 (x) + exp2 + rcp = 13; backward 11 FMA + 4 mul/add + exp2 + rcp = 28.
 # HBM bytes of one backward-stage launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (calibrated on a
 # 1 GiB copy; see profiles/stage_kernels_cfg3.md).  Only the headline workload has been measured.
-MEASURED_BWD_TRAFFIC_BYTES = {"cfg3": 1.0540e9}
+MEASURED_BWD_TRAFFIC_BYTES = {"cfg3": 1.1128e9}
 FLOPS_FWD_PER_ELEM_STEP = 13.0
 FLOPS_BWD_PER_ELEM_STEP = 28.0
 
