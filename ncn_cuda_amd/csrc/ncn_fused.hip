@@ -15,7 +15,7 @@ namespace {
     X(2, 16) X(4, 16) X(2, 32) X(4, 32)
 
 constexpr int kFusedMaxGridFwd = 4096;           // forward: a few windows per workgroup, so that each can fetch its next one early
-constexpr int kFusedMaxGridBwd = 2048;           // backward: one dW partial row per n_head workgroups and stage
+constexpr int kFusedMaxGridBwd = 4096;           // backward: one dW partial row per n_head workgroups and stage
 
 size_t fused_lds_bytes(int nc, int ec, bool backward, uint32_t window, int n_stages) {
     const TileShape t = fast_tile(nc, ec);
