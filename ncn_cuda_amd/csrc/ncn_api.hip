@@ -18,7 +18,7 @@ bool known_dtype(int d) { return d == NCN_F32 || d == NCN_BF16; }
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // 2 = register kernels, 1 = generic LDS kernels, 0 = unsupported
-int kernel_path(const ncn_shape* sh, int activation) {
+int kernel_path(const ncn_shape* sh, int /*activation*/) {
     if (sh->n_cache < 1 || sh->n_cache > 64) return 0;
     const int64_t ec = sh->E / sh->n_head;
     if (ec <= 128 && fast_tile(sh->n_cache, (int)ec).r != 0) return 2;

@@ -12,9 +12,9 @@
 namespace ncn {
 
 #if NCN_INDEXED_BUILD
-hipError_t launch_fast_forward_indexed(Pass pass, const StageArgs& a, int n_head, int grid_x, hipStream_t s) {
+hipError_t launch_fast_forward_indexed(Pass pass, const StageArgs& a, int /*n_head*/, int grid_x, hipStream_t s) {
 #else
-hipError_t launch_fast_forward(Pass pass, const StageArgs& a, int n_head, int grid_x, hipStream_t s) {
+hipError_t launch_fast_forward(Pass pass, const StageArgs& a, int /*n_head*/, int grid_x, hipStream_t s) {
 #endif
     constexpr bool kIndexed = NCN_INDEXED_BUILD != 0;
     const dim3 grid(grid_x), block(kBlockThreads);
