@@ -2,7 +2,7 @@
 """Headline benchmark: NCN forward + backward of the full stage stack on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg3|cfg2|cfg4|cfg5] [--no-cpu]
-                    [--grouping closed|stride-table|radix-table|ragged]
+                    [--grouping closed|stride-table|radix-table|ragged|radix]
 
 One step = forward of all L stages (each stage saving its outputs, like the reference's autograd
 node) + reversible backward of all L stages producing dx, dxa and every dW_l, on inputs that are
@@ -51,11 +51,13 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--config", default="cfg3", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--grouping", default="closed", choices=["closed", "stride-table", "radix-table", "ragged"],
+    ap.add_argument("--grouping", default="closed", choices=["closed", "stride-table", "radix-table", "ragged", "radix"],
                     help="closed: the stride permutation in closed form (the headline path).  The others go through "
                          "the *_indexed entry points, one call per stage: the same permutation as a table, the "
                          "radix-n digit grouping as a table, or the stride table with one context length per batch "
-                         "entry (N - 1 - b mod n_cache live rows)")
+                         "entry (N - 1 - b mod n_cache live rows).  radix: levels 0 .. L-1 of the radix-n digit grouping "
+                         "through ncn_forward_radix / ncn_backward_radix (needs n_cache^L to divide N; several levels "
+                         "per LDS pass for n_cache 2 and 4; float32 between calls)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one plain 1 GiB device copy, so that a rocprofv3 --pmc run has a kernel of known "
                          "traffic to calibrate FETCH_SIZE / WRITE_SIZE against")
@@ -91,9 +93,9 @@ def main():
     # Stages per saved checkpoint: 1 for the headline shape (every stage saves its outputs, like the reference's
     # autograd node); small groups run whole segments per call (multi-stage LDS passes) and reverse them from the
     # segment's outputs: rounding grows like (1/m)^(n_cache * stages), kept below 16x.
-    save_every = max(1, 26 // n) if args.grouping == "closed" else 1   # tables run stage by stage
+    save_every = max(1, 26 // n) if args.grouping in ("closed", "radix") else 1   # tables run stage by stage
     tables = lens = None
-    if args.grouping != "closed":
+    if args.grouping not in ("closed", "radix"):
         from ncn_cuda_amd import chunk_linear as CL
         if args.grouping == "radix-table":
             levels = 1
@@ -111,7 +113,10 @@ def main():
         saved = []
         cx, cxa = gx, gxa
         for a, cnt in segs:
-            if tables is not None:
+            if args.grouping == "radix":
+                cx, cxa = M.forward_radix(cx, cxa, Wst[a:a + cnt], alpha, 0, n, C, a, cnt)
+                saved.append((cx, cxa))
+            elif tables is not None:
                 cx, cxa, y32, ya32 = M.forward_stages(cx, cxa, Wst[a], alpha, 0, n, C, a, 1, save_fp32=True,
                                                       group_index=tables[a], ctx_len=lens, check_tables=False)
                 saved.append((y32, ya32))
@@ -129,9 +134,14 @@ def main():
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 e0.record()
             extra = {} if tables is None else dict(group_index=tables[a], ctx_len=lens, check_tables=False)
-            _, _, dy, dya_, dWs[k] = M.backward_stages(saved[k][0], saved[k][1], dy, dya_, Wst[a:a + cnt], alpha, 0, n,
-                                                       C, a, cnt, grad_dtype=io_dtype if cnt == 1 else torch.float32,
-                                                       want_inputs=cnt > 1, **extra)
+            if args.grouping == "radix":
+                _, _, dy, dya_, dWs[k] = M.backward_radix(saved[k][0], saved[k][1], dy, dya_, Wst[a:a + cnt], alpha, 0,
+                                                          n, C, a, cnt)
+            else:
+                _, _, dy, dya_, dWs[k] = M.backward_stages(saved[k][0], saved[k][1], dy, dya_, Wst[a:a + cnt], alpha,
+                                                           0, n, C, a, cnt,
+                                                           grad_dtype=io_dtype if cnt == 1 else torch.float32,
+                                                           want_inputs=cnt > 1, **extra)
             if events is not None:
                 e1.record()
                 events.append((e0, e1, cnt))

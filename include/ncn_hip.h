@@ -177,6 +177,44 @@ int ncn_inverse_indexed(const void* y, const void* ya, int in_dtype,
                         const ncn_shape* shape, int first_stage, int n_stages,
                         float alpha, float m, int activation, void* stream);
 
+/*
+ * Levels first_level .. first_level+n_levels-1 of the radix-n digit grouping: level l groups the n_cache positions
+ * of the N axis that differ only in base-n_cache digit l (slot = that digit; the remaining digits, the upper ones
+ * moved down one place, number the group).
+ * Replaces: the grouping of ncn_triton/group_tensors.py:8-18 (extract_group_index), which the reference only has as a
+ *           helper that writes index tensors; level 0 is stage 0 of the stride permutation.  The same levels can be
+ *           run through ncn_*_indexed with tables; these entry points need no table and, for n_cache 2 or 4 with a
+ *           head width of 16 or 32, keep windows of n_cache^k rows in LDS over k levels per pass (such windows are
+ *           closed: no halo, every pass in place), so a stack of log_n(N) levels costs two or three passes over HBM.
+ * n_cache^(first_level+n_levels) must divide N (NCN_ERR_SHAPE otherwise).  W, dW: [n_levels, 2E].
+ * Arguments as in ncn_forward / ncn_backward.  Levels after the first pass run in place on y, ya (forward) and on
+ * x_rec, xa_rec, dx, dxa (backward): use float32 outputs when more than one pass is needed, or the values between
+ * passes are rounded to the output type.  ncn_backward_radix needs ncn_workspace_bytes(shape) of scratch.
+ */
+int ncn_forward_radix(const void* x, const void* xa, int in_dtype,
+                      void* y, void* ya, int out_dtype,
+                      float* y32, float* ya32,
+                      const float* W,
+                      const ncn_shape* shape, int first_level, int n_levels,
+                      float alpha, float m, int activation, void* stream);
+
+int ncn_backward_radix(const void* y, const void* ya, int y_dtype,
+                       const void* dy, const void* dya, int dy_dtype,
+                       void* dx, void* dxa, int dx_dtype,
+                       float* x_rec, float* xa_rec,
+                       const float* W, float* dW,
+                       void* workspace, size_t workspace_bytes,
+                       const ncn_shape* shape, int first_level, int n_levels,
+                       float alpha, float m, int activation, void* stream);
+
+/* How the two calls above cut the levels into passes; returns the number of passes or a negative error code and
+ * writes up to max_passes records of 6 int32 into `out` (may be NULL):
+ *   [0] first level of the pass relative to first_level   [1] levels in the pass   [2] 0 one-stage launch, 1 LDS windows
+ *   [3] n_cache^(first level): distance in rows between the rows of a window   [4] rows of a window   [5] rows per workgroup
+ * No reference counterpart. */
+int ncn_plan_radix(const ncn_shape* shape, int first_level, int n_levels, int activation, int backward, int32_t* out,
+                   int max_passes);
+
 /* Bytes of scratch ncn_backward needs for this shape (0 on an invalid shape).  No reference counterpart:
  * the reference allocates a [batch,N,2E] partial-dW tensor per call (ncn_bwd_cuda_kernel.cu:251). */
 size_t ncn_workspace_bytes(const ncn_shape* shape);

@@ -14,7 +14,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libncn_hip.so")
 SOURCES = ["ncn_api.hip", "ncn_fwd.hip", "ncn_bwd.hip", "ncn_fwd_indexed.hip", "ncn_bwd_indexed.hip", "ncn_generic.hip",
-           "ncn_fused.hip"]
+           "ncn_fused.hip", "ncn_fused_radix.hip"]
 # packed-fp32 VALU instructions are switched off for device code on purpose (flag is device-only;
 # the host pass prints a harmless "not a recognized feature" note).
 HIPCC_FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17",
@@ -42,7 +42,7 @@ def build(verbose=False):
     build_dir = os.path.join(PKG_DIR, "build")
     os.makedirs(build_dir, exist_ok=True)
     jobs = [(s, os.path.join(build_dir, s.replace(".hip", ".o"))) for s in SOURCES]
-    with ThreadPoolExecutor(max_workers=min(7, len(jobs))) as pool:
+    with ThreadPoolExecutor(max_workers=min(8, len(jobs))) as pool:
         objs = list(pool.map(_compile, jobs))
     tmp = LIB_PATH + ".tmp"
     cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs]

@@ -130,8 +130,26 @@ void fill_step_table(StepTable& t, int n_cache, float alpha, float m, int activa
 struct Grouping {
     const int32_t* table;    // [n_stages, N] or null
     const int32_t* ctx_len;  // [batch] or null
-    bool plain() const { return !table && !ctx_len; }
+    int radix_first = -1;    // >= 0: stage k is radix level radix_first + k (no table then)
+    bool plain() const { return !table && !ctx_len && radix_first < 0; }
 };
+
+uint32_t upow(uint32_t b, int e) {
+    uint64_t r = 1;
+    for (int k = 0; k < e; ++k) r *= b;
+    return (uint32_t)r;
+}
+
+// levels first .. first+count-1 exist when n^(first+count) divides N
+int check_radix(const ncn_shape* sh, int first, int count) {
+    if (first < 0 || count < 1) return NCN_ERR_SHAPE;
+    int64_t p = 1;
+    for (int k = 0; k < first + count; ++k) {
+        p *= sh->n_cache;
+        if (p > sh->N) return NCN_ERR_SHAPE;
+    }
+    return (sh->N % p == 0) ? NCN_OK : NCN_ERR_SHAPE;
+}
 
 int check_grouping(const Grouping& g, const ncn_shape* sh) {
     if ((reinterpret_cast<uintptr_t>(g.table) & 3u) || (reinterpret_cast<uintptr_t>(g.ctx_len) & 3u)) return NCN_ERR_ALIGN;
@@ -144,6 +162,7 @@ void fill_common(StageArgs& a, const ncn_shape* sh, const Plan& p, int stage, fl
     a.table = g.table ? g.table + (int64_t)rel_stage * sh->N : nullptr;
     a.ctx_len = g.ctx_len;
     a.edge = 0;
+    a.radix_stride = g.radix_first >= 0 ? upow((uint32_t)sh->n_cache, g.radix_first + rel_stage) : 0u;
     a.N = sh->N;
     a.E = sh->E;
     a.total_tiles = p.total_tiles;
@@ -540,6 +559,133 @@ int ncn_backward_indexed(const void* y, const void* ya, int y_dtype, const void*
     return backward_impl(y, ya, y_dtype, dy, dya, dy_dtype, dx, dxa, dx_dtype, x_rec, xa_rec, W, dW, workspace,
                          workspace_bytes, Grouping{group_index, ctx_len}, shape, first_stage, n_stages, alpha, m,
                          activation, stream);
+}
+
+int ncn_forward_radix(const void* x, const void* xa, int in_dtype, void* y, void* ya, int out_dtype, float* y32,
+                      float* ya32, const float* W, const ncn_shape* shape, int first_level, int n_levels, float alpha,
+                      float m, int activation, void* stream) {
+    int rc = check_shape(shape, 0, n_levels, activation);
+    if (rc != NCN_OK) return rc;
+    rc = check_radix(shape, first_level, n_levels);
+    if (rc != NCN_OK) return rc;
+    if (!x || !xa || !y || !ya || !W) return NCN_ERR_NULL;
+    if ((y32 == nullptr) != (ya32 == nullptr)) return NCN_ERR_NULL;
+    if (!known_dtype(in_dtype) || !known_dtype(out_dtype)) return NCN_ERR_DTYPE;
+    if (!aligned16(x) || !aligned16(xa) || !aligned16(y) || !aligned16(ya) || !aligned16(W) || !aligned16(y32) ||
+        !aligned16(ya32))
+        return NCN_ERR_ALIGN;
+    const Plan p = make_plan(shape, activation);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int64_t wstride = 2 * shape->E;
+    const std::vector<RadixPass> passes = plan_radix(shape, first_level, n_levels, false);
+    // every pass is closed: the first reads x, xa and the later ones run in place on y, ya; passes of several levels
+    // keep their state in float32 LDS and convert on the way out
+    for (size_t k = 0; k < passes.size(); ++k) {
+        const RadixPass& ps = passes[k];
+        const bool first = (k == 0), last = (k + 1 == passes.size());
+        hipError_t err;
+        if (ps.single) {
+            StageArgs a{};
+            Grouping g{nullptr, nullptr, first_level + ps.first};
+            fill_common(a, shape, p, 0, alpha, m, activation, g, 0);
+            a.in0 = first ? x : y; a.in1 = first ? xa : ya; a.in_dtype = first ? in_dtype : out_dtype;
+            a.out0 = y; a.out1 = ya; a.out_dtype = out_dtype;
+            a.aux0 = last ? y32 : nullptr; a.aux1 = last ? ya32 : nullptr;
+            a.W = W + ps.first * wstride;
+            err = (p.path != 2) ? launch_generic(kForward, a, shape->n_head, p.grid_fwd, s)
+                                : launch_fast_forward_indexed(kForward, a, shape->n_head, p.grid_fwd, s);
+        } else {
+            FusedArgs a{};
+            a.in0 = first ? x : y; a.in1 = first ? xa : ya; a.in_dtype = first ? in_dtype : out_dtype;
+            a.out0 = y; a.out1 = ya; a.out_dtype = out_dtype;
+            a.aux0 = last ? y32 : nullptr; a.aux1 = last ? ya32 : nullptr;
+            a.W = W + ps.first * wstride;
+            fill_step_table(a.tab, shape->n_cache, alpha, m, activation);
+            err = launch_fused_radix(false, a, shape, ps, s);
+        }
+        if (err != hipSuccess) return (int)err;
+    }
+    return NCN_OK;
+}
+
+int ncn_backward_radix(const void* y, const void* ya, int y_dtype, const void* dy, const void* dya, int dy_dtype,
+                       void* dx, void* dxa, int dx_dtype, float* x_rec, float* xa_rec, const float* W, float* dW,
+                       void* workspace, size_t workspace_bytes, const ncn_shape* shape, int first_level, int n_levels,
+                       float alpha, float m, int activation, void* stream) {
+    int rc = check_shape(shape, 0, n_levels, activation);
+    if (rc != NCN_OK) return rc;
+    rc = check_radix(shape, first_level, n_levels);
+    if (rc != NCN_OK) return rc;
+    if (!y || !ya || !dy || !dx || !dxa || !W || !dW) return NCN_ERR_NULL;
+    if ((x_rec == nullptr) != (xa_rec == nullptr)) return NCN_ERR_NULL;
+    if (!known_dtype(y_dtype) || !known_dtype(dy_dtype) || !known_dtype(dx_dtype)) return NCN_ERR_DTYPE;
+    if (n_levels > 1 && (!x_rec || dx_dtype != NCN_F32)) return NCN_ERR_ALIAS;
+    if (!workspace || workspace_bytes < ncn_workspace_bytes(shape)) return NCN_ERR_WORKSPACE;
+    if (!aligned16(y) || !aligned16(ya) || !aligned16(dy) || !aligned16(dya) || !aligned16(dx) || !aligned16(dxa) ||
+        !aligned16(x_rec) || !aligned16(xa_rec) || !aligned16(W) || !aligned16(dW) || !aligned16(workspace))
+        return NCN_ERR_ALIGN;
+    const Plan p = make_plan(shape, activation);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    float* partials = static_cast<float*>(workspace);
+    float* level1 = partials + (int64_t)kMaxGridX * 2 * shape->E;
+    const int64_t wstride = 2 * shape->E;
+    const std::vector<RadixPass> passes = plan_radix(shape, first_level, n_levels, true);
+    // last pass first; the first one to run reads y, ya, dy, dya, the others run in place on x_rec, xa_rec, dx, dxa
+    for (size_t e = 0; e < passes.size(); ++e) {
+        const RadixPass& ps = passes[passes.size() - 1 - e];
+        const bool top = (e == 0);
+        hipError_t err;
+        if (ps.single) {
+            StageArgs a{};
+            Grouping g{nullptr, nullptr, first_level + ps.first};
+            fill_common(a, shape, p, 0, alpha, m, activation, g, 0);
+            a.in0 = top ? y : x_rec; a.in1 = top ? ya : xa_rec; a.in_dtype = top ? y_dtype : NCN_F32;
+            a.g0 = top ? dy : dx; a.g1 = top ? dya : dxa; a.g_dtype = top ? dy_dtype : NCN_F32;
+            a.out0 = dx; a.out1 = dxa; a.out_dtype = dx_dtype;
+            a.aux0 = x_rec; a.aux1 = xa_rec;
+            a.W = W + ps.first * wstride;
+            a.dw_partials = partials;
+            err = (p.path != 2) ? launch_generic(kBackward, a, shape->n_head, p.grid_x, s)
+                                : launch_fast_backward_indexed(a, shape->n_head, p.grid_x, s);
+            if (err != hipSuccess) return (int)err;
+            err = launch_reduce_dw(partials, p.partial_rows, wstride, wstride, level1, dW + ps.first * wstride, s);
+        } else {
+            FusedArgs a{};
+            a.in0 = top ? y : x_rec; a.in1 = top ? ya : xa_rec; a.in_dtype = top ? y_dtype : NCN_F32;
+            a.g0 = top ? dy : dx; a.g1 = top ? dya : dxa; a.g_dtype = top ? dy_dtype : NCN_F32;
+            a.out0 = dx; a.out1 = dxa; a.out_dtype = dx_dtype;
+            a.aux0 = x_rec; a.aux1 = xa_rec;
+            a.W = W + ps.first * wstride;
+            a.dw_partials = partials;
+            fill_step_table(a.tab, shape->n_cache, alpha, m, activation);
+            err = launch_fused_radix(true, a, shape, ps, s);
+            if (err != hipSuccess) return (int)err;
+            const int rows = radix_grid(shape, ps, true) / shape->n_head;
+            err = launch_reduce_dw(partials, rows, (int64_t)ps.count * wstride, (int64_t)ps.count * wstride, level1,
+                                   dW + ps.first * wstride, s);
+        }
+        if (err != hipSuccess) return (int)err;
+    }
+    return NCN_OK;
+}
+
+int ncn_plan_radix(const ncn_shape* shape, int first_level, int n_levels, int activation, int backward, int32_t* out,
+                   int max_passes) {
+    int rc = check_shape(shape, 0, n_levels, activation);
+    if (rc != NCN_OK) return rc;
+    rc = check_radix(shape, first_level, n_levels);
+    if (rc != NCN_OK) return rc;
+    const std::vector<RadixPass> passes = plan_radix(shape, first_level, n_levels, backward != 0);
+    int k = 0;
+    for (const RadixPass& p : passes) {
+        if (out && k < max_passes) {
+            int32_t* o = out + 6 * k;
+            o[0] = p.first; o[1] = p.count; o[2] = p.single ? 0 : 1;
+            o[3] = (int32_t)p.s0; o[4] = (int32_t)p.span; o[5] = (int32_t)p.rows;
+        }
+        ++k;
+    }
+    return k;
 }
 
 }  // extern "C"

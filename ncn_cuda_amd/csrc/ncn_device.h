@@ -30,8 +30,9 @@ struct StepTable {
 //   inverse : in0,in1 = y,ya        out0,out1 = x,xa
 //   backward: in0,in1 = y,ya        g0,g1 = dy,dya (g1 may be null = zeros)
 //             out0,out1 = dx,dxa    aux0,aux1 = optional float32 reconstructed x,xa
-// Grouping: slot o of group g sits at position table[g * n_cache + o] when a table is given, else at the stride
-// permutation's ((g + o * stride) % groups) * n_cache + o.  With ctx_len, batch entry b only has its first
+// Grouping: slot o of group g sits at position table[g * n_cache + o] when a table is given, at the radix-n digit
+// position (g div s) * n * s + o * s + g mod s when radix_stride = s is set, else at the stride permutation's
+// ((g + o * stride) % groups) * n_cache + o.  With ctx_len, batch entry b only has its first
 // ctx_len[b] slots (in group order); the launches split the work: `edge == 0` runs the groups that are wholly
 // live, `edge == 1` (generic kernel only) the one partly live group of each batch entry.
 struct StageArgs {
@@ -57,6 +58,8 @@ struct StageArgs {
     int32_t in_dtype, g_dtype, out_dtype;
     int32_t activation;
     int32_t edge;
+    uint32_t radix_stride;   // n_cache^level: groups are the radix-n digit groups of that level (0: not used)
+    uint32_t reserved;
     StepTable tab;
 };
 
@@ -259,6 +262,10 @@ __device__ __forceinline__ int64_t slot_position(const StageArgs& A, uint32_t gr
     if (A.table) {
         const int32_t p = A.table[(int64_t)group * A.n_cache + slot];
         return (int64_t)max(0, min(p, (int32_t)A.N - 1));
+    }
+    if (A.radix_stride) {   // the positions that differ only in one base-n digit (ncn_triton/group_tensors.py:8-18)
+        const uint32_t s = A.radix_stride, hi = group / s;
+        return ((int64_t)hi * A.n_cache + slot) * s + (group - hi * s);
     }
     return (int64_t)stage_block(A, group, slot) * A.n_cache + slot;
 }

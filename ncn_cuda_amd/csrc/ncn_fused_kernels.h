@@ -24,6 +24,13 @@
 // whole pass (the step counter just keeps counting across stages; backward keeps p = (1-m) g + h in place of h),
 // so true values exist only in HBM.  The pass's weights sit in LDS.  Backward sums each wave's dW share of a stage into a per-wave LDS
 // slot (one writer per slot, fixed order: deterministic) and leaves one partial row per workgroup and stage.
+//
+// RADIX builds of the same kernels run levels of the radix-n digit grouping (ncn_triton/group_tensors.py:8-18)
+// instead: level l groups the n_cache positions that differ only in base-n_cache digit l.  A run of levels a .. a+k-1
+// only ever mixes the positions lower + n^a * d + n^(a+k) * upper, d = 0 .. n^k - 1, of one (lower, upper): a closed
+// window of n^k rows, no halo at all, any pass may run in place.  A workgroup holds rows / n^k such windows; the LDS
+// row of digit string d is d itself, and level a+j pairs the rows whose d differ in digit j.  (n_cache 2 and 4
+// only: every size below is a power of two and the digit arithmetic is shifts.)
 #pragma once
 #include "ncn_stage_kernels.h"
 
@@ -50,6 +57,8 @@ struct FusedArgs {
     int64_t N, E;
     int32_t n_head, n_stages;
     int32_t in_dtype, g_dtype, out_dtype, reserved;
+    // RADIX builds read: class_stride = n^a in rows, ring = n^k rows per window, window = rows / n_cache,
+    // class_groups = workgroup-loads per batch entry, sub_stride[j] = n^j in rows, closed = 1
     uint32_t class_stride;    // S0, in blocks
     uint32_t ring;            // sub-blocks per class = groups / S0 (power of two)
     uint32_t window;          // sub-blocks held in LDS
@@ -70,7 +79,9 @@ struct FusedItem {
     int64_t base;  // element offset of (batch, row 0, head slice)
 };
 
-template <int EC>
+__device__ __forceinline__ uint32_t log2u(uint32_t v) { return 31u - (uint32_t)__clz((int)v); }
+
+template <int NC, int EC, bool RADIX>
 __device__ __forceinline__ FusedItem fused_item(const FusedArgs& A, uint32_t item) {
     FusedItem it;
     it.head = item % A.n_head;
@@ -79,7 +90,12 @@ __device__ __forceinline__ FusedItem fused_item(const FusedArgs& A, uint32_t ite
     t /= A.tiles_per_ring;
     const uint32_t cg = t % A.class_groups;
     const uint32_t b = t / A.class_groups;
-    if (A.closed) {
+    if (RADIX) {
+        it.cls = cg * (A.window * NC / A.ring);   // number of the first window: (upper, lower) = (u / n^a, u % n^a)
+        it.sub0 = 0u;
+        it.own_lo = 0u;
+        it.own_cnt = A.window;
+    } else if (A.closed) {
         it.cls = cg * (A.window / A.ring);   // first class of the window
         it.sub0 = 0u;
         it.own_lo = 0u;
@@ -96,8 +112,15 @@ __device__ __forceinline__ FusedItem fused_item(const FusedArgs& A, uint32_t ite
 }
 
 // element offset (without the feature) of local row `lr` = (window sub-block qi) * NC + slot
-template <int NC>
+template <int NC, bool RADIX>
 __device__ __forceinline__ int64_t fused_row_offset(const FusedArgs& A, const FusedItem& it, uint32_t lr) {
+    if (RADIX) {
+        const uint32_t lg_span = log2u(A.ring), lg_s0 = log2u(A.class_stride);
+        const uint32_t d = lr & (A.ring - 1u), u = it.cls + (lr >> lg_span);
+        const int64_t pos = (int64_t)(u & (A.class_stride - 1u)) + ((int64_t)d << lg_s0) +
+                            ((int64_t)(u >> lg_s0) << (lg_s0 + lg_span));
+        return it.base + pos * A.E;
+    }
     const uint32_t qi = lr / NC, o = lr - qi * NC;
     const uint32_t sub = (it.sub0 + qi) & (A.ring - 1u);
     const uint32_t cls = A.closed ? it.cls + qi / A.ring : it.cls;
@@ -106,8 +129,17 @@ __device__ __forceinline__ int64_t fused_row_offset(const FusedArgs& A, const Fu
 }
 
 // LDS row of slot i of the group whose slot-0 sub-block is window position qg
-template <int NC>
+// (RADIX: row of digit i at level log_n(sstride) of group qg; groups are numbered window by window)
+template <int NC, bool RADIX>
 __device__ __forceinline__ uint32_t fused_lds_row(const FusedArgs& A, uint32_t qg, uint32_t i, uint32_t sstride) {
+    if (RADIX) {
+        constexpr uint32_t lg_nc = NC == 2 ? 1u : 2u;
+        static_assert(NC == 2 || NC == 4, "digit arithmetic by shifts");
+        const uint32_t lg_span = log2u(A.ring), lg_sj = log2u(sstride);
+        const uint32_t gpw = A.ring >> lg_nc;                       // groups per window
+        const uint32_t wq = qg >> (lg_span - lg_nc), g = qg & (gpw - 1u);
+        return (wq << lg_span) + ((g >> lg_sj) << (lg_sj + lg_nc)) + (i << lg_sj) + (g & (sstride - 1u));
+    }
     uint32_t qi = qg + i * sstride;
     if (A.closed) qi = (qg & ~(A.ring - 1u)) | (qi & (A.ring - 1u));  // wrap inside the group's own ring
     return qi * NC + i;
@@ -131,7 +163,7 @@ __device__ __forceinline__ void lds_store_frag(float* row, const float (&v)[F]) 
 // Window rows on their way from global memory to LDS: 4 features per thread and trip, kept as raw bits so that
 // nothing waits for the loads until fused_commit_rows turns them into floats.  A workgroup fetches the window of
 // its next item while it computes the current one.
-template <int NC, int EC, int NW, int K>
+template <int NC, int EC, int NW, int K, bool RADIX>
 __device__ __forceinline__ void fused_window_offsets(const FusedArgs& A, const FusedItem& it, uint32_t rows,
                                                      int64_t (&off)[K]) {
     constexpr uint32_t CPR = EC / 4;
@@ -140,7 +172,7 @@ __device__ __forceinline__ void fused_window_offsets(const FusedArgs& A, const F
         // a trip past the end re-reads the last chunk, which fused_commit_rows ignores
         const uint32_t c = min(threadIdx.x + k * 64 * NW, rows * CPR - 1u);
         const uint32_t lr = c / CPR, c4 = c - lr * CPR;
-        off[k] = fused_row_offset<NC>(A, it, lr) + c4 * 4;
+        off[k] = fused_row_offset<NC, RADIX>(A, it, lr) + c4 * 4;
     }
 }
 
@@ -186,7 +218,7 @@ __device__ __forceinline__ void fused_commit_rows(const uint4 (&raw)[K], int dty
 }
 
 // LDS -> global for the owned rows, each value times `scale`
-template <int NC, int EC, int NW>
+template <int NC, int EC, int NW, bool RADIX>
 __device__ __forceinline__ void fused_store_rows_scaled(const FusedArgs& A, const FusedItem& it, const float* src,
                                                         float scale, void* dst, int dtype, float* copy32) {
     constexpr uint32_t CPR = EC / 4;
@@ -197,7 +229,7 @@ __device__ __forceinline__ void fused_store_rows_scaled(const FusedArgs& A, cons
         lds_load_frag<4>(src + lr * EC + c4 * 4, v);
 #pragma unroll
         for (int k = 0; k < 4; ++k) v[k] *= scale;
-        const int64_t off = fused_row_offset<NC>(A, it, lr) + c4 * 4;
+        const int64_t off = fused_row_offset<NC, RADIX>(A, it, lr) + c4 * 4;
         store_frag<4>(dst, dtype, off, true, v);
         if (copy32) store_frag<4>(copy32, NCN_F32, off, true, v);
     }
@@ -213,7 +245,7 @@ __device__ __forceinline__ void fused_load_weights(const FusedArgs& A, int head,
 }
 
 // TANH_ONLY as in the one-stage kernels: the tanh build has no branch on the activation code.
-template <int NC, int EC, int R, int F, bool TANH_ONLY>
+template <int NC, int EC, int R, int F, bool TANH_ONLY, bool RADIX = false>
 __global__ void __launch_bounds__(64 * kFusedWavesFwd) fused_forward_kernel(const FusedArgs A) {
     constexpr int NW = kFusedWavesFwd;
     using T = Tile<NC, EC, R, F>;
@@ -233,18 +265,18 @@ __global__ void __launch_bounds__(64 * kFusedWavesFwd) fused_forward_kernel(cons
     uint4 rx[K], ra[K];
     if (blockIdx.x < A.total_items) {
         int64_t off[K];
-        fused_window_offsets<NC, EC, NW, K>(A, fused_item<EC>(A, blockIdx.x), rows, off);
+        fused_window_offsets<NC, EC, NW, K, RADIX>(A, fused_item<NC, EC, RADIX>(A, blockIdx.x), rows, off);
         fused_fetch_rows<K>(A.in0, A.in_dtype, off, rx);
         fused_fetch_rows<K>(A.in1, A.in_dtype, off, ra);
     }
     for (uint32_t item = blockIdx.x; item < A.total_items; item += gridDim.x) {
-        const FusedItem it = fused_item<EC>(A, item);
+        const FusedItem it = fused_item<NC, EC, RADIX>(A, item);
         fused_commit_rows<EC, NW, K>(rx, A.in_dtype, xs, rows);
         fused_commit_rows<EC, NW, K>(ra, A.in_dtype, as, rows);
         __syncthreads();
         if (item + gridDim.x < A.total_items) {   // the next window travels while this one is computed
             int64_t off[K];
-            fused_window_offsets<NC, EC, NW, K>(A, fused_item<EC>(A, item + gridDim.x), rows, off);
+            fused_window_offsets<NC, EC, NW, K, RADIX>(A, fused_item<NC, EC, RADIX>(A, item + gridDim.x), rows, off);
             fused_fetch_rows<K>(A.in0, A.in_dtype, off, rx);
             fused_fetch_rows<K>(A.in1, A.in_dtype, off, ra);
         }
@@ -261,7 +293,7 @@ __global__ void __launch_bounds__(64 * kFusedWavesFwd) fused_forward_kernel(cons
                 uint32_t row[R];
 #pragma unroll
                 for (int rr = 0; rr < R; ++rr) {
-                    row[rr] = fused_lds_row<NC>(A, valid ? qg : 0u, rl * R + rr, ss) * EC + fl * F;
+                    row[rr] = fused_lds_row<NC, RADIX>(A, valid ? qg : 0u, rl * R + rr, ss) * EC + fl * F;
                     lds_load_frag<F>(xs + row[rr], x[rr]);
                     lds_load_frag<F>(as + row[rr], a[rr]);
                 }
@@ -276,13 +308,13 @@ __global__ void __launch_bounds__(64 * kFusedWavesFwd) fused_forward_kernel(cons
             }
             __syncthreads();
         }
-        fused_store_rows_scaled<NC, EC, NW>(A, it, xs, A.scale_dn, A.out0, A.out_dtype, A.aux0);
-        fused_store_rows_scaled<NC, EC, NW>(A, it, as, A.scale_dn, A.out1, A.out_dtype, A.aux1);
+        fused_store_rows_scaled<NC, EC, NW, RADIX>(A, it, xs, A.scale_dn, A.out0, A.out_dtype, A.aux0);
+        fused_store_rows_scaled<NC, EC, NW, RADIX>(A, it, as, A.scale_dn, A.out1, A.out_dtype, A.aux1);
         __syncthreads();
     }
 }
 
-template <int NC, int EC, int R, int F, bool TANH_ONLY>
+template <int NC, int EC, int R, int F, bool TANH_ONLY, bool RADIX = false>
 __global__ void __launch_bounds__(64 * kFusedWavesBwd, TANH_ONLY ? 4 : 1) fused_backward_kernel(const FusedArgs A) {
     constexpr int NW = kFusedWavesBwd;
     using T = Tile<NC, EC, R, F>;
@@ -315,7 +347,7 @@ __global__ void __launch_bounds__(64 * kFusedWavesBwd, TANH_ONLY ? 4 : 1) fused_
     };
     auto fetch = [&](uint32_t item, Raw& r) {
         int64_t off[K];
-        fused_window_offsets<NC, EC, NW, K>(A, fused_item<EC>(A, item), rows, off);
+        fused_window_offsets<NC, EC, NW, K, RADIX>(A, fused_item<NC, EC, RADIX>(A, item), rows, off);
         fused_fetch_rows<K>(A.in0, A.in_dtype, off, r.y);
         fused_fetch_rows<K>(A.in1, A.in_dtype, off, r.b);
         fused_fetch_rows<K>(A.g0, A.g_dtype, off, r.g);
@@ -346,7 +378,7 @@ __global__ void __launch_bounds__(64 * kFusedWavesBwd, TANH_ONLY ? 4 : 1) fused_
     }
     __syncthreads();
     for (uint32_t item = blockIdx.x; item < A.total_items; item += gridDim.x) {
-        const FusedItem it = fused_item<EC>(A, item);
+        const FusedItem it = fused_item<NC, EC, RADIX>(A, item);
         for (int st = A.n_stages - 1; st >= 0; --st) {
             const uint32_t ss = A.sub_stride[st];
             const uint32_t ngroups = A.closed ? A.window : A.window - (NC - 1) * ss;
@@ -363,7 +395,7 @@ __global__ void __launch_bounds__(64 * kFusedWavesBwd, TANH_ONLY ? 4 : 1) fused_
                 uint32_t row[R];
 #pragma unroll
                 for (int rr = 0; rr < R; ++rr) {
-                    row[rr] = fused_lds_row<NC>(A, valid ? qg : 0u, rl * R + rr, ss) * EC + fl * F;
+                    row[rr] = fused_lds_row<NC, RADIX>(A, valid ? qg : 0u, rl * R + rr, ss) * EC + fl * F;
                     lds_load_frag<F>(ys + row[rr], Y[rr]);
                     lds_load_frag<F>(bs + row[rr], B[rr]);
                     lds_load_frag<F>(gs + row[rr], G[rr]);
@@ -407,7 +439,7 @@ __global__ void __launch_bounds__(64 * kFusedWavesBwd, TANH_ONLY ? 4 : 1) fused_
             const uint32_t r0 = it.own_lo * NC, nrows = it.own_cnt * NC;
             for (uint32_t c = threadIdx.x; c < nrows * CPR; c += 64 * NW) {
                 const uint32_t lr = r0 + c / CPR, c4 = c % CPR;
-                const int64_t off = fused_row_offset<NC>(A, it, lr) + c4 * 4;
+                const int64_t off = fused_row_offset<NC, RADIX>(A, it, lr) + c4 * 4;
                 float g[4], h[4];
                 lds_load_frag<4>(gs + lr * EC + c4 * 4, g);
                 lds_load_frag<4>(ps + lr * EC + c4 * 4, h);
@@ -420,8 +452,8 @@ __global__ void __launch_bounds__(64 * kFusedWavesBwd, TANH_ONLY ? 4 : 1) fused_
                 store_frag<4>(A.out1, A.out_dtype, off, true, h);
             }
             if (A.aux0) {
-                fused_store_rows_scaled<NC, EC, NW>(A, it, ys, A.scale_up, A.aux0, NCN_F32, nullptr);
-                fused_store_rows_scaled<NC, EC, NW>(A, it, bs, A.scale_up, A.aux1, NCN_F32, nullptr);
+                fused_store_rows_scaled<NC, EC, NW, RADIX>(A, it, ys, A.scale_up, A.aux0, NCN_F32, nullptr);
+                fused_store_rows_scaled<NC, EC, NW, RADIX>(A, it, bs, A.scale_up, A.aux1, NCN_F32, nullptr);
             }
         };
         if (item + gridDim.x < A.total_items) {   // the same for the whole workgroup

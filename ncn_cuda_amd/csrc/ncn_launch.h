@@ -71,4 +71,19 @@ std::vector<FusedPass> plan_fused(const ncn_shape* sh, int first, int count, boo
 int fused_grid(const ncn_shape* sh, const FusedPass& p, bool backward);
 hipError_t launch_fused(bool backward, FusedArgs& a, const ncn_shape* sh, const FusedPass& p, hipStream_t s);
 
+
+// ---- multi-stage passes over radix-n levels, ncn_fused_radix.hip ---------------------------------------------
+struct RadixPass {
+    int first, count;  // levels [first, first + count) relative to the range that was planned
+    int single;        // 1: one level, run with the one-stage kernel
+    uint32_t s0;       // n^(first level of the pass): distance in rows between the rows of a window
+    uint32_t span;     // n^count: rows of a window
+    uint32_t rows;     // rows a workgroup holds (a whole number of windows)
+    uint32_t loads;    // workgroup-loads per batch entry and head
+};
+bool radix_fused_supported(const ncn_shape* sh);
+std::vector<RadixPass> plan_radix(const ncn_shape* sh, int first, int count, bool backward);
+int radix_grid(const ncn_shape* sh, const RadixPass& p, bool backward);
+hipError_t launch_fused_radix(bool backward, FusedArgs& a, const ncn_shape* sh, const RadixPass& p, hipStream_t s);
+
 }  // namespace ncn

@@ -269,6 +269,58 @@ def inverse_stages(y, ya, W, alpha, activation, cache_dim, nhead, first_stage, n
     return x, xa
 
 
+def forward_radix(x, xa, W, alpha, activation, cache_dim, nhead, first_level, n_levels, *, m=M_DEFAULT,
+                  out_dtype=None):
+    """Levels first_level .. first_level+n_levels-1 of the radix-n digit grouping (ncn_triton/group_tensors.py:8-18)
+    without index tensors; W: [n_levels, 2E].  Several levels per pass stay in LDS for n_cache 2 and 4.  Outputs are
+    float32 unless out_dtype says otherwise (values between passes live in the outputs)."""
+    shape = validate(x, xa, W, cache_dim, nhead, activation, 0, n_levels)
+    dev = _require_gpu(x, xa, W)
+    x, xa, w = _prep(x.detach()), _prep(xa.detach()), _w32(W)
+    out_dtype = torch.float32 if out_dtype is None else out_dtype
+    y = torch.empty(x.shape, dtype=out_dtype, device=dev)
+    ya = torch.empty(x.shape, dtype=out_dtype, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.load().ncn_forward_radix(_ptr(x), _ptr(xa), _DTYPES[x.dtype], _ptr(y), _ptr(ya), _DTYPES[out_dtype],
+                                           _ptr(None), _ptr(None), _ptr(w), ctypes.byref(shape), int(first_level),
+                                           int(n_levels), float(alpha), float(m), int(activation), _stream(dev))
+    if rc == -2:
+        raise ValueError(f"radix levels {first_level}..{first_level + n_levels - 1}: n_cache^(last level + 1) must "
+                         f"divide N = {x.shape[1]}")
+    _lib.check(rc, "ncn_forward_radix")
+    return y, ya
+
+
+def backward_radix(y, ya, dy, dya, W, alpha, activation, cache_dim, nhead, first_level, n_levels, *, m=M_DEFAULT):
+    """Reversible backward of forward_radix from its outputs.  Returns (x_rec, xa_rec, dx, dxa, dW[n_levels, 2E]), all
+    float32."""
+    shape = validate(y, ya, W, cache_dim, nhead, activation, 0, n_levels, what="y")
+    if dy.shape != y.shape or (dya is not None and dya.shape != y.shape):
+        raise ValueError("dy/dya must have the shape of y")
+    if dy.dtype not in _DTYPES or (dya is not None and dya.dtype != dy.dtype):
+        raise TypeError("dy and dya must both be float32 or bfloat16")
+    dev = _require_gpu(y, ya, dy, dya, W)
+    y, ya, dy, w = _prep(y.detach()), _prep(ya.detach()), _prep(dy.detach()), _w32(W)
+    dya = _prep(dya.detach()) if dya is not None else None
+    f32 = torch.float32
+    dx, dxa = torch.empty(y.shape, dtype=f32, device=dev), torch.empty(y.shape, dtype=f32, device=dev)
+    x_rec, xa_rec = torch.empty(y.shape, dtype=f32, device=dev), torch.empty(y.shape, dtype=f32, device=dev)
+    dW = torch.empty(n_levels, 2 * y.shape[2], dtype=f32, device=dev)
+    lib = _lib.load()
+    ws_bytes = lib.ncn_workspace_bytes(ctypes.byref(shape))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        rc = lib.ncn_backward_radix(_ptr(y), _ptr(ya), _DTYPES[y.dtype], _ptr(dy), _ptr(dya), _DTYPES[dy.dtype],
+                                    _ptr(dx), _ptr(dxa), _lib.NCN_F32, _ptr(x_rec), _ptr(xa_rec), _ptr(w), _ptr(dW),
+                                    _ptr(ws), ctypes.c_size_t(ws_bytes), ctypes.byref(shape), int(first_level),
+                                    int(n_levels), float(alpha), float(m), int(activation), _stream(dev))
+    if rc == -2:
+        raise ValueError(f"radix levels {first_level}..{first_level + n_levels - 1}: n_cache^(last level + 1) must "
+                         f"divide N = {y.shape[1]}")
+    _lib.check(rc, "ncn_backward_radix")
+    return x_rec, xa_rec, dx, dxa, dW
+
+
 # ---- the reference module's two callables (ncn_cuda/ncn_cuda.cpp:3-25) -------------------------------------
 def forward(X, Xa, W, alpha, activation, cache_dim, nhead, module_l):
     y, ya = forward_stages(X, Xa, W, alpha, activation, cache_dim, nhead, module_l, 1)

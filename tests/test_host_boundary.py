@@ -122,6 +122,33 @@ def test_indexed_entry_points_reject_bad_arguments_before_touching_the_gpu(lib):
     assert h.ncn_backward_indexed(*args, p, ctypes.c_size_t(ws), p, p, ctypes.byref(bad), 0, 1, 0.9, 0.9, 0, z) == -2
 
 
+def test_radix_plan_and_argument_checks(lib):
+    h = lib.load()
+    buf = (ctypes.c_int32 * 96)()
+    deep = _shape(lib, 128, 8192, 128, 4, 2)
+    assert h.ncn_plan_radix(ctypes.byref(deep), 0, 13, 0, 0, buf, 16) == 2
+    assert list(buf[0:6]) == [0, 8, 1, 1, 256, 256] and list(buf[6:12]) == [8, 5, 1, 256, 32, 256]
+    assert h.ncn_plan_radix(ctypes.byref(deep), 0, 13, 0, 1, buf, 16) == 2
+    assert list(buf[0:6]) == [0, 7, 1, 1, 128, 128] and list(buf[6:12]) == [7, 6, 1, 128, 64, 128]
+    assert h.ncn_plan_radix(ctypes.byref(deep), 0, 14, 0, 0, None, 0) == -2          # 2^14 > N
+    assert h.ncn_plan_radix(ctypes.byref(_shape(lib, 2, 96, 32, 2, 2)), 0, 6, 0, 0, None, 0) == -2   # 64 does not divide 96
+    assert h.ncn_plan_radix(ctypes.byref(_shape(lib, 2, 96, 32, 2, 2)), 0, 5, 0, 0, buf, 16) == 1
+    assert list(buf[0:6]) == [0, 5, 1, 1, 32, 96]                                    # three windows per workgroup
+    small = _shape(lib, 2, 64, 32, 4, 4)
+    p = ctypes.c_void_p(4096)       # never dereferenced: every call below fails validation first
+    z = ctypes.c_void_p(0)
+    fwd = lambda x, first, count: h.ncn_forward_radix(x, p, 0, p, p, 0, z, z, p, ctypes.byref(small), first, count,
+                                                      0.9, 0.9, 0, z)
+    assert fwd(z, 0, 3) == -1
+    assert fwd(p, 0, 4) == -2 and fwd(p, 2, 2) == -2 and fwd(p, -1, 1) == -2
+    args = [p, p, 0, p, p, 0, p, p, 0, z, z, p, p]
+    ws = h.ncn_workspace_bytes(ctypes.byref(small))
+    bwd = lambda nbytes, count, dxt=0: h.ncn_backward_radix(*args[:8], dxt, *args[9:], p, ctypes.c_size_t(nbytes),
+                                                            ctypes.byref(small), 0, count, 0.9, 0.9, 0, z)
+    assert bwd(ws - 1, 1) == -5
+    assert bwd(ws, 3) == -8             # several levels carry their state in x_rec, xa_rec
+
+
 def test_python_grouping_validation():
     from ncn_cuda_amd import ncn_cuda_module as M
     good = torch.randperm(64)
