@@ -19,8 +19,9 @@ from torch import nn
 
 from . import ncn_cuda_module
 
-__all__ = ["ACTIVATION_CODES", "NCNFunction", "NCNNetFunction", "NCNModuleCuda", "NCNNetCuda", "NCNNetTestCuda",
-           "default_save_every", "fused_ncn_cuda_v2", "fused_ncn_net", "ncn_inverse"]
+__all__ = ["ACTIVATION_CODES", "NCNFunction", "NCNNetFunction", "NCNRadixNetFunction", "NCNModuleCuda", "NCNNetCuda",
+           "NCNNetTestCuda", "default_save_every", "fused_ncn_cuda_v2", "fused_ncn_net", "fused_ncn_radix_net",
+           "ncn_inverse"]
 
 # names and codes of ncn_pytorch_wrapper_v2.py:111, plus the leaky relu of the Triton kernels (ncn_triton.py:101)
 ACTIVATION_CODES = {"tanh": 0, "relu": 1, "sigmoid": 2, "linear": -1, "leaky-relu": 3}
@@ -100,6 +101,47 @@ class NCNNetFunction(torch.autograd.Function):
             for j in range(cnt):
                 dWs[a + j] = dW[j].reshape(w_shapes[a + j]).to(w_dtypes[a + j])
         return (g.to(io_dtype), ga.to(io_dtype), None, None, None, None, None, None, *dWs)
+
+
+class NCNRadixNetFunction(torch.autograd.Function):
+    """Like NCNNetFunction, for levels first_level .. of the radix-n digit grouping (ncn_triton/group_tensors.py:8-18)
+    instead of the stride permutation: weights[k] belongs to level first_level + k."""
+
+    @staticmethod
+    def forward(ctx, x, xa, alpha, activation, n_cache, n_head, first_level, save_every, *weights):
+        L = len(weights)
+        save_every = default_save_every(n_cache) if not save_every else int(save_every)
+        W = torch.stack([w.detach().reshape(-1).to(torch.float32) for w in weights])
+        saved = []
+        cx, cxa = x, xa
+        segs = [(a, min(save_every, L - a)) for a in range(0, L, save_every)]
+        for a, cnt in segs:
+            cx, cxa = ncn_cuda_module.forward_radix(cx, cxa, W[a:a + cnt], alpha, activation, n_cache, n_head,
+                                                    first_level + a, cnt)
+            saved.extend([cx, cxa])
+        ctx.save_for_backward(W, *saved)
+        ctx.cfg = (alpha, activation, n_cache, n_head, first_level, segs, x.dtype, [w.dtype for w in weights],
+                   [w.shape for w in weights])
+        return cx.to(x.dtype), cxa.to(x.dtype)
+
+    @staticmethod
+    def backward(ctx, dyi, dya):
+        W, *saved = ctx.saved_tensors
+        alpha, activation, n_cache, n_head, first_level, segs, io_dtype, w_dtypes, w_shapes = ctx.cfg
+        dWs = [None] * W.shape[0]
+        g, ga = dyi, dya
+        for k in range(len(segs) - 1, -1, -1):
+            a, cnt = segs[k]
+            _, _, g, ga, dW = ncn_cuda_module.backward_radix(saved[2 * k], saved[2 * k + 1], g, ga, W[a:a + cnt], alpha,
+                                                             activation, n_cache, n_head, first_level + a, cnt)
+            for j in range(cnt):
+                dWs[a + j] = dW[j].reshape(w_shapes[a + j]).to(w_dtypes[a + j])
+        return (g.to(io_dtype), ga.to(io_dtype), None, None, None, None, None, None, *dWs)
+
+
+def fused_ncn_radix_net(x, xa, weights, alpha, activation, n_cache, n_head, first_level=0, save_every=None):
+    """Radix levels first_level .. first_level+len(weights)-1 as one autograd node; activation is the int code."""
+    return NCNRadixNetFunction.apply(x, xa, alpha, activation, n_cache, n_head, first_level, save_every, *weights)
 
 
 def fused_ncn_net(x, xa, weights, alpha, activation, n_cache, n_head, first_stage=0, save_every=None):

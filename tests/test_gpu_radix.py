@@ -94,3 +94,22 @@ def test_radix_bf16_input_and_other_activation(M):
     _, _, dx, dxa, dW = M.backward_radix(y, ya, dy.cuda(), dya.cuda(), W, 0.9, 2, n, C, 0, L)
     tol = 2e-6 * (1 / 0.9) ** (n * L)
     assert O.rel_err(dx, ref[2]) < tol and O.rel_err(dW[0], ref[4][0]) < tol and O.rel_err(dW[L - 1], ref[4][L - 1]) < tol
+
+
+def test_radix_net_autograd_node(M):
+    """fused_ncn_radix_net through torch autograd, bf16 in and out, segments of 26 // n levels."""
+    import ncn_cuda_amd as pkg
+    batch, N, E, C, n, L = 2, 4096, 64, 2, 4, 6          # 4^6 = 4096; two saved segments of three levels
+    x, xa, Ws, dy, dya = O.make_inputs(batch, N, E, L, n, seed=43, xa_zero=False)
+    tables = [O.radix_group_table(N, n, l) for l in range(L)]
+    d = torch.float64
+    ref = O.net_autograd_indexed(x.to(d), xa.to(d), [w.to(d) for w in Ws], dy.to(d), dya.to(d), 0.9, n, C, tables)
+    gx, gxa = x.cuda().requires_grad_(), xa.cuda().requires_grad_()
+    gw = [w.cuda().requires_grad_() for w in Ws]
+    yi, ya = pkg.fused_ncn_radix_net(gx, gxa, gw, 0.9, 0, n, C, save_every=3)
+    torch.autograd.backward([yi, ya], [dy.cuda(), dya.cuda()])
+    tol = 2e-6 * (1 / 0.9) ** (n * 3)
+    assert O.rel_err(yi, ref[0]) < 1e-5 and O.rel_err(ya, ref[1]) < 1e-5
+    assert O.rel_err(gx.grad, ref[2]) < tol and O.rel_err(gxa.grad, ref[3]) < tol
+    for l in range(L):
+        assert gw[l].grad.shape == gw[l].shape and O.rel_err(gw[l].grad, ref[4][l]) < tol
