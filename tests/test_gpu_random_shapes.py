@@ -96,3 +96,19 @@ def test_random_problem(M, case):
     if act != 3:
         assert O.rel_err(idx, iref[2]) < gtol and O.rel_err(idxa, iref[3]) < gtol
         assert O.rel_err(idW[0], iref[4][0]) < gtol
+    # the first levels of the radix-n grouping that N admits, without tables
+    levels = 0
+    while n > 1 and levels < L and N % n ** (levels + 1) == 0:
+        levels += 1
+    if levels:
+        rtables = [O.radix_group_table(N, n, l) for l in range(levels)]
+        rref = O.net_autograd_indexed(x.to(d), xa.to(d), [w.to(d) for w in Ws[:levels]], dy.to(d), dya.to(d), alpha, n, C,
+                                      rtables, activation=act)
+        ry, rya = M.forward_radix(gx, gxa, W[:levels], alpha, act, n, C, 0, levels)
+        assert O.rel_err(ry, rref[0]) < 1e-5 and O.rel_err(rya, rref[1]) < 1e-5
+        if (1 / 0.9) ** (n * levels) < 50 and act != 3:
+            rxr, _, rdx, rdxa, rdW = M.backward_radix(ry, rya, gdy, gdya, W[:levels], alpha, act, n, C, 0, levels)
+            tol = max(1e-5, 2e-6 * (1 / 0.9) ** (n * levels))
+            assert O.rel_err(rdx, rref[2]) < tol and O.rel_err(rdxa, rref[3]) < tol and O.rel_err(rxr, x) < tol
+            for l in range(levels):
+                assert O.rel_err(rdW[l], rref[4][l]) < tol
