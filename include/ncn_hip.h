@@ -127,7 +127,9 @@ int ncn_backward(const void* y, const void* ya, int y_dtype,
  * Inverse of stages first_stage+n_stages-1 .. first_stage: x, xa such that ncn_forward(x, xa) = y, ya.
  * Follows NCNFunctionPytorch.invert (torch_ref/ncn_pytorch_invertible.py:87-113), which the
  * reference's CUDA module only runs inside backward (ncn_bwd_cuda_kernel.cu:88-115).
- * May run in place (x == y, xa == ya) when the dtypes are equal.
+ * May run in place (x == y, xa == ya) when the dtypes are equal.  With n_stages > 1, float32 outputs and small
+ * groups it uses the multi-stage LDS passes that can work without scratch (every closed pass, and a halo pass when it
+ * is the first to run and x, xa are not y, ya) and one launch per stage for the rest.
  */
 int ncn_inverse(const void* y, const void* ya, int in_dtype,
                 void* x, void* xa, int out_dtype,
@@ -207,7 +209,14 @@ int ncn_backward_radix(const void* y, const void* ya, int y_dtype,
                        const ncn_shape* shape, int first_level, int n_levels,
                        float alpha, float m, int activation, void* stream);
 
-/* How the two calls above cut the levels into passes; returns the number of passes or a negative error code and
+/* Inverse of ncn_forward_radix: x, xa with ncn_forward_radix(x, xa) = y, ya; may run in place. */
+int ncn_inverse_radix(const void* y, const void* ya, int in_dtype,
+                      void* x, void* xa, int out_dtype,
+                      const float* W,
+                      const ncn_shape* shape, int first_level, int n_levels,
+                      float alpha, float m, int activation, void* stream);
+
+/* How the calls above cut the levels into passes (the inverse uses the forward's cut); returns the number of passes or a negative error code and
  * writes up to max_passes records of 6 int32 into `out` (may be NULL):
  *   [0] first level of the pass relative to first_level   [1] levels in the pass   [2] 0 one-stage launch, 1 LDS windows
  *   [3] n_cache^(first level): distance in rows between the rows of a window   [4] rows of a window   [5] rows per workgroup

@@ -12,7 +12,7 @@ NCN_F32, NCN_BF16 = 0, 1
 ACT_TANH, ACT_RELU, ACT_SIGMOID, ACT_LEAKY_RELU, ACT_LINEAR = 0, 1, 2, 3, -1
 
 EXPORTS = ("ncn_forward", "ncn_backward", "ncn_inverse", "ncn_forward_indexed", "ncn_backward_indexed",
-           "ncn_inverse_indexed", "ncn_forward_radix", "ncn_backward_radix", "ncn_plan_radix", "ncn_workspace_bytes", "ncn_workspace_bytes_stages",
+           "ncn_inverse_indexed", "ncn_forward_radix", "ncn_backward_radix", "ncn_inverse_radix", "ncn_plan_radix", "ncn_workspace_bytes", "ncn_workspace_bytes_stages",
            "ncn_plan_passes", "ncn_kernel_path",
            "ncn_check_shape", "ncn_error_string", "ncn_version")
 
@@ -56,6 +56,8 @@ def load():
     lib.ncn_backward_radix.restype = i
     lib.ncn_backward_radix.argtypes = [vp, vp, i, vp, vp, i, vp, vp, i, f32p, f32p, f32p, f32p, vp, ctypes.c_size_t,
                                        shp, i, i, fl, fl, i, vp]
+    lib.ncn_inverse_radix.restype = i
+    lib.ncn_inverse_radix.argtypes = [vp, vp, i, vp, vp, i, f32p, shp, i, i, fl, fl, i, vp]
     lib.ncn_plan_radix.restype = i
     lib.ncn_plan_radix.argtypes = [shp, i, i, i, i, ctypes.POINTER(ctypes.c_int32), i]
     lib.ncn_workspace_bytes.restype = ctypes.c_size_t

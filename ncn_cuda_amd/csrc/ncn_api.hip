@@ -337,7 +337,7 @@ static int forward_impl(const void* x, const void* xa, int in_dtype, void* y, vo
                 a.aux0 = last ? y32 : nullptr; a.aux1 = last ? ya32 : nullptr;
                 a.W = W + ps.first * wstride;
                 fill_step_table(a.tab, shape->n_cache, alpha, m, activation);
-                err = launch_fused(false, a, shape, ps, s);
+                err = launch_fused(kForward, a, shape, ps, s);
             }
             if (err != hipSuccess) return (int)err;
             cur0 = d0; cur1 = d1; cur_dtype = d_dtype;
@@ -379,6 +379,44 @@ static int inverse_impl(const void* y, const void* ya, int in_dtype, void* x, vo
     if (!aligned16(x) || !aligned16(xa) || !aligned16(y) || !aligned16(ya) || !aligned16(W)) return NCN_ERR_ALIGN;
     const Plan p = make_plan(shape, activation);
     hipStream_t s = static_cast<hipStream_t>(stream);
+
+    // several stages: LDS-resident passes, last pass of the range first.  There is no scratch to ping-pong with: the
+    // first pass to run goes from y, ya to x, xa and the others work in place on x, xa, which a halo pass must not,
+    // so the stages of such a pass are undone by one-stage launches (closed passes and one-stage launches may).
+    std::vector<FusedPass> passes;
+    if (grouping.plain() && (out_dtype == NCN_F32 || n_stages == 1))
+        passes = multi_stage_plan(shape, first_stage, n_stages, activation, false);
+    if (!passes.empty()) {
+        const int64_t wstride = 2 * shape->E;
+        const size_t np = passes.size();
+        for (size_t e = 0; e < np; ++e) {
+            const FusedPass& ps = passes[np - 1 - e];
+            const bool top = (e == 0);
+            const bool in_place = !top || x == y || xa == ya;
+            if (ps.single || (!ps.closed && in_place)) {
+                for (int k = ps.first + ps.count - 1; k >= ps.first; --k) {
+                    StageArgs a{};
+                    fill_common(a, shape, p, first_stage + k, alpha, m, activation);
+                    const bool from_y = top && k == ps.first + ps.count - 1;
+                    a.in0 = from_y ? y : x; a.in1 = from_y ? ya : xa; a.in_dtype = from_y ? in_dtype : out_dtype;
+                    a.out0 = x; a.out1 = xa; a.out_dtype = out_dtype;
+                    a.W = W + k * wstride;
+                    hipError_t err = launch_fast_forward(kInverse, a, shape->n_head, p.grid_fwd, s);
+                    if (err != hipSuccess) return (int)err;
+                }
+            } else {
+                FusedArgs a{};
+                a.in0 = top ? y : x; a.in1 = top ? ya : xa; a.in_dtype = top ? in_dtype : out_dtype;
+                a.out0 = x; a.out1 = xa; a.out_dtype = out_dtype;
+                a.W = W + ps.first * wstride;
+                fill_step_table(a.tab, shape->n_cache, alpha, m, activation);
+                hipError_t err = launch_fused(kInverse, a, shape, ps, s);
+                if (err != hipSuccess) return (int)err;
+            }
+        }
+        return NCN_OK;
+    }
+
     for (int k = n_stages - 1; k >= 0; --k) {
         StageArgs a{};
         fill_common(a, shape, p, first_stage + k, alpha, m, activation, grouping, k);
@@ -470,7 +508,7 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
                 a.W = W + ps.first * wstride;
                 a.dw_partials = partials;
                 fill_step_table(a.tab, shape->n_cache, alpha, m, activation);
-                err = launch_fused(true, a, shape, ps, s);
+                err = launch_fused(kBackward, a, shape, ps, s);
                 if (err != hipSuccess) return (int)err;
                 // a partial row holds the pass's stages side by side, as dW does: one reduction for all of them
                 // (rows * count <= kMaxGridX: the chunk sums take at most kMaxGridX / 32 + count rows of 2E)
@@ -601,7 +639,7 @@ int ncn_forward_radix(const void* x, const void* xa, int in_dtype, void* y, void
             a.aux0 = last ? y32 : nullptr; a.aux1 = last ? ya32 : nullptr;
             a.W = W + ps.first * wstride;
             fill_step_table(a.tab, shape->n_cache, alpha, m, activation);
-            err = launch_fused_radix(false, a, shape, ps, s);
+            err = launch_fused_radix(kForward, a, shape, ps, s);
         }
         if (err != hipSuccess) return (int)err;
     }
@@ -658,11 +696,51 @@ int ncn_backward_radix(const void* y, const void* ya, int y_dtype, const void* d
             a.W = W + ps.first * wstride;
             a.dw_partials = partials;
             fill_step_table(a.tab, shape->n_cache, alpha, m, activation);
-            err = launch_fused_radix(true, a, shape, ps, s);
+            err = launch_fused_radix(kBackward, a, shape, ps, s);
             if (err != hipSuccess) return (int)err;
             const int rows = radix_grid(shape, ps, true) / shape->n_head;
             err = launch_reduce_dw(partials, rows, (int64_t)ps.count * wstride, (int64_t)ps.count * wstride, level1,
                                    dW + ps.first * wstride, s);
+        }
+        if (err != hipSuccess) return (int)err;
+    }
+    return NCN_OK;
+}
+
+int ncn_inverse_radix(const void* y, const void* ya, int in_dtype, void* x, void* xa, int out_dtype, const float* W,
+                      const ncn_shape* shape, int first_level, int n_levels, float alpha, float m, int activation,
+                      void* stream) {
+    int rc = check_shape(shape, 0, n_levels, activation);
+    if (rc != NCN_OK) return rc;
+    rc = check_radix(shape, first_level, n_levels);
+    if (rc != NCN_OK) return rc;
+    if (!x || !xa || !y || !ya || !W) return NCN_ERR_NULL;
+    if (!known_dtype(in_dtype) || !known_dtype(out_dtype)) return NCN_ERR_DTYPE;
+    if (!aligned16(x) || !aligned16(xa) || !aligned16(y) || !aligned16(ya) || !aligned16(W)) return NCN_ERR_ALIGN;
+    const Plan p = make_plan(shape, activation);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int64_t wstride = 2 * shape->E;
+    const std::vector<RadixPass> passes = plan_radix(shape, first_level, n_levels, false);
+    for (size_t e = 0; e < passes.size(); ++e) {   // last pass first; every pass is closed: in place after the first
+        const RadixPass& ps = passes[passes.size() - 1 - e];
+        const bool top = (e == 0);
+        hipError_t err;
+        if (ps.single) {
+            StageArgs a{};
+            Grouping g{nullptr, nullptr, first_level + ps.first};
+            fill_common(a, shape, p, 0, alpha, m, activation, g, 0);
+            a.in0 = top ? y : x; a.in1 = top ? ya : xa; a.in_dtype = top ? in_dtype : out_dtype;
+            a.out0 = x; a.out1 = xa; a.out_dtype = out_dtype;
+            a.W = W + ps.first * wstride;
+            err = (p.path != 2) ? launch_generic(kInverse, a, shape->n_head, p.grid_fwd, s)
+                                : launch_fast_forward_indexed(kInverse, a, shape->n_head, p.grid_fwd, s);
+        } else {
+            FusedArgs a{};
+            a.in0 = top ? y : x; a.in1 = top ? ya : xa; a.in_dtype = top ? in_dtype : out_dtype;
+            a.out0 = x; a.out1 = xa; a.out_dtype = out_dtype;
+            a.W = W + ps.first * wstride;
+            fill_step_table(a.tab, shape->n_cache, alpha, m, activation);
+            err = launch_fused_radix(kInverse, a, shape, ps, s);
         }
         if (err != hipSuccess) return (int)err;
     }

@@ -137,7 +137,8 @@ std::vector<FusedPass> plan_fused(const ncn_shape* sh, int first, int count, boo
 }
 
 template <int NC, int EC>
-static hipError_t launch_fused_t(bool backward, const FusedArgs& a, int grid, size_t lds, hipStream_t s) {
+static hipError_t launch_fused_t(Pass pass, const FusedArgs& a, int grid, size_t lds, hipStream_t s) {
+    const bool backward = pass == kBackward;
     constexpr TileShape t = fast_tile(NC, EC);
     static_assert(t.r != 0, "multi-stage shapes must be one-stage shapes too");
     hipError_t err;
@@ -147,6 +148,12 @@ static hipError_t launch_fused_t(bool backward, const FusedArgs& a, int grid, si
         err = hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (err != hipSuccess) return err;
         hipLaunchKernelGGL(k, dim3(grid), dim3(64 * kFusedWavesBwd), lds, s, a);
+    } else if (pass == kInverse) {
+        auto k = tanh_only ? fused_forward_kernel<NC, EC, t.r, t.f, true, false, true>
+                           : fused_forward_kernel<NC, EC, t.r, t.f, false, false, true>;
+        err = hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (err != hipSuccess) return err;
+        hipLaunchKernelGGL(k, dim3(grid), dim3(64 * kFusedWavesFwd), lds, s, a);
     } else {
         auto k = tanh_only ? fused_forward_kernel<NC, EC, t.r, t.f, true> : fused_forward_kernel<NC, EC, t.r, t.f, false>;
         err = hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -169,7 +176,8 @@ int fused_grid(const ncn_shape* sh, const FusedPass& p, bool backward) {
     return (int)g;
 }
 
-hipError_t launch_fused(bool backward, FusedArgs& a, const ncn_shape* sh, const FusedPass& p, hipStream_t s) {
+hipError_t launch_fused(Pass pass, FusedArgs& a, const ncn_shape* sh, const FusedPass& p, hipStream_t s) {
+    const bool backward = pass == kBackward;
     const int nc = sh->n_cache, ec = (int)(sh->E / sh->n_head);
     a.N = sh->N;
     a.E = sh->E;
@@ -190,7 +198,7 @@ hipError_t launch_fused(bool backward, FusedArgs& a, const ncn_shape* sh, const 
     const int grid = fused_grid(sh, p, backward);
     const size_t lds = fused_lds_bytes(nc, ec, backward, p.window, p.count);
 #define NCN_CASE(NC, EC) \
-    if (nc == NC && ec == EC) return launch_fused_t<NC, EC>(backward, a, grid, lds, s);
+    if (nc == NC && ec == EC) return launch_fused_t<NC, EC>(pass, a, grid, lds, s);
     NCN_FOR_EACH_FUSED_CONFIG(NCN_CASE)
 #undef NCN_CASE
     return hipErrorInvalidConfiguration;

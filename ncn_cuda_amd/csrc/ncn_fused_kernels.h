@@ -245,7 +245,8 @@ __device__ __forceinline__ void fused_load_weights(const FusedArgs& A, int head,
 }
 
 // TANH_ONLY as in the one-stage kernels: the tanh build has no branch on the activation code.
-template <int NC, int EC, int R, int F, bool TANH_ONLY, bool RADIX = false>
+// INVERSE: the same kernel undoes the stages instead, last one first (in0, in1 = y, ya; out0, out1 = x, xa).
+template <int NC, int EC, int R, int F, bool TANH_ONLY, bool RADIX = false, bool INVERSE = false>
 __global__ void __launch_bounds__(64 * kFusedWavesFwd) fused_forward_kernel(const FusedArgs A) {
     constexpr int NW = kFusedWavesFwd;
     using T = Tile<NC, EC, R, F>;
@@ -280,7 +281,8 @@ __global__ void __launch_bounds__(64 * kFusedWavesFwd) fused_forward_kernel(cons
             fused_fetch_rows<K>(A.in0, A.in_dtype, off, rx);
             fused_fetch_rows<K>(A.in1, A.in_dtype, off, ra);
         }
-        for (int st = 0; st < A.n_stages; ++st) {
+        for (int sq = 0; sq < A.n_stages; ++sq) {
+            const int st = INVERSE ? A.n_stages - 1 - sq : sq;
             const uint32_t ss = A.sub_stride[st];
             const uint32_t ngroups = A.closed ? A.window : A.window - (NC - 1) * ss;
             float wi[F], wj[F];
@@ -297,7 +299,8 @@ __global__ void __launch_bounds__(64 * kFusedWavesFwd) fused_forward_kernel(cons
                     lds_load_frag<F>(xs + row[rr], x[rr]);
                     lds_load_frag<F>(as + row[rr], a[rr]);
                 }
-                forward_core<NC, EC, R, F, TANH_ONLY, false, true>(x, a, wi, wj, A.tab, st * NC, lane, slots);
+                if (INVERSE) inverse_core<NC, EC, R, F, TANH_ONLY, false, true>(x, a, wi, wj, A.tab, sq * NC, lane, slots);
+                else forward_core<NC, EC, R, F, TANH_ONLY, false, true>(x, a, wi, wj, A.tab, sq * NC, lane, slots);
                 if (valid) {
 #pragma unroll
                     for (int rr = 0; rr < R; ++rr) {
@@ -308,8 +311,9 @@ __global__ void __launch_bounds__(64 * kFusedWavesFwd) fused_forward_kernel(cons
             }
             __syncthreads();
         }
-        fused_store_rows_scaled<NC, EC, NW, RADIX>(A, it, xs, A.scale_dn, A.out0, A.out_dtype, A.aux0);
-        fused_store_rows_scaled<NC, EC, NW, RADIX>(A, it, as, A.scale_dn, A.out1, A.out_dtype, A.aux1);
+        const float back = INVERSE ? A.scale_up : A.scale_dn;   // out of the m-power-scaled form
+        fused_store_rows_scaled<NC, EC, NW, RADIX>(A, it, xs, back, A.out0, A.out_dtype, A.aux0);
+        fused_store_rows_scaled<NC, EC, NW, RADIX>(A, it, as, back, A.out1, A.out_dtype, A.aux1);
         __syncthreads();
     }
 }

@@ -34,7 +34,8 @@ size_t radix_lds_bytes(int nc, int ec, bool backward, uint32_t rows, int n_stage
 }
 
 template <int NC, int EC>
-hipError_t launch_t(bool backward, const FusedArgs& a, int grid, size_t lds, hipStream_t s) {
+hipError_t launch_t(Pass pass, const FusedArgs& a, int grid, size_t lds, hipStream_t s) {
+    const bool backward = pass == kBackward;
     constexpr TileShape t = fast_tile(NC, EC);
     static_assert(t.r != 0, "radix shapes must be one-stage shapes too");
     const bool tanh_only = a.tab.activation == NCN_ACT_TANH;
@@ -45,6 +46,12 @@ hipError_t launch_t(bool backward, const FusedArgs& a, int grid, size_t lds, hip
         err = hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (err != hipSuccess) return err;
         hipLaunchKernelGGL(k, dim3(grid), dim3(64 * kFusedWavesBwd), lds, s, a);
+    } else if (pass == kInverse) {
+        auto k = tanh_only ? fused_forward_kernel<NC, EC, t.r, t.f, true, true, true>
+                           : fused_forward_kernel<NC, EC, t.r, t.f, false, true, true>;
+        err = hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (err != hipSuccess) return err;
+        hipLaunchKernelGGL(k, dim3(grid), dim3(64 * kFusedWavesFwd), lds, s, a);
     } else {
         auto k = tanh_only ? fused_forward_kernel<NC, EC, t.r, t.f, true, true>
                            : fused_forward_kernel<NC, EC, t.r, t.f, false, true>;
@@ -114,7 +121,8 @@ int radix_grid(const ncn_shape* sh, const RadixPass& p, bool backward) {
     return (int)g;
 }
 
-hipError_t launch_fused_radix(bool backward, FusedArgs& a, const ncn_shape* sh, const RadixPass& p, hipStream_t s) {
+hipError_t launch_fused_radix(Pass pass, FusedArgs& a, const ncn_shape* sh, const RadixPass& p, hipStream_t s) {
+    const bool backward = pass == kBackward;
     const int nc = sh->n_cache, ec = (int)(sh->E / sh->n_head);
     a.N = sh->N;
     a.E = sh->E;
@@ -135,7 +143,7 @@ hipError_t launch_fused_radix(bool backward, FusedArgs& a, const ncn_shape* sh, 
     const int grid = radix_grid(sh, p, backward);
     const size_t lds = radix_lds_bytes(nc, ec, backward, p.rows, p.count);
 #define NCN_CASE(NC, EC) \
-    if (nc == NC && ec == EC) return launch_t<NC, EC>(backward, a, grid, lds, s);
+    if (nc == NC && ec == EC) return launch_t<NC, EC>(pass, a, grid, lds, s);
     NCN_FOR_EACH_RADIX_CONFIG(NCN_CASE)
 #undef NCN_CASE
     return hipErrorInvalidConfiguration;

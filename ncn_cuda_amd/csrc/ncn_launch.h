@@ -69,7 +69,7 @@ struct FusedPass {
 bool fused_supported(const ncn_shape* sh, int activation);
 std::vector<FusedPass> plan_fused(const ncn_shape* sh, int first, int count, bool backward);
 int fused_grid(const ncn_shape* sh, const FusedPass& p, bool backward);
-hipError_t launch_fused(bool backward, FusedArgs& a, const ncn_shape* sh, const FusedPass& p, hipStream_t s);
+hipError_t launch_fused(Pass pass, FusedArgs& a, const ncn_shape* sh, const FusedPass& p, hipStream_t s);
 
 
 // ---- multi-stage passes over radix-n levels, ncn_fused_radix.hip ---------------------------------------------
@@ -84,6 +84,6 @@ struct RadixPass {
 bool radix_fused_supported(const ncn_shape* sh);
 std::vector<RadixPass> plan_radix(const ncn_shape* sh, int first, int count, bool backward);
 int radix_grid(const ncn_shape* sh, const RadixPass& p, bool backward);
-hipError_t launch_fused_radix(bool backward, FusedArgs& a, const ncn_shape* sh, const RadixPass& p, hipStream_t s);
+hipError_t launch_fused_radix(Pass pass, FusedArgs& a, const ncn_shape* sh, const RadixPass& p, hipStream_t s);
 
 }  // namespace ncn

@@ -201,28 +201,20 @@ __device__ __forceinline__ void forward_steps(float (&x)[R][F], float (&a)[R][F]
 // STEP_MASK: a group with `live` < NC live rows only undoes its steps live-1 .. 0.  The skipped steps come first in
 // the loop, so the registers are first scaled as if they had been done (m^(NC-live)): every later step then
 // finds the scaling its table entry assumes, and the final factor is the same for all groups.
-template <int NC, int EC, int R, int F, bool TANH_ONLY, bool STEP_MASK = false>
-__device__ __forceinline__ void inverse_steps(float (&y)[R][F], float (&b)[R][F], const float (&wi)[F],
-                                              const float (&wj)[F], const StepTable& S, int lane, float4* slots,
-                                              int live = NC) {
+// inverse_core: the n_cache steps of one stage on registers that hold m^t0 x, m^t0 xa with t0 = step_base inversion
+// steps done before; leaves them scaled by t0 + n_cache steps (several stages in a row just keep counting).
+template <int NC, int EC, int R, int F, bool TANH_ONLY, bool STEP_MASK = false, bool ROWS = false>
+__device__ __forceinline__ void inverse_core(float (&y)[R][F], float (&b)[R][F], const float (&wi)[F],
+                                             const float (&wj)[F], const StepTable& S, int step_base, int lane,
+                                             float4* slots, int live = NC) {
     using T = Tile<NC, EC, R, F>;
     const float nom = S.m - 1.0f;
-    if (STEP_MASK && live != NC) {
-        const float sc = pow_steps(S.m, NC - live);
-#pragma unroll
-        for (int rr = 0; rr < R; ++rr)
-#pragma unroll
-            for (int f = 0; f < F; ++f) {
-                y[rr][f] *= sc;
-                b[rr][f] *= sc;
-            }
-    }
 #pragma unroll 1
     for (int jo = T::LR - 1; jo >= 0; --jo) {
 #pragma unroll
         for (int jr = R - 1; jr >= 0; --jr) {
             if (STEP_MASK && jo * R + jr >= live) continue;
-            const int ts = (T::LR - 1 - jo) * R + (R - 1 - jr);   // inversion steps done so far
+            const int ts = step_base + (T::LR - 1 - jo) * R + (R - 1 - jr);   // inversion steps done so far
             const float lam = S.step[ts].lam, kc2 = S.step[ts].kc2, kap = S.step[ts].kap;
 #pragma unroll
             for (int rr = 0; rr < R; ++rr)
@@ -233,7 +225,7 @@ __device__ __forceinline__ void inverse_steps(float (&y)[R][F], float (&b)[R][F]
             const float e = dot_frag<F>(xj, wj);
 #pragma unroll
             for (int rr = 0; rr < R; ++rr) {
-                const float s = lane_sum<1, T::LF>(dot_frag<F>(y[rr], wi) + e);
+                const float s = lane_sum<1, T::LF, ROWS>(dot_frag<F>(y[rr], wi) + e);
                 const float c = kc2 * s;
 #pragma unroll
                 for (int f = 0; f < F; ++f) {
@@ -245,6 +237,24 @@ __device__ __forceinline__ void inverse_steps(float (&y)[R][F], float (&b)[R][F]
             }
         }
     }
+}
+
+// one stage from true values to true values
+template <int NC, int EC, int R, int F, bool TANH_ONLY, bool STEP_MASK = false>
+__device__ __forceinline__ void inverse_steps(float (&y)[R][F], float (&b)[R][F], const float (&wi)[F],
+                                              const float (&wj)[F], const StepTable& S, int lane, float4* slots,
+                                              int live = NC) {
+    if (STEP_MASK && live != NC) {
+        const float sc = pow_steps(S.m, NC - live);
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr)
+#pragma unroll
+            for (int f = 0; f < F; ++f) {
+                y[rr][f] *= sc;
+                b[rr][f] *= sc;
+            }
+    }
+    inverse_core<NC, EC, R, F, TANH_ONLY, STEP_MASK>(y, b, wi, wj, S, 0, lane, slots, live);
     const float up = S.inv_m_pow_n;
 #pragma unroll
     for (int rr = 0; rr < R; ++rr)

@@ -291,6 +291,24 @@ def forward_radix(x, xa, W, alpha, activation, cache_dim, nhead, first_level, n_
     return y, ya
 
 
+def inverse_radix(y, ya, W, alpha, activation, cache_dim, nhead, first_level, n_levels, *, m=M_DEFAULT):
+    """x, xa (float32) with forward_radix(x, xa, ...) == (y, ya)."""
+    shape = validate(y, ya, W, cache_dim, nhead, activation, 0, n_levels, what="y")
+    dev = _require_gpu(y, ya, W)
+    y, ya, w = _prep(y.detach()), _prep(ya.detach()), _w32(W)
+    x = torch.empty(y.shape, dtype=torch.float32, device=dev)
+    xa = torch.empty(y.shape, dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.load().ncn_inverse_radix(_ptr(y), _ptr(ya), _DTYPES[y.dtype], _ptr(x), _ptr(xa), _lib.NCN_F32, _ptr(w),
+                                           ctypes.byref(shape), int(first_level), int(n_levels), float(alpha), float(m),
+                                           int(activation), _stream(dev))
+    if rc == -2:
+        raise ValueError(f"radix levels {first_level}..{first_level + n_levels - 1}: n_cache^(last level + 1) must "
+                         f"divide N = {y.shape[1]}")
+    _lib.check(rc, "ncn_inverse_radix")
+    return x, xa
+
+
 def backward_radix(y, ya, dy, dya, W, alpha, activation, cache_dim, nhead, first_level, n_levels, *, m=M_DEFAULT):
     """Reversible backward of forward_radix from its outputs.  Returns (x_rec, xa_rec, dx, dxa, dW[n_levels, 2E]), all
     float32."""

@@ -125,3 +125,34 @@ def test_multi_stage_other_activations(M, case, act):
     assert O.rel_err(dx, ref[2]) < tol and O.rel_err(dxa, ref[3]) < tol
     for l in range(L):
         assert O.rel_err(dW[l], ref[4][l]) < tol
+
+
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "b%d_N%d_E%d_C%d_n%d_s%d_L%d" % c)
+def test_multi_stage_inverse(M, case):
+    """ncn_inverse over a stage range (LDS passes where they can run without scratch) against one inverse call per
+    stage and against the inputs of the forward."""
+    batch, N, E, C, n, first, L = case
+    alpha = 0.9
+    x, xa, Ws, _, _ = O.make_inputs(batch, N, E, L, n, seed=19, xa_zero=False)
+    gx, gxa = x.cuda(), xa.cuda()
+    Wst = torch.stack(Ws).cuda()
+    y, ya = M.forward_stages(gx, gxa, Wst, alpha, 0, n, C, first, L)
+    xi, xai = M.inverse_stages(y, ya, Wst, alpha, 0, n, C, first, L)
+    tol = max(1e-5, 5e-7 * (1 / 0.9) ** (n * L))
+    assert O.rel_err(xi, x) < tol and O.rel_err(xai, xa) < tol
+    cy, cya = y, ya
+    for l in range(L - 1, -1, -1):
+        cy, cya = M.inverse_stages(cy, cya, Wst[l], alpha, 0, n, C, first + l, 1)
+    assert O.rel_err(xi, cy) < tol and O.rel_err(xai, cya) < tol
+    # in place (x, xa are y, ya): halo passes fall back to one launch per stage
+    py, pya = y.clone(), ya.clone()
+    from ncn_cuda_amd import _lib
+    import ctypes
+    shape = _lib.NcnShape(batch, N, E, C, n)
+    rc = _lib.load().ncn_inverse(ctypes.c_void_p(py.data_ptr()), ctypes.c_void_p(pya.data_ptr()), 0,
+                                 ctypes.c_void_p(py.data_ptr()), ctypes.c_void_p(pya.data_ptr()), 0,
+                                 ctypes.c_void_p(Wst.data_ptr()), ctypes.byref(shape), first, L, alpha, 0.9, 0,
+                                 ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert O.rel_err(py, xi) < tol and O.rel_err(pya, xai) < tol

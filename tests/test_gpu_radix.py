@@ -60,6 +60,8 @@ def test_radix_levels_vs_oracle_tables(M, case):
     for l in range(L):
         assert O.rel_err(dW[l], ref[4][l]) < tol, f"dW{l}"
     assert O.rel_err(xr, x) < tol and O.rel_err(xar, xa) < tol
+    ix, ixa = M.inverse_radix(y, ya, W, alpha, 0, n, C, first, L)
+    assert O.rel_err(ix, x) < tol and O.rel_err(ixa, xa) < tol
     # the table path of the library on the same levels (one launch per level): rounding-level agreement
     gt = torch.stack(tables).to(torch.int32).cuda()
     ty, tya = M.forward_stages(gx, gxa, W, alpha, 0, n, C, 0, L, group_index=gt)
