@@ -179,6 +179,36 @@ def main():
     copy_gbps = 5 * 2.0 * src.numel() * 4 / (c0.elapsed_time(c1) * 1e-3) / 1e9
     del src, dst
 
+    # the invertible-inverse pass over the whole stack (not part of the step; BASELINE's configuration 5 counts it):
+    # from the final outputs back to the inputs, segment by segment as the backward reverses them
+    inverse_ms = None
+    if args.grouping in ("closed", "radix"):
+        fy, fya = gx, gxa          # float32 outputs of the stack (the step above may have stored bf16)
+        for a, cnt in segs:
+            if args.grouping == "radix":
+                fy, fya = M.forward_radix(fy, fya, Wst[a:a + cnt], alpha, 0, n, C, a, cnt)
+            else:
+                fy, fya = M.forward_stages(fy, fya, Wst[a:a + cnt], alpha, 0, n, C, a, cnt, out_dtype=torch.float32)
+
+        def inverse_all():
+            cy, cya = fy, fya
+            for a, cnt in reversed(segs):
+                if args.grouping == "radix":
+                    cy, cya = M.inverse_radix(cy, cya, Wst[a:a + cnt], alpha, 0, n, C, a, cnt)
+                else:
+                    cy, cya = M.inverse_stages(cy, cya, Wst[a:a + cnt], alpha, 0, n, C, a, cnt)
+            return cy, cya
+
+        inverse_all()
+        i0, i1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        i0.record()
+        for _ in range(5):
+            rx, rxa = inverse_all()
+        i1.record()
+        torch.cuda.synchronize()
+        inverse_ms = i0.elapsed_time(i1) / 5
+        recon_err = ((rx - gx.float()).abs().max() / gx.float().abs().max()).item()
+
     # dominant kernel: backward stage launch (its event bracket also holds the microsecond-scale dW reduce)
     # (with multi-stage segments the bracket holds a whole segment: per-stage figures are the segment's / its stages)
     bwd_ms = sum(e0.elapsed_time(e1) for e0, e1, _ in events) / sum(cnt for _, _, cnt in events)
@@ -218,6 +248,8 @@ def main():
                   "fp32_flops_per_step": flops_step,
                   "achieved_TFLOPs": flops_step / (ms_per_step * 1e-3) / 1e12,
                   "frac_of_fp32_vector_peak": flops_step / (ms_per_step * 1e-3) / 1e12 / VALU_PEAK_TFLOPS,
+                  "inverse_ms_per_stack": inverse_ms,
+                  "inverse_reconstruction_rel_err": recon_err if inverse_ms is not None else None,
                   "note": "the step is bound by float32 VALU + exp2/rcp issue, not by HBM or MFMA: "
                           "each element takes n_cache sequential tanh steps per stage"},
     }
