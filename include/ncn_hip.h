@@ -23,7 +23,9 @@
  * slice of both halves (torch_ref/ncn_pytorch.py:60-61).
  *
  * All pointers are device pointers, 16-byte aligned.  Calls are re-entrant; two calls that write the
- * same buffers must be ordered by the caller (same stream, or events).
+ * same buffers must be ordered by the caller (same stream, or events).  Kernels are launched on `stream`
+ * (NULL: the default stream) of the device that is current when the call is made: make the device that
+ * owns the buffers and the stream current first (hipSetDevice).
  */
 #ifndef NCN_HIP_H
 #define NCN_HIP_H

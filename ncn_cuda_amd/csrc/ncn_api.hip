@@ -220,7 +220,7 @@ size_t temp_bytes(const ncn_shape* sh, bool backward) {
 
 extern "C" {
 
-const char* ncn_version(void) { return "0.3"; }
+const char* ncn_version(void) { return "0.4"; }
 
 int ncn_plan_passes(const ncn_shape* shape, int first_stage, int n_stages, int activation, int backward, int32_t* out,
                     int max_passes) {
