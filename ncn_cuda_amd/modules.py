@@ -163,6 +163,14 @@ def fused_ncn_cuda_v2(
     return yi, ya
 
 
+def _check_grouping(grouping):
+    """"stride": the stage permutation of torch_ref (the reference's only layout on this surface); "radix": module l is
+    level l of the radix-n digit grouping of ncn_triton/group_tensors.py (keyword only, not in the reference)."""
+    if grouping not in ("stride", "radix"):
+        raise ValueError(f"grouping must be 'stride' or 'radix', got {grouping!r}")
+    return grouping
+
+
 class NCNModuleCuda(nn.Module):
     def __init__(self, alpha, activation, n_cache, n_head, module_nr, embed_dim):
         super().__init__()
@@ -189,7 +197,7 @@ class NCNNetCuda(nn.Module):
     """Same constructor as the reference.  `fuse_stages=True` (keyword only, not in the reference) runs the stack as
     one NCNNetFunction node instead of one node per module; parameters and state_dict are the same either way."""
 
-    def __init__(self, alpha, activation, n_cache, n_head, num_modules, embed_dim, *, fuse_stages=False,
+    def __init__(self, alpha, activation, n_cache, n_head, num_modules, embed_dim, *, grouping="stride", fuse_stages=False,
                  save_every=None):
         super().__init__()
         self.num_modules = num_modules
@@ -199,11 +207,15 @@ class NCNNetCuda(nn.Module):
         self.n_head = n_head
         self.fuse_stages = fuse_stages
         self.save_every = save_every
+        self.grouping = _check_grouping(grouping)
         self.ncn_modules = nn.ModuleList(
             [NCNModuleCuda(alpha, self.activation_nr, n_cache, n_head, module_nr, embed_dim)
              for module_nr in range(num_modules)])
 
     def forward(self, x, xa):
+        if self.grouping == "radix":
+            return fused_ncn_radix_net(x, xa, [m.weight for m in self.ncn_modules], self.alpha, self.activation_nr,
+                                       self.n_cache, self.n_head, 0, self.save_every)
         if self.fuse_stages:
             return fused_ncn_net(x, xa, [m.weight for m in self.ncn_modules], self.alpha, self.activation_nr,
                                  self.n_cache, self.n_head, 0, self.save_every)
@@ -213,7 +225,8 @@ class NCNNetCuda(nn.Module):
 
 
 class NCNNetTestCuda(nn.Module):
-    def __init__(self, alpha, activation, n_cache, n_head, num_modules, weights, *, fuse_stages=False, save_every=None):
+    def __init__(self, alpha, activation, n_cache, n_head, num_modules, weights, *, grouping="stride", fuse_stages=False,
+                 save_every=None):
         super().__init__()
         self.num_modules = num_modules
         self.alpha = alpha
@@ -223,8 +236,12 @@ class NCNNetTestCuda(nn.Module):
         self.weights = weights
         self.fuse_stages = fuse_stages
         self.save_every = save_every
+        self.grouping = _check_grouping(grouping)
 
     def forward(self, x, xa):
+        if self.grouping == "radix":
+            return fused_ncn_radix_net(x, xa, list(self.weights[:self.num_modules]), self.alpha, self.activation_nr,
+                                       self.n_cache, self.n_head, 0, self.save_every)
         if self.fuse_stages:
             return fused_ncn_net(x, xa, list(self.weights[:self.num_modules]), self.alpha, self.activation_nr,
                                  self.n_cache, self.n_head, 0, self.save_every)

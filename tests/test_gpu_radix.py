@@ -115,3 +115,24 @@ def test_radix_net_autograd_node(M):
     assert O.rel_err(gx.grad, ref[2]) < tol and O.rel_err(gxa.grad, ref[3]) < tol
     for l in range(L):
         assert gw[l].grad.shape == gw[l].shape and O.rel_err(gw[l].grad, ref[4][l]) < tol
+
+
+def test_net_modules_with_radix_grouping(M):
+    import ncn_cuda_amd as pkg
+    batch, N, E, C, n, L = 2, 256, 64, 2, 2, 8
+    x, xa, Ws, dy, dya = O.make_inputs(batch, N, E, L, n, seed=44, xa_zero=False)
+    tables = [O.radix_group_table(N, n, l) for l in range(L)]
+    d = torch.float64
+    ref = O.net_autograd_indexed(x.to(d), xa.to(d), [w.to(d) for w in Ws], dy.to(d), dya.to(d), 0.9, n, C, tables)
+    gw = [w.cuda().requires_grad_() for w in Ws]
+    net = pkg.NCNNetTestCuda(0.9, "tanh", n, C, L, gw, grouping="radix")
+    gx, gxa = x.cuda().requires_grad_(), xa.cuda().requires_grad_()
+    yi, ya = net(gx, gxa)
+    torch.autograd.backward([yi, ya], [dy.cuda(), dya.cuda()])
+    assert O.rel_err(yi, ref[0]) < 1e-5 and O.rel_err(gx.grad, ref[2]) < 3e-5 and O.rel_err(gw[3].grad, ref[4][3]) < 3e-5
+    mod = pkg.NCNNetCuda(0.9, "tanh", n, C, L, E, grouping="radix").cuda()
+    assert sorted(mod.state_dict()) == [f"ncn_modules.{l}.weight" for l in range(L)]
+    y2, _ = mod(x.cuda(), xa.cuda())
+    assert y2.shape == x.shape and torch.isfinite(y2).all()
+    with pytest.raises(ValueError):
+        pkg.NCNNetCuda(0.9, "tanh", n, C, L, E, grouping="butterfly")
