@@ -210,9 +210,10 @@ def main():
         recon_err = ((rx - gx.float()).abs().max() / gx.float().abs().max()).item()
 
     # dominant kernel: backward stage launch (its event bracket also holds the microsecond-scale dW reduce)
-    # (with multi-stage segments the bracket holds a whole segment: per-stage figures are the segment's / its stages)
-    bwd_ms = sum(e0.elapsed_time(e1) for e0, e1, _ in events) / sum(cnt for _, _, cnt in events)
-    bytes_bwd_launch = 6.0 * P * sbytes            # read y, ya, dy, dya; write dx, dxa (per stage)
+    # (with multi-stage segments the bracket holds one backward call over a whole segment, and the algorithmic bytes
+    # are those of one call: its inputs and outputs once, however many stages it runs)
+    bwd_ms = sum(e0.elapsed_time(e1) for e0, e1, _ in events) / len(events)
+    bytes_bwd_launch = 6.0 * P * (sbytes if save_every == 1 else 4)   # read y, ya, dy, dya; write dx, dxa
     achieved = bytes_bwd_launch / (bwd_ms * 1e-3) / 1e9
     elem_steps_stage = float(P) * n
     flops_step = (FLOPS_FWD_PER_ELEM_STEP + FLOPS_BWD_PER_ELEM_STEP) * elem_steps_stage * L
@@ -237,7 +238,7 @@ def main():
                      "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_BWD_TRAFFIC_BYTES.get(args.config) if args.grouping == "closed" else None,
                      "kernel": (f"stage_backward_kernel<{n},{E // C}>" + (" (indexed build)" if tables else "")
                                 if save_every == 1 else
-                                f"backward of {save_every}-stage segments (multi-stage passes), per stage"),
+                                f"backward call over a segment of up to {save_every} stages (multi-stage passes)"),
                      "avg_launch_ms": bwd_ms,
                      "attainable_copy_GBps": copy_gbps, "frac_of_attainable_copy": achieved / copy_gbps,
                      "algorithmic_bytes_per_launch": bytes_bwd_launch},
