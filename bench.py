@@ -212,7 +212,11 @@ def main():
     # dominant kernel: backward stage launch (its event bracket also holds the microsecond-scale dW reduce)
     # (with multi-stage segments the bracket holds one backward call over a whole segment, and the algorithmic bytes
     # are those of one call: its inputs and outputs once, however many stages it runs)
-    bwd_ms = sum(e0.elapsed_time(e1) for e0, e1, _ in events) / len(events)
+    # (n_cache >= 8 never uses multi-stage passes: a call over a segment is one launch per stage, so the figures
+    # stay per stage launch there)
+    lds_passes = save_every > 1 and n in (2, 4)
+    bracket_ms = sum(e0.elapsed_time(e1) for e0, e1, _ in events)
+    bwd_ms = bracket_ms / len(events) if lds_passes else bracket_ms / sum(cnt for _, _, cnt in events)
     bytes_bwd_launch = 6.0 * P * (sbytes if save_every == 1 else 4)   # read y, ya, dy, dya; write dx, dxa
     achieved = bytes_bwd_launch / (bwd_ms * 1e-3) / 1e9
     elem_steps_stage = float(P) * n
@@ -237,7 +241,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_BWD_TRAFFIC_BYTES.get(args.config) if args.grouping == "closed" else None,
                      "kernel": (f"stage_backward_kernel<{n},{E // C}>" + (" (indexed build)" if tables else "")
-                                if save_every == 1 else
+                                if not lds_passes else
                                 f"backward call over a segment of up to {save_every} stages (multi-stage passes)"),
                      "avg_launch_ms": bwd_ms,
                      "attainable_copy_GBps": copy_gbps, "frac_of_attainable_copy": achieved / copy_gbps,
