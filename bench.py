@@ -38,8 +38,9 @@ VALU_PEAK_TFLOPS = 157.3   # MI355X FP32 vector peak (packed); 78.6 without pack
 # rcp = 1 each), without the per-row and per-lane bookkeeping: forward 1 FMA (dot) + 2 (z) + 1 (t+1) + 2 FMA (xa)
 # + 2 (x) + exp2 + rcp = 13; backward 11 FMA + 4 mul/add + exp2 + rcp = 28.
 # HBM bytes of one backward-stage launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (calibrated on a
-# 1 GiB copy; see profiles/stage_kernels_cfg3.md).  Only the headline workload has been measured.
-MEASURED_BWD_TRAFFIC_BYTES = {"cfg3": 1.1128e9}
+# 1 GiB copy; see profiles/stage_kernels_cfg3.md); for cfg4 the three passes of one backward call over the 13 stages
+# (profiles/fused_kernels_cfg4.md: 7.19 GB read + 6.46 GB written).
+MEASURED_BWD_TRAFFIC_BYTES = {"cfg3": 1.1128e9, "cfg4": 13.65e9}
 FLOPS_FWD_PER_ELEM_STEP = 13.0
 FLOPS_BWD_PER_ELEM_STEP = 28.0
 
