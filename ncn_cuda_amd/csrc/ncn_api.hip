@@ -43,9 +43,12 @@ int check_shape(const ncn_shape* sh, int first_stage, int n_stages, int activati
 // 2^(stage-1) mod groups without overflow (torch_ref/ncn_pytorch.py:38 uses Python big integers)
 uint32_t stage_stride(int stage, uint32_t groups) {
     if (stage == 0) return 0;
-    uint64_t s = 1 % groups;
-    for (int k = 1; k < stage; ++k) s = (s * 2) % groups;
-    return (uint32_t)s;
+    uint64_t r = 1 % groups, b = 2 % groups;
+    for (uint32_t e = (uint32_t)stage - 1; e; e >>= 1) {   // square and multiply: any stage number costs 31 rounds
+        if (e & 1) r = r * b % groups;
+        b = b * b % groups;
+    }
+    return (uint32_t)r;
 }
 
 struct Plan {
@@ -249,7 +252,7 @@ const char* ncn_error_string(int code) {
         case NCN_ERR_ACTIVATION: return "unknown activation code (0 tanh, 1 relu, 2 sigmoid, 3 leaky relu, -1 linear)";
         case NCN_ERR_WORKSPACE: return "workspace is NULL or smaller than ncn_workspace_bytes()";
         case NCN_ERR_UNSUPPORTED: return "unsupported shape: n_cache must be <= 64 and the head width <= 64 (128 for power-of-two n_cache <= 16)";
-        case NCN_ERR_ALIGN: return "a pointer is not 16-byte aligned";
+        case NCN_ERR_ALIGN: return "a pointer is not 16-byte aligned (4-byte for group_index and ctx_len)";
         case NCN_ERR_ALIAS: return "n_stages > 1 needs float32 x_rec, xa_rec, dx, dxa to carry the state";
         default: break;
     }

@@ -218,3 +218,18 @@ def test_in_place_forward_and_inverse(M):
     bx, bxa = gx.clone(), gxa.clone()
     M.forward_stages(bx, bxa, gW, 0.9, 0, n, C, 2, 1, out=(bx, bxa))
     assert torch.equal(bx, y) and torch.equal(bxa, ya)
+
+
+@pytest.mark.parametrize("stage", [33, 70, 1000003])
+def test_high_stage_numbers(M, stage):
+    """The stride is 2^(stage-1) mod groups (torch_ref/ncn_pytorch.py:38, Python integers): stage numbers whose
+    power of two overflows 32 and 64 bits, on a group count that is not a power of two."""
+    batch, N, E, C, n = 2, 48, 32, 2, 4          # 12 groups
+    x, xa, Ws, dyi, dya = O.make_inputs(batch, N, E, 1, n, seed=5, xa_zero=False)
+    assert O.stage_stride(N, n, stage) == pow(2, stage - 1, N // n) != 0
+    ref_y, ref_ya = O.stage_forward(x, xa, Ws[0], 0.9, n, C, stage)
+    gx, gxa, gw = _dev(x, xa, Ws[0])
+    y, ya = M.forward(gx, gxa, gw, 0.9, 0, n, C, stage)
+    assert O.rel_err(y, ref_y) < TOL_F32 and O.rel_err(ya, ref_ya) < TOL_F32
+    rx, rxa = M.inverse(y, ya, gw, 0.9, 0, n, C, stage)
+    assert O.rel_err(rx, x) < TOL_F32 and O.rel_err(rxa, xa) < TOL_F32
