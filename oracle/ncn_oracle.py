@@ -20,14 +20,19 @@ Pinning (see tests/test_oracle_*.py): every function is checked against the comm
 vectors that tests/golden/make_golden.py wrote from the reference's own CPU code, the closed-form
 backward additionally against autograd through stage_forward in float64, the inverse against
 forward round trips, the index map against the bijection/hand values.  No function here is
-"parity unpinned" for activation == tanh.  The relu / sigmoid / linear activations exist only in the
-reference's CUDA kernels (ncn_fwd_cuda_kernel.cu:86-95) and leaky relu only in its Triton kernels
-(ncn_triton/ncn_triton.py:22-28), none of which can be built or run here; for them the oracle is
-pinned only by autograd-vs-closed-form and special cases: parity unpinned.  The same holds for
-stage_forward_indexed with context lengths (the reference's only statement of it is a Triton kernel
-that cannot run here and that leaves rows past the length undefined): it is pinned by reduction to the
-pinned stage_forward (full lengths, stride table) and by literal loops on the cut group, but its
-pass-through of dead rows is this build's choice: parity unpinned.
+"parity unpinned" for activation == tanh.
+The leaky-relu and linear activations (forward and closed-form backward), grouping by a table, the
+radix tables and context lengths are pinned by tests/golden/triton_*.npz, which
+tests/golden/make_golden_triton.py wrote by running the reference's Triton kernels
+(ncn_triton/ncn_triton.py, ncn_triton_old.py) under Triton's CPU interpreter: whole groups below a
+length forward and backward, the group a length cuts forward only (the reference's backward of a cut
+group reads rows that alias position 0, an artefact).
+Still parity unpinned:
+  * the relu and sigmoid activations: they exist only in the reference's CUDA kernels
+    (ncn_fwd_cuda_kernel.cu:86-95), which cannot be built here; pinned by autograd-vs-closed-form and
+    special cases only;
+  * the backward of a cut group, and what happens to rows past a length: the reference leaves those rows
+    unwritten; stage_forward_indexed passes them through, which is this build's choice.
 """
 import math
 

@@ -29,6 +29,12 @@ def load_golden(name):
     return out
 
 
+def load_npz(name):
+    """A committed fixture as a dict of numpy arrays, untouched (for fixtures with their own layout)."""
+    with np.load(os.path.join(GOLDEN_DIR, name + ".npz"), allow_pickle=False) as z:
+        return {k: z[k] for k in z.files}
+
+
 GOLDEN_CASES = ["cfg1_n2_L8", "small_n4_L3", "bench_like_n8_L5", "odd_n3_L3"]
 
 
