@@ -86,6 +86,23 @@ def activations(T):
     return blob
 
 
+def headline_tile(T):
+    """The headline shape's tile (groups of 16 rows, 4 heads of 32 features, tanh, 3 stages) on a short sequence:
+    torch_ref's fixtures stop at groups of 8."""
+    batch, N, E, C, n, L = 1, 64, 128, 4, 16, 3
+    gen = torch.Generator().manual_seed(16)
+    x, xa = _draw(gen, batch, N, E), _draw(gen, batch, N, E)
+    Ws = [_draw(gen, 2 * E, scale=0.25) for _ in range(L)]
+    dyi, dya = _draw(gen, batch, N, E), _draw(gen, batch, N, E)
+    out = _run(lambda a, b, ws: T.NCNNetTestTriton(ALPHA, "tanh", n, C, L, ws)(a, b), x, xa, Ws, dyi, dya)
+    blob = {"meta": np.array([batch, N, E, C, n, L], dtype=np.int64), "alpha": np.array(ALPHA),
+            "x": x.numpy(), "xa": xa.numpy(), "dyi": dyi.numpy(), "dya": dya.numpy()}
+    for l, w in enumerate(Ws):
+        blob[f"W{l}"] = w.numpy()
+    blob.update(out)
+    return blob
+
+
 def radix_table(G, N, n, level):
     """Positions in (group, slot) order from the reference's digit split (group_tensors.py:8-18)."""
     strides = [n ** k for k in range(16)]
@@ -169,7 +186,8 @@ def main():
     from ncn_triton import ncn_triton_old as TO
     np.savez_compressed(os.path.join(HERE, "triton_activations.npz"), **activations(T))
     np.savez_compressed(os.path.join(HERE, "triton_tables_lengths.npz"), **tables_and_lengths(TO, G))
-    print("wrote triton_activations.npz, triton_tables_lengths.npz")
+    np.savez_compressed(os.path.join(HERE, "triton_headline_tile.npz"), **headline_tile(T))
+    print("wrote triton_activations.npz, triton_tables_lengths.npz, triton_headline_tile.npz")
 
 
 if __name__ == "__main__":

@@ -90,3 +90,21 @@ def test_cut_group_forward_live_rows(surfaces, k):
                                        "tanh", C, n, 0)
     assert O.rel_err(yi.cpu()[check], torch.from_numpy(g[tag + "yi"])[check]) < TOL
     assert O.rel_err(ya.cpu()[check], torch.from_numpy(g[tag + "ya"])[check]) < TOL
+
+
+@pytest.mark.parametrize("storage", ["f32", "bf16"])
+def test_headline_tile_stack(surfaces, storage):
+    """The tile of the headline shape (groups of 16 rows, heads of 32 features, 3 stages) against the reference's
+    Triton stack class; bfloat16 storage with float32 arithmetic at 2e-2."""
+    T, _ = surfaces
+    g = load_npz("triton_headline_tile")
+    batch, N, E, C, n, L = (int(v) for v in g["meta"])
+    dt, tol = (torch.float32, TOL) if storage == "f32" else (torch.bfloat16, 2e-2)
+    Ws = [_g(g[f"W{l}"]).to(dt).requires_grad_() for l in range(L)]
+    x, xa = _g(g["x"]).to(dt).requires_grad_(), _g(g["xa"]).to(dt).requires_grad_()
+    yi, ya = T.NCNNetTestTriton(float(g["alpha"]), "tanh", n, C, L, Ws)(x, xa)
+    torch.autograd.backward([yi, ya], [_g(g["dyi"]).to(dt), _g(g["dya"]).to(dt)])
+    for got, key in ((yi, "yi"), (ya, "ya"), (x.grad, "dx"), (xa.grad, "dxa")):
+        assert O.rel_err(got.detach().float().cpu(), torch.from_numpy(g[key])) < tol, key
+    for l in range(L):
+        assert O.rel_err(Ws[l].grad.float().cpu(), torch.from_numpy(g[f"dW{l}"])) < tol, l

@@ -112,3 +112,18 @@ def test_cut_group_forward_live_rows(k):
     cut_rows[:, 0] = False
     m = cut_rows[:, :, None].expand(batch, N, E)
     assert O.rel_err(yi_full[m], _t(g[tag + "yi"])[m]) > 1e-3
+
+
+def test_headline_tile_stack():
+    """Groups of 16 rows, 4 heads of 32 features, 3 stages, tanh: the reference's Triton stack class."""
+    g = load_npz("triton_headline_tile")
+    batch, N, E, C, n, L = (int(v) for v in g["meta"])
+    assert (n, E // C) == (16, 32)
+    d = torch.float64
+    Ws = [_t(g[f"W{l}"]).to(d) for l in range(L)]
+    yi, ya, dx, dxa, dWs = O.net_autograd(_t(g["x"]).to(d), _t(g["xa"]).to(d), Ws, _t(g["dyi"]).to(d),
+                                          _t(g["dya"]).to(d), float(g["alpha"]), n, C)
+    for got, key in ((yi, "yi"), (ya, "ya"), (dx, "dx"), (dxa, "dxa")):
+        assert O.rel_err(got, _t(g[key])) < TOL, key
+    for l in range(L):
+        assert O.rel_err(dWs[l], _t(g[f"dW{l}"])) < TOL, l
