@@ -219,6 +219,57 @@ size_t temp_bytes(const ncn_shape* sh, bool backward) {
     return align256((size_t)sh->batch * sh->N * sh->E * sizeof(float)) * (backward ? 4 : 2);
 }
 
+// The backward launches of one call write their dW partial rows side by side into the partial buffer and are summed
+// together: two reduction launches per call instead of two per launch, as long as the buffer (kMaxGridX rows of 2E)
+// and the job (kReduceMaxSegments launches, kReduceMaxStages stages) hold them.
+class DwReducer {
+  public:
+    DwReducer(float* partials, float* level1, int64_t two_e, hipStream_t s)
+        : partials_(partials), level1_(level1), two_e_(two_e), stream_(s) { job_.n = 0; }
+    // Where a launch of `rows` partial rows of `stages` stages each may write; earlier launches are summed first
+    // if it would not fit behind them.
+    hipError_t reserve(int rows, int stages, float** region) {
+        hipError_t err = hipSuccess;
+        if (job_.n == kReduceMaxSegments || stages_ + stages > kReduceMaxStages ||
+            used_rows_ + (int64_t)rows * stages > kMaxGridX)
+            err = flush();
+        *region = partials_ + used_rows_ * two_e_;
+        return err;
+    }
+    // The launch that got `region` from reserve() has been enqueued: its column sums go to dW_out[stages * 2E].
+    void add(const float* region, int rows, int stages, float* dW_out) {
+        ReduceSegment& g = job_.seg[job_.n];
+        g.in = region;
+        g.out = dW_out;
+        g.cols = stages * two_e_;
+        g.rows = rows;
+        g.chunk0 = chunks_;
+        g.level1_offset = level1_floats_;
+        const int chunks = (rows + kReduceRowsPerBlock - 1) / kReduceRowsPerBlock;
+        chunks_ += chunks;
+        level1_floats_ += (int64_t)chunks * g.cols;
+        used_rows_ += (int64_t)rows * stages;
+        stages_ += stages;
+        ++job_.n;
+    }
+    hipError_t flush() {
+        const hipError_t err = launch_reduce_job(job_, level1_, stream_);
+        job_.n = 0;
+        used_rows_ = level1_floats_ = 0;
+        stages_ = chunks_ = 0;
+        return err;
+    }
+
+  private:
+    float* partials_;
+    float* level1_;
+    int64_t two_e_;
+    hipStream_t stream_;
+    ReduceJob job_;
+    int64_t used_rows_ = 0, level1_floats_ = 0;
+    int stages_ = 0, chunks_ = 0;
+};
+
 }  // namespace
 
 extern "C" {
@@ -481,6 +532,7 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
                        reinterpret_cast<float*>(tb + 2 * one), reinterpret_cast<float*>(tb + 3 * one)};
         const void* cy = y; const void* cya = ya; int cy_dtype = y_dtype;
         const void* cg = dy; const void* cga = dya; int cg_dtype = dy_dtype;
+        DwReducer reducer(partials, level1, wstride, s);
         for (size_t e = 0; e < np; ++e) {
             const FusedPass& ps = passes[np - 1 - e];
             const bool to_out = ((np - 1 - e) % 2) == 0;
@@ -489,7 +541,11 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
             void* ddx = to_out ? dx : static_cast<void*>(t[2]);
             void* ddxa = to_out ? dxa : static_cast<void*>(t[3]);
             const int d_dtype = to_out ? dx_dtype : NCN_F32;
-            hipError_t err;
+            // a partial row of a multi-stage pass holds its stages side by side, as dW does
+            const int rows = ps.single ? p.partial_rows : fused_grid(shape, ps, true) / shape->n_head;
+            float* region;
+            hipError_t err = reducer.reserve(rows, ps.count, &region);
+            if (err != hipSuccess) return (int)err;
             if (ps.single) {
                 StageArgs a{};
                 fill_common(a, shape, p, first_stage + ps.first, alpha, m, activation);
@@ -498,10 +554,8 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
                 a.out0 = ddx; a.out1 = ddxa; a.out_dtype = d_dtype;
                 a.aux0 = dxr; a.aux1 = dxar;
                 a.W = W + ps.first * wstride;
-                a.dw_partials = partials;
+                a.dw_partials = region;
                 err = launch_fast_backward(a, shape->n_head, p.grid_x, s);
-                if (err != hipSuccess) return (int)err;
-                err = launch_reduce_dw(partials, p.partial_rows, wstride, wstride, level1, dW + ps.first * wstride, s);
             } else {
                 FusedArgs a{};
                 a.in0 = cy; a.in1 = cya; a.in_dtype = cy_dtype;
@@ -509,24 +563,23 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
                 a.out0 = ddx; a.out1 = ddxa; a.out_dtype = d_dtype;
                 a.aux0 = dxr; a.aux1 = dxar;
                 a.W = W + ps.first * wstride;
-                a.dw_partials = partials;
+                a.dw_partials = region;
                 fill_step_table(a.tab, shape->n_cache, alpha, m, activation);
                 err = launch_fused(kBackward, a, shape, ps, s);
-                if (err != hipSuccess) return (int)err;
-                // a partial row holds the pass's stages side by side, as dW does: one reduction for all of them
-                // (rows * count <= kMaxGridX: the chunk sums take at most kMaxGridX / 32 + count rows of 2E)
-                const int rows = fused_grid(shape, ps, true) / shape->n_head;
-                err = launch_reduce_dw(partials, rows, (int64_t)ps.count * wstride, (int64_t)ps.count * wstride, level1,
-                                       dW + ps.first * wstride, s);
             }
             if (err != hipSuccess) return (int)err;
+            reducer.add(region, rows, ps.count, dW + ps.first * wstride);
             cy = dxr; cya = dxar; cy_dtype = NCN_F32;
             cg = ddx; cga = ddxa; cg_dtype = d_dtype;
         }
-        return NCN_OK;
+        return (int)reducer.flush();
     }
 
+    DwReducer reducer(partials, level1, wstride, s);
     for (int k = n_stages - 1; k >= 0; --k) {
+        float* region;
+        hipError_t err = reducer.reserve(p.partial_rows + extra_rows, 1, &region);
+        if (err != hipSuccess) return (int)err;
         StageArgs a{};
         fill_common(a, shape, p, first_stage + k, alpha, m, activation, grouping, k);
         const bool top = (k == n_stages - 1);
@@ -542,16 +595,15 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
         a.aux0 = x_rec;
         a.aux1 = xa_rec;
         a.W = W + (int64_t)k * 2 * shape->E;
-        a.dw_partials = partials;
-        hipError_t err = (p.path != 2)      ? launch_generic(kBackward, a, shape->n_head, p.grid_x, s)
-                         : grouping.plain() ? launch_fast_backward(a, shape->n_head, p.grid_x, s)
-                                            : launch_fast_backward_indexed(a, shape->n_head, p.grid_x, s);
+        a.dw_partials = region;
+        err = (p.path != 2)      ? launch_generic(kBackward, a, shape->n_head, p.grid_x, s)
+              : grouping.plain() ? launch_fast_backward(a, shape->n_head, p.grid_x, s)
+                                 : launch_fast_backward_indexed(a, shape->n_head, p.grid_x, s);
         if (err == hipSuccess && grouping.ctx_len) err = launch_ragged_rest(kBackward, a, shape, p.path, p.partial_rows, s);
         if (err != hipSuccess) return (int)err;
-        err = launch_reduce_dw(partials, p.partial_rows + extra_rows, wstride, wstride, level1, dW + k * wstride, s);
-        if (err != hipSuccess) return (int)err;
+        reducer.add(region, p.partial_rows + extra_rows, 1, dW + k * wstride);
     }
-    return NCN_OK;
+    return (int)reducer.flush();
 }
 
 int ncn_forward(const void* x, const void* xa, int in_dtype, void* y, void* ya, int out_dtype, float* y32, float* ya32,
@@ -672,10 +724,14 @@ int ncn_backward_radix(const void* y, const void* ya, int y_dtype, const void* d
     const int64_t wstride = 2 * shape->E;
     const std::vector<RadixPass> passes = plan_radix(shape, first_level, n_levels, true);
     // last pass first; the first one to run reads y, ya, dy, dya, the others run in place on x_rec, xa_rec, dx, dxa
+    DwReducer reducer(partials, level1, wstride, s);
     for (size_t e = 0; e < passes.size(); ++e) {
         const RadixPass& ps = passes[passes.size() - 1 - e];
         const bool top = (e == 0);
-        hipError_t err;
+        const int rows = ps.single ? p.partial_rows : radix_grid(shape, ps, true) / shape->n_head;
+        float* region;
+        hipError_t err = reducer.reserve(rows, ps.count, &region);
+        if (err != hipSuccess) return (int)err;
         if (ps.single) {
             StageArgs a{};
             Grouping g{nullptr, nullptr, first_level + ps.first};
@@ -685,11 +741,9 @@ int ncn_backward_radix(const void* y, const void* ya, int y_dtype, const void* d
             a.out0 = dx; a.out1 = dxa; a.out_dtype = dx_dtype;
             a.aux0 = x_rec; a.aux1 = xa_rec;
             a.W = W + ps.first * wstride;
-            a.dw_partials = partials;
+            a.dw_partials = region;
             err = (p.path != 2) ? launch_generic(kBackward, a, shape->n_head, p.grid_x, s)
                                 : launch_fast_backward_indexed(a, shape->n_head, p.grid_x, s);
-            if (err != hipSuccess) return (int)err;
-            err = launch_reduce_dw(partials, p.partial_rows, wstride, wstride, level1, dW + ps.first * wstride, s);
         } else {
             FusedArgs a{};
             a.in0 = top ? y : x_rec; a.in1 = top ? ya : xa_rec; a.in_dtype = top ? y_dtype : NCN_F32;
@@ -697,17 +751,14 @@ int ncn_backward_radix(const void* y, const void* ya, int y_dtype, const void* d
             a.out0 = dx; a.out1 = dxa; a.out_dtype = dx_dtype;
             a.aux0 = x_rec; a.aux1 = xa_rec;
             a.W = W + ps.first * wstride;
-            a.dw_partials = partials;
+            a.dw_partials = region;
             fill_step_table(a.tab, shape->n_cache, alpha, m, activation);
             err = launch_fused_radix(kBackward, a, shape, ps, s);
-            if (err != hipSuccess) return (int)err;
-            const int rows = radix_grid(shape, ps, true) / shape->n_head;
-            err = launch_reduce_dw(partials, rows, (int64_t)ps.count * wstride, (int64_t)ps.count * wstride, level1,
-                                   dW + ps.first * wstride, s);
         }
         if (err != hipSuccess) return (int)err;
+        reducer.add(region, rows, ps.count, dW + ps.first * wstride);
     }
-    return NCN_OK;
+    return (int)reducer.flush();
 }
 
 int ncn_inverse_radix(const void* y, const void* ya, int in_dtype, void* x, void* xa, int out_dtype, const float* W,

@@ -186,24 +186,48 @@ __global__ void __launch_bounds__(64) generic_backward_kernel(const StageArgs A)
     }
 }
 
-// out[blockIdx.y][col] = sum of rows [blockIdx.y * rows_per_block, +rows_per_block) of in[row][col].
-// 64 columns x 4 row lanes per block; launched twice (many blocks over row chunks, then one row of blocks) so
-// that the first level has enough loads in flight to run at memory speed.  The order of additions is fixed.
-__global__ void __launch_bounds__(256) reduce_rows_kernel(const float* __restrict__ in, int rows, int64_t row_stride,
-                                                          int64_t cols, int rows_per_block, float* __restrict__ out) {
-    __shared__ float red[4][64];
-    const int cx = threadIdx.x & 63, ry = threadIdx.x >> 6;
-    const int64_t col = (int64_t)blockIdx.x * 64 + cx;
-    const int r0 = blockIdx.y * rows_per_block;
-    const int r1 = min(rows, r0 + rows_per_block);
+// dW partial rows are summed in two launches so that the first has enough loads in flight to run at memory speed:
+// level 1 sums chunks of kReduceRowsPerBlock rows (block y = one chunk of one segment of the job), level 2 the chunk
+// sums of each segment (block y = segment).  A block is 256 / RL columns x RL row lanes (level 2 has few rows of
+// blocks, so it takes narrow blocks with many row lanes); the order of additions is fixed.
+template <int RL>
+__device__ __forceinline__ void reduce_rows(const float* __restrict__ in, int r0, int r1, int64_t row_stride, int64_t cols,
+                                            float* __restrict__ out) {
+    constexpr int CW = 256 / RL;
+    __shared__ float red[RL][CW];
+    const int cx = threadIdx.x % CW, ry = threadIdx.x / CW;
+    const int64_t col = (int64_t)blockIdx.x * CW + cx;
     float sum = 0.f;
     if (col < cols) {
 #pragma unroll 4
-        for (int r = r0 + ry; r < r1; r += 4) sum += in[(int64_t)r * row_stride + col];
+        for (int r = r0 + ry; r < r1; r += RL) sum += in[(int64_t)r * row_stride + col];
     }
     red[ry][cx] = sum;
     __syncthreads();
-    if (ry == 0 && col < cols) out[(int64_t)blockIdx.y * cols + col] = (red[0][cx] + red[1][cx]) + (red[2][cx] + red[3][cx]);
+    if (ry == 0 && col < cols) {
+        float total = 0.f;
+#pragma unroll
+        for (int k = 0; k < RL; k += 4) total += (red[k][cx] + red[k + 1][cx]) + (red[k + 2][cx] + red[k + 3][cx]);
+        out[col] = total;
+    }
+}
+
+constexpr int kReduceLevel1Lanes = 4, kReduceLevel2Lanes = 16;
+
+__global__ void __launch_bounds__(256) reduce_chunks_kernel(const ReduceJob J, float* __restrict__ level1) {
+    int s = 0;
+    while (s + 1 < J.n && (int)blockIdx.y >= J.seg[s + 1].chunk0) ++s;   // at most kReduceMaxSegments - 1 rounds
+    const ReduceSegment& g = J.seg[s];
+    const int chunk = blockIdx.y - g.chunk0;
+    const int r0 = chunk * kReduceRowsPerBlock;
+    reduce_rows<kReduceLevel1Lanes>(g.in, r0, min(g.rows, r0 + kReduceRowsPerBlock), g.cols, g.cols,
+                                    level1 + g.level1_offset + chunk * g.cols);
+}
+
+__global__ void __launch_bounds__(256) reduce_segments_kernel(const ReduceJob J, const float* __restrict__ level1) {
+    const ReduceSegment& g = J.seg[blockIdx.y];
+    const int chunks = (g.rows + kReduceRowsPerBlock - 1) / kReduceRowsPerBlock;
+    reduce_rows<kReduceLevel2Lanes>(level1 + g.level1_offset, 0, chunks, g.cols, g.cols, g.out);
 }
 
 // Rows past a batch entry's context length take no part in the stage: they pass through.
@@ -263,15 +287,19 @@ hipError_t launch_generic(Pass pass, const StageArgs& a, int n_head, int grid_x,
     return hipGetLastError();
 }
 
-hipError_t launch_reduce_dw(const float* partials, int rows, int64_t row_stride, int64_t cols, float* level1, float* dW,
-                            hipStream_t s) {
-    const unsigned col_blocks = (unsigned)((cols + 63) / 64);
-    const int chunks = (rows + kReduceRowsPerBlock - 1) / kReduceRowsPerBlock;  // <= kReduceLevel1Rows
-    hipLaunchKernelGGL(reduce_rows_kernel, dim3(col_blocks, chunks), dim3(256), 0, s, partials, rows, row_stride, cols,
-                       kReduceRowsPerBlock, level1);
+hipError_t launch_reduce_job(const ReduceJob& job, float* level1, hipStream_t s) {
+    if (job.n == 0) return hipSuccess;
+    int64_t max_cols = 0;
+    for (int k = 0; k < job.n; ++k) max_cols = job.seg[k].cols > max_cols ? job.seg[k].cols : max_cols;
+    const ReduceSegment& last = job.seg[job.n - 1];
+    const int chunks = last.chunk0 + (last.rows + kReduceRowsPerBlock - 1) / kReduceRowsPerBlock;
+    constexpr int cw1 = 256 / kReduceLevel1Lanes, cw2 = 256 / kReduceLevel2Lanes;
+    hipLaunchKernelGGL(reduce_chunks_kernel, dim3((unsigned)((max_cols + cw1 - 1) / cw1), chunks), dim3(256), 0, s, job,
+                       level1);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess) return err;
-    hipLaunchKernelGGL(reduce_rows_kernel, dim3(col_blocks, 1), dim3(256), 0, s, level1, chunks, cols, cols, chunks, dW);
+    hipLaunchKernelGGL(reduce_segments_kernel, dim3((unsigned)((max_cols + cw2 - 1) / cw2), job.n), dim3(256), 0, s, job,
+                       level1);
     return hipGetLastError();
 }
 

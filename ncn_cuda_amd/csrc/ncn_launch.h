@@ -40,9 +40,27 @@ constexpr int kMaxGridX = 16384;
 constexpr int kMaxForwardGridX = 1 << 18;
 // dW partial rows are summed in two levels: chunks of kReduceRowsPerBlock rows, then the chunk sums.
 constexpr int kReduceRowsPerBlock = 32;
-// (+ 8: a multi-stage pass reduces its up to 8 stages at once, ceil(rows / 32) chunks of `stages` rows each, where
-// rows * stages <= kMaxGridX)
-constexpr int kReduceLevel1Rows = kMaxGridX / kReduceRowsPerBlock + 8;
+// One reduction job sums up to kReduceMaxSegments partial arrays (one per backward launch of a call) that lie side by
+// side in the partial buffer and hold at most kReduceMaxStages stages between them.
+constexpr int kReduceMaxSegments = 8;
+constexpr int kReduceMaxStages = 8;
+// Rows of 2E floats that level 1 may need: sum over segments of ceil(rows / 32) * stages, where the segments' rows *
+// stages add up to at most kMaxGridX and their stages to at most kReduceMaxStages.
+constexpr int kReduceLevel1Rows = kMaxGridX / kReduceRowsPerBlock + kReduceMaxStages;
+struct ReduceSegment {
+    const float* in;        // [rows][cols], dense
+    float* out;             // [cols]
+    int64_t cols;           // stages of the launch * 2E
+    int64_t level1_offset;  // floats before this segment's chunk sums in the level-1 scratch
+    int rows;
+    int chunk0;             // chunks of the segments before this one
+};
+struct ReduceJob {
+    ReduceSegment seg[kReduceMaxSegments];
+    int n;
+};
+// out[col] of every segment = sum of its rows, in a fixed order; level1 is scratch of kReduceLevel1Rows * 2E floats.
+hipError_t launch_reduce_job(const ReduceJob& job, float* level1, hipStream_t s);
 
 hipError_t launch_fast_forward(Pass pass, const StageArgs& a, int n_head, int grid_x, hipStream_t s);
 hipError_t launch_fast_backward(const StageArgs& a, int n_head, int grid_x, hipStream_t s);
@@ -54,10 +72,6 @@ hipError_t launch_generic(Pass pass, const StageArgs& a, int n_head, int grid_x,
 hipError_t launch_pass_through(Pass pass, const StageArgs& a, int64_t batch, hipStream_t s);
 // gridDim.x of the generic kernel's edge launch (the partly live group of each batch entry) == its dW partial rows.
 constexpr int kEdgeGridX = 256;
-// dW[col] = sum over `rows` rows of partials[row * row_stride + col]; level1 is scratch of kReduceLevel1Rows * cols floats.
-hipError_t launch_reduce_dw(const float* partials, int rows, int64_t row_stride, int64_t cols, float* level1, float* dW,
-                            hipStream_t s);
-
 // ---- multi-stage (LDS-resident) passes, ncn_fused.hip --------------------------------------------------------
 struct FusedArgs;
 struct FusedPass {
