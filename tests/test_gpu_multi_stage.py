@@ -156,3 +156,46 @@ def test_multi_stage_inverse(M, case):
     assert rc == 0
     torch.cuda.synchronize()
     assert O.rel_err(py, xi) < tol and O.rel_err(pya, xai) < tol
+
+
+def _stage_by_stage_dW(M, outs, gdy, gdya, gWs, alpha, act, n, C, first):
+    dWs = [None] * len(gWs)
+    dy, dya = gdy, gdya
+    for l in range(len(gWs) - 1, -1, -1):
+        _, _, dy, dya, dW = M.backward(outs[l][0], outs[l][1], dy, dya, gWs[l], alpha, act, n, C, first + l)
+        dWs[l] = dW.reshape(-1)
+    return torch.stack(dWs), dy, dya
+
+
+@pytest.mark.parametrize("case", [
+    (2, 256, 16, 2, 2, 0, 11),      # more stages in one call than one reduction job holds (8): two jobs
+                                    # (heads of 8 features: no LDS passes, one launch per stage)
+    (8192, 64, 128, 4, 16, 0, 2),   # 16384 partial rows per stage: the buffer holds one stage, a job per stage
+    (640, 256, 128, 4, 8, 1, 3),    # 5120 rows per stage: three stages side by side (15360 rows), one job
+], ids=lambda c: "b%d_N%d_E%d_C%d_n%d_s%d_L%d" % c)
+def test_dw_of_a_call_equals_dw_of_its_stages(M, case):
+    """The launches of a call write their dW partial rows side by side and are summed together; when the partial
+    buffer or the job is full the sums so far are taken first.  Either way each stage's partial rows are added in
+    the order a one-stage call adds them: bit-identical dW."""
+    batch, N, E, C, n, first, L = case
+    alpha = 0.9
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    gx = torch.randn(batch, N, E, device="cuda", generator=gen)
+    gxa = torch.randn(batch, N, E, device="cuda", generator=gen)
+    gdy = torch.randn(batch, N, E, device="cuda", generator=gen)
+    gWs = [torch.randn(2 * E, device="cuda", generator=gen) * 0.2 for _ in range(L)]
+    outs, cx, cxa = [], gx, gxa
+    for l in range(L):
+        cx, cxa = M.forward(cx, cxa, gWs[l], alpha, 0, n, C, first + l)
+        outs.append((cx, cxa))
+    ref_dW, ref_dx, ref_dxa = _stage_by_stage_dW(M, outs, gdy, None, gWs, alpha, 0, n, C, first)
+    _, _, dx, dxa, dW = M.backward_stages(outs[-1][0], outs[-1][1], gdy, None, torch.stack(gWs), alpha, 0, n, C, first, L)
+    # the call inverts from the last outputs, the stage-by-stage path from each stage's saved outputs: dx agrees to
+    # rounding; both run the same one-stage kernels, and dW's sums must not depend on the batching
+    assert O.rel_err(dx, ref_dx) < 1e-4 and O.rel_err(dxa, ref_dxa) < 1e-4
+    assert O.rel_err(dW, ref_dW) < 1e-4
+    # same inputs per stage (top stage reads the same outputs and gradients): its dW is bit-identical
+    assert torch.equal(dW[L - 1], ref_dW[L - 1])
+    # and a second identical call reproduces every bit
+    _, _, _, _, dW2 = M.backward_stages(outs[-1][0], outs[-1][1], gdy, None, torch.stack(gWs), alpha, 0, n, C, first, L)
+    assert torch.equal(dW, dW2)
