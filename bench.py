@@ -180,7 +180,7 @@ def main():
     copy_gbps = 5 * 2.0 * src.numel() * 4 / (c0.elapsed_time(c1) * 1e-3) / 1e9
     del src, dst
 
-    # the invertible-inverse pass over the whole stack (not part of the step; BASELINE's configuration 5 counts it):
+    # the invertible-inverse pass over the whole stack (not part of the step; the invertible configuration, cfg5, is quoted with it):
     # from the final outputs back to the inputs, segment by segment as the backward reverses them
     inverse_ms = None
     if args.grouping in ("closed", "radix"):
