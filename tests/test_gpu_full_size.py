@@ -102,3 +102,43 @@ def test_full_size_inverse_round_trip(M, name):
         xi, xai = M.inverse_stages(y, ya, W[a:a + cnt], 0.9, 0, n, C, a, cnt)
         assert O.rel_err(xi, x) < 1e-4 and O.rel_err(xai, xa) < 1e-4
         x, xa = y, ya
+
+
+@pytest.mark.parametrize("case", [
+    (4100, 4096, 128, 4, 16, 1, 1, torch.bfloat16),   # one-stage register kernels, 2.15e9 elements per array
+    (2060, 8192, 128, 4, 2, 0, 6, torch.float32),     # multi-stage passes, 2.16e9 elements per array
+], ids=["n16_bf16_one_stage", "n2_f32_six_stages"])
+def test_more_than_2_31_elements_per_array(M, case):
+    """Arrays past 2^31 elements (a 288 GB card holds them): element offsets must be 64-bit all the way.  Batch entries
+    are independent, so the first, middle and last entries are checked against the oracle on just those entries, and dW
+    against the sum of the dW of the two halves of the batch."""
+    batch, N, E, C, n, stage, L, dtype = case
+    assert batch * N * E > 2 ** 31
+    g = torch.Generator(device="cuda").manual_seed(1)
+    x = torch.empty(batch, N, E, device="cuda", dtype=dtype).normal_(generator=g)
+    xa = torch.empty(batch, N, E, device="cuda", dtype=dtype).normal_(generator=g)
+    dy = torch.empty(batch, N, E, device="cuda", dtype=dtype).normal_(generator=g)
+    W = torch.randn(L, 2 * E, device="cuda", generator=g) * (0.5 / n ** 0.5)
+    if L > 1:
+        y, ya = M.forward_stages(x, xa, W, 0.9, 0, n, C, stage, L)
+        sy, sya, gd = y, ya, torch.float32
+    else:
+        y, ya, sy, sya = M.forward_stages(x, xa, W[0], 0.9, 0, n, C, stage, 1, save_fp32=True)
+        gd = dtype
+    Wc = W if L > 1 else W[0]
+    xr, xar, dx, dxa, dW = M.backward_stages(sy, sya, dy, None, Wc, 0.9, 0, n, C, stage, L, grad_dtype=gd)
+    sel = [0, batch // 2, batch - 2, batch - 1]
+    f = torch.float64
+    xs, xas, dys = x[sel].cpu().to(f), xa[sel].cpu().to(f), dy[sel].cpu().to(f)
+    ref = O.net_autograd(xs, xas, [w.cpu().to(f) for w in W], dys, torch.zeros_like(dys), 0.9, n, C, first_stage=stage)
+    tol = 2e-2 if dtype == torch.bfloat16 else max(1e-5, 2e-6 * (1 / 0.9) ** (n * L))
+    for got, want in ((y, ref[0]), (ya, ref[1]), (dx, ref[2]), (dxa, ref[3]), (xr, xs), (xar, xas)):
+        assert O.rel_err(got[sel].float().cpu(), want) < tol
+    del x, xa, y, ya, dx, dxa, xr, xar
+    torch.cuda.empty_cache()
+    h = batch // 2
+    halves = [M.backward_stages(sy[sl].contiguous(), sya[sl].contiguous(), dy[sl].contiguous(), None, Wc, 0.9, 0, n, C,
+                                stage, L, grad_dtype=gd)[4] for sl in (slice(0, h), slice(h, batch))]
+    assert O.rel_err(dW, halves[0] + halves[1]) < 1e-4
+    del sy, sya, dy, halves
+    torch.cuda.empty_cache()
