@@ -30,9 +30,12 @@ size_t fused_lds_bytes(int nc, int ec, bool backward, uint32_t window, int n_sta
 
 uint32_t stage_stride_of(int stage, uint32_t groups) {
     if (stage == 0) return 0;
-    uint64_t s = 1 % groups;
-    for (int k = 1; k < stage; ++k) s = (s * 2) % groups;
-    return (uint32_t)s;
+    uint64_t r = 1 % groups, b = 2 % groups;
+    for (uint32_t e = (uint32_t)stage - 1; e; e >>= 1) {   // 2^(stage-1) mod groups by square and multiply
+        if (e & 1) r = r * b % groups;
+        b = b * b % groups;
+    }
+    return (uint32_t)r;
 }
 
 uint32_t floor_pow2(uint32_t v) {

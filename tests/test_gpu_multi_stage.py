@@ -26,6 +26,7 @@ CASES = [
     (2, 2048, 64, 2, 2, 3, 6),     # range that starts at stage 3 (stride 4)
     (1, 256, 32, 1, 2, 0, 8),      # one head; whole ring fits the window from the start
     (5, 64, 128, 4, 4, 0, 3),      # tiny ring (16 groups)
+    (2, 256, 64, 2, 2, 1000003, 3),  # a very high first stage: 2^(stage-1) mod groups is 0 from stage log2(groups)+1 on
 ]
 
 
