@@ -12,11 +12,12 @@ B=16384, D=4096, g=16, bf16 storage / float32 arithmetic, i.e. [batch=128, N=409
 
 Prints ONE JSON line.  `roofline` describes the dominant kernel (the backward stage kernel):
 algorithmic bytes of one launch divided by its average duration, measured with HIP events on the
-launch stream inside the timed region.  `cpu_baseline` times the CPU oracle on a bounded batch
-slice of the same workload on the host cores.
+launch stream inside the timed region.  `cpu_baseline` times the checker's plain C restatement (and, beside it,
+the PyTorch one) on a bounded batch slice of the same workload on the host cores.
 """
 import argparse
 import json
+import math
 import os
 import sys
 import time
@@ -71,7 +72,6 @@ def main():
     import torch
 
     from ncn_cuda_amd import ncn_cuda_module as M
-    from oracle import ncn_oracle as O
 
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
@@ -84,8 +84,13 @@ def main():
     P = batch * N * E
     sbytes = 2 if cfg["dtype"] == "bf16" else 4
 
-    x, xa, Ws, dyi, dya = O.make_inputs(batch, N, E, L, n, seed=0, xa_zero=True, w_scale=cfg["w_scale"],
-                                        dtype=io_dtype)
+    # synthetic inputs, seeded on the CPU: x ~ N(0,1), xa = 0 (as the reference's script starts it), W_l ~ N(0, 1/g)
+    # (times the configuration's scale), upstream gradient ~ N(0,1) on yi only
+    gen = torch.Generator().manual_seed(0)
+    x = torch.randn(batch, N, E, generator=gen).to(io_dtype)
+    xa = torch.zeros(batch, N, E, dtype=io_dtype)
+    Ws = [(torch.randn(2 * E, generator=gen) * (cfg["w_scale"] / math.sqrt(n))).to(io_dtype) for _ in range(L)]
+    dyi = torch.randn(batch, N, E, generator=gen).to(io_dtype)
     dev = torch.device("cuda:0")
     gx, gxa, gdyi = x.to(dev), xa.to(dev), dyi.to(dev)
     gWs = [w.to(dev) for w in Ws]
@@ -261,6 +266,7 @@ def main():
     }
 
     if not args.no_cpu:
+        from oracle import ncn_oracle as O   # the checker, timed here as the CPU baseline and nowhere else in this file
         ncores = os.cpu_count() or 1
         threads = min(ncores, 16)
         torch.set_num_threads(threads)
@@ -285,12 +291,32 @@ def main():
         tl = time.perf_counter()
         O.literal_net_forward(lx, lxa, lWs, alpha, 2, 1)
         literal_s = time.perf_counter() - tl
-        result["cpu_baseline"] = {"value": cpu_tokens_s, "unit": "tokens/s", "cores": threads, "kind": "port",
-                                  "sample": f"first {sample_b} of {batch} batch entries of the same workload "
-                                            f"({sample_b * E} of {tokens} tokens), float32, vectorised PyTorch "
-                                            f"restatement of torch_ref (forward + reversible backward), "
-                                            f"{ts:.1f} s wall",
+        # the plain C restatement (oracle/ncn_oracle.c: scalar loops per group, OpenMP over groups), same step:
+        # forward keeping every stage's outputs, then the reversible backward stage by stage
+        from oracle import c_oracle as CO
+
+        def c_run(b):
+            xs, xas, dys = x[:b].to(f), xa[:b].to(f), dyi[:b].to(f)
+            w32 = [w.to(f) for w in Ws]
+            t = time.perf_counter()
+            CO.net_forward_backward(xs, xas, w32, dys, None, alpha, n, C)
+            return time.perf_counter() - t
+
+        c_run(1)
+        tcp = c_run(probe_b)
+        c_sample_b = int(max(probe_b, min(batch, round(12.0 / max(tcp / probe_b, 1e-6)))))
+        tcs = c_run(c_sample_b)
+        result["cpu_baseline"] = {"value": c_sample_b * E / tcs, "unit": "tokens/s", "cores": CO.threads(),
+                                  "kind": "port",
+                                  "sample": f"first {c_sample_b} of {batch} batch entries of the same workload "
+                                            f"({c_sample_b * E} of {tokens} tokens), float32, plain C restatement of "
+                                            f"torch_ref with OpenMP over the groups (forward + reversible backward), "
+                                            f"{tcs:.1f} s wall",
                                   "host_cpus_visible": ncores,
+                                  "pytorch_restatement": {
+                                      "value": cpu_tokens_s, "unit": "tokens/s", "cores": threads,
+                                      "sample": f"first {sample_b} of {batch} batch entries, float32, vectorised "
+                                                f"PyTorch restatement (forward + reversible backward), {ts:.1f} s wall"},
                                   "literal_loops_cfg1": {"value": 32 / literal_s, "unit": "tokens/s", "cores": 1,
                                                          "sample": "configuration 1 (B=32 D=256 g=2, 8 stages), forward "
                                                                    "only, per-row Python loops as in torch_ref"}}

@@ -1,0 +1,143 @@
+"""ctypes binding and build recipe of oracle/ncn_oracle.c -- TEST INFRASTRUCTURE ONLY (see that file's header).
+
+build() compiles the C restatement twice (float and double) into oracle/libncn_oracle.so with gcc; the CPU tests, and
+the cpu_baseline leg of bench.py, load it.  The shipped package never does.
+"""
+import ctypes
+import os
+import shutil
+import subprocess
+
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libncn_oracle.so")
+SRC = os.path.join(HERE, "ncn_oracle.c")
+# No -march=native: the library is built in one container and run on another machine.  No -ffast-math either: this is
+# a checker.
+CFLAGS = ["-O3", "-fPIC", "-fopenmp", "-std=c11", "-fno-math-errno"]
+
+
+def build(verbose=False):
+    gcc = shutil.which("gcc")
+    if not gcc:
+        raise RuntimeError("gcc not found: cannot build oracle/libncn_oracle.so")
+    objs = []
+    for real, suffix in (("float", "_f32"), ("double", "_f64")):
+        obj = os.path.join(HERE, f"ncn_oracle{suffix}.o")
+        cmd = [gcc, *CFLAGS, f"-DREAL={real}", f"-DSUFFIX={suffix}", "-c", SRC, "-o", obj]
+        proc = subprocess.run(cmd, capture_output=True, text=True)
+        if proc.returncode != 0:
+            raise RuntimeError(f"gcc failed:\n{proc.stdout}\n{proc.stderr}")
+        objs.append(obj)
+    tmp = LIB_PATH + ".tmp"
+    proc = subprocess.run([gcc, "-shared", "-fopenmp", "-o", tmp, *objs, "-lm"], capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"link failed:\n{proc.stdout}\n{proc.stderr}")
+    os.replace(tmp, LIB_PATH)
+    for obj in objs:
+        os.remove(obj)
+    if verbose:
+        print(f"built {LIB_PATH}")
+    return LIB_PATH
+
+
+_lib = None
+
+
+def load():
+    """The built library (built on first use if it is not there: gcc takes a second)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            build()
+        lib = ctypes.CDLL(LIB_PATH)
+        vp, i64, i = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+        for suffix, real in (("_f32", ctypes.c_float), ("_f64", ctypes.c_double)):
+            f = getattr(lib, "ncn_ref_stage_forward" + suffix)
+            f.restype = i
+            f.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i, i, i64, real, real, i, i]
+            b = getattr(lib, "ncn_ref_stage_backward" + suffix)
+            b.restype = i
+            b.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i, i, i64, real, real, i]
+            getattr(lib, "ncn_ref_threads" + suffix).restype = i
+        _lib = lib
+    return _lib
+
+
+def threads():
+    return load().ncn_ref_threads_f32()
+
+
+def _suffix(t):
+    if t.dtype == torch.float32:
+        return "_f32"
+    if t.dtype == torch.float64:
+        return "_f64"
+    raise TypeError("the C oracle takes float32 or float64 CPU tensors")
+
+
+def _c(t):
+    if t.device.type != "cpu":
+        raise ValueError("the C oracle takes CPU tensors")
+    return t.contiguous()
+
+
+def stage_forward(X, Xa, W, alpha, n, C, stage, m=0.9, activation=0, inverse=False):
+    """One stage (or its inverse) on CPU tensors [batch, N, E]; returns (Y, Ya)."""
+    X, Xa, W = _c(X), _c(Xa), _c(W).to(X.dtype)
+    Y, Ya = torch.empty_like(X), torch.empty_like(Xa)
+    batch, N, E = X.shape
+    rc = getattr(load(), "ncn_ref_stage_forward" + _suffix(X))(
+        X.data_ptr(), Xa.data_ptr(), Y.data_ptr(), Ya.data_ptr(), W.data_ptr(), batch, N, E, C, n, stage, alpha, m,
+        activation, 1 if inverse else 0)
+    if rc:
+        raise ValueError(f"C oracle refused the shape (rc {rc})")
+    return Y, Ya
+
+
+def net_forward(x, xa, weights, alpha, n, C, m=0.9, activation=0, first_stage=0):
+    for l, W in enumerate(weights):
+        x, xa = stage_forward(x, xa, W, alpha, n, C, first_stage + l, m, activation)
+    return x, xa
+
+
+def net_inverse(y, ya, weights, alpha, n, C, m=0.9, activation=0, first_stage=0):
+    for l in range(len(weights) - 1, -1, -1):
+        y, ya = stage_forward(y, ya, weights[l], alpha, n, C, first_stage + l, m, activation, inverse=True)
+    return y, ya
+
+
+def stage_backward(Y, Ya, dY, dYa, W, alpha, n, C, stage, m=0.9, activation=0):
+    """Reversible backward of one stage from its outputs; returns (x_rec, xa_rec, dx, dxa, dW[2E] float64)."""
+    Y, Ya, dY, W = _c(Y), _c(Ya), _c(dY), _c(W).to(Y.dtype)
+    dYa = _c(dYa) if dYa is not None else None
+    xr, xar, dx, dxa = (torch.empty_like(Y) for _ in range(4))
+    batch, N, E = Y.shape
+    dW = torch.empty(2 * E, dtype=torch.float64)
+    rc = getattr(load(), "ncn_ref_stage_backward" + _suffix(Y))(
+        Y.data_ptr(), Ya.data_ptr(), dY.data_ptr(), dYa.data_ptr() if dYa is not None else None, W.data_ptr(),
+        xr.data_ptr(), xar.data_ptr(), dx.data_ptr(), dxa.data_ptr(), dW.data_ptr(), batch, N, E, C, n, stage, alpha, m,
+        activation)
+    if rc:
+        raise ValueError(f"C oracle refused the shape (rc {rc})")
+    return xr, xar, dx, dxa, dW
+
+
+def net_forward_backward(x, xa, weights, dy, dya, alpha, n, C, m=0.9, activation=0, first_stage=0):
+    """Forward keeping every stage's outputs, then the reversible backward stage by stage (what an autograd node per
+    stage does).  Returns (yi, ya, dx, dxa, [dW_l])."""
+    outs = []
+    for l, W in enumerate(weights):
+        x, xa = stage_forward(x, xa, W, alpha, n, C, first_stage + l, m, activation)
+        outs.append((x, xa))
+    g, h = dy, dya
+    dWs = [None] * len(weights)
+    for l in range(len(weights) - 1, -1, -1):
+        _, _, g, h, dWs[l] = stage_backward(outs[l][0], outs[l][1], g, h, weights[l], alpha, n, C, first_stage + l, m,
+                                            activation)
+    return outs[-1][0], outs[-1][1], g, h, dWs
+
+
+if __name__ == "__main__":
+    build(verbose=True)

@@ -1,7 +1,8 @@
 """CPU oracle for the NCN layer -- TEST INFRASTRUCTURE ONLY.
 
 Nothing in the shipped package imports this file: it is the checker used by tests/, by
-__graft_entry__.smoke() and by the cpu_baseline leg of bench.py.  It restates, in plain PyTorch on
+__graft_entry__.smoke() and by the cpu_baseline leg of bench.py.  (oracle/ncn_oracle.c is a second, independent
+restatement in plain C, bound by oracle/c_oracle.py; tests/test_oracle_c.py holds the two to each other.)  It restates, in plain PyTorch on
 the CPU, the algorithm of the reference:
 
   * index map            torch_ref/ncn_pytorch.py:12-41        -> group_pos_to_index, stage_positions
