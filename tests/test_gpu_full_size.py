@@ -142,3 +142,25 @@ def test_more_than_2_31_elements_per_array(M, case):
     assert O.rel_err(dW, halves[0] + halves[1]) < 1e-4
     del sy, sya, dy, halves
     torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("name,entries", [("cfg2", None), ("cfg5", None), ("cfg3", None), ("cfg4", None)])
+def test_whole_tensor_against_the_c_oracle(M, name, entries):
+    """Every element, not a slice: the configuration as bench.py runs it against the plain C restatement in float64
+    (oracle/ncn_oracle.c on the host threads: about 25 s for the four configurations on 16 threads).  `entries` cuts
+    the comparison to that many batch entries spread over the batch, for a machine where that is too long."""
+    from oracle import c_oracle as CO
+    batch, N, E, C, n, L, dtype, _ = CONFIGS[name]
+    x, xa, dy, W = _inputs(name)
+    y, ya, dx, dxa, dW = _run(M, x, xa, dy, W, C, n, L, dtype)
+    sel = list(range(batch)) if entries is None else sorted({(k * batch) // entries for k in range(entries)} | {batch - 1})
+    d = torch.float64
+    ref = CO.net_forward_backward(x[sel].cpu().to(d), xa[sel].cpu().to(d), [w.cpu().to(d) for w in W], dy[sel].cpu().to(d),
+                                  None, 0.9, n, C)
+    tol = 2e-2 if dtype == torch.bfloat16 else 1e-5
+    gtol = max(tol, 3e-6 * (1 / 0.9) ** (n * max(1, 26 // n)))     # rounding growth of the reversal per segment
+    assert O.rel_err(y[sel].float().cpu(), ref[0]) < tol and O.rel_err(ya[sel].float().cpu(), ref[1]) < tol
+    assert O.rel_err(dx[sel].float().cpu(), ref[2]) < gtol and O.rel_err(dxa[sel].float().cpu(), ref[3]) < gtol
+    if entries is None:                                            # dW sums over the whole batch
+        for l in range(L):
+            assert O.rel_err(dW[l].cpu(), ref[4][l]) < gtol, l
