@@ -56,10 +56,10 @@ def load():
         for suffix, real in (("_f32", ctypes.c_float), ("_f64", ctypes.c_double)):
             f = getattr(lib, "ncn_ref_stage_forward" + suffix)
             f.restype = i
-            f.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i, i, i64, real, real, i, i]
+            f.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i, i, i64, real, real, i, i, vp, vp]
             b = getattr(lib, "ncn_ref_stage_backward" + suffix)
             b.restype = i
-            b.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i, i, i64, real, real, i]
+            b.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i, i, i64, real, real, i, vp, vp]
             getattr(lib, "ncn_ref_threads" + suffix).restype = i
         _lib = lib
     return _lib
@@ -83,14 +83,27 @@ def _c(t):
     return t.contiguous()
 
 
-def stage_forward(X, Xa, W, alpha, n, C, stage, m=0.9, activation=0, inverse=False):
-    """One stage (or its inverse) on CPU tensors [batch, N, E]; returns (Y, Ya)."""
+def _i32(t, count, what):
+    """An optional int32 array for the C side (None stays NULL); the caller keeps the returned tensor alive."""
+    if t is None:
+        return None, None
+    t = torch.as_tensor(t).to(torch.int32).contiguous()
+    if t.numel() != count:
+        raise ValueError(f"{what} must have {count} entries")
+    return t, t.data_ptr()
+
+
+def stage_forward(X, Xa, W, alpha, n, C, stage, m=0.9, activation=0, inverse=False, table=None, ctx_len=None):
+    """One stage (or its inverse) on CPU tensors [batch, N, E]; returns (Y, Ya).  `table` [N] replaces the stride
+    map (position of slot o of group g at entry g*n + o), `ctx_len` [batch] gives each batch entry its live slots."""
     X, Xa, W = _c(X), _c(Xa), _c(W).to(X.dtype)
     Y, Ya = torch.empty_like(X), torch.empty_like(Xa)
     batch, N, E = X.shape
+    tk, tp = _i32(table, N, "table")
+    lk, lp = _i32(ctx_len, batch, "ctx_len")
     rc = getattr(load(), "ncn_ref_stage_forward" + _suffix(X))(
         X.data_ptr(), Xa.data_ptr(), Y.data_ptr(), Ya.data_ptr(), W.data_ptr(), batch, N, E, C, n, stage, alpha, m,
-        activation, 1 if inverse else 0)
+        activation, 1 if inverse else 0, tp, lp)
     if rc:
         raise ValueError(f"C oracle refused the shape (rc {rc})")
     return Y, Ya
@@ -108,34 +121,38 @@ def net_inverse(y, ya, weights, alpha, n, C, m=0.9, activation=0, first_stage=0)
     return y, ya
 
 
-def stage_backward(Y, Ya, dY, dYa, W, alpha, n, C, stage, m=0.9, activation=0):
+def stage_backward(Y, Ya, dY, dYa, W, alpha, n, C, stage, m=0.9, activation=0, table=None, ctx_len=None):
     """Reversible backward of one stage from its outputs; returns (x_rec, xa_rec, dx, dxa, dW[2E] float64)."""
     Y, Ya, dY, W = _c(Y), _c(Ya), _c(dY), _c(W).to(Y.dtype)
     dYa = _c(dYa) if dYa is not None else None
     xr, xar, dx, dxa = (torch.empty_like(Y) for _ in range(4))
     batch, N, E = Y.shape
     dW = torch.empty(2 * E, dtype=torch.float64)
+    tk, tp = _i32(table, N, "table")
+    lk, lp = _i32(ctx_len, batch, "ctx_len")
     rc = getattr(load(), "ncn_ref_stage_backward" + _suffix(Y))(
         Y.data_ptr(), Ya.data_ptr(), dY.data_ptr(), dYa.data_ptr() if dYa is not None else None, W.data_ptr(),
         xr.data_ptr(), xar.data_ptr(), dx.data_ptr(), dxa.data_ptr(), dW.data_ptr(), batch, N, E, C, n, stage, alpha, m,
-        activation)
+        activation, tp, lp)
     if rc:
         raise ValueError(f"C oracle refused the shape (rc {rc})")
     return xr, xar, dx, dxa, dW
 
 
-def net_forward_backward(x, xa, weights, dy, dya, alpha, n, C, m=0.9, activation=0, first_stage=0):
+def net_forward_backward(x, xa, weights, dy, dya, alpha, n, C, m=0.9, activation=0, first_stage=0, tables=None,
+                         ctx_len=None):
     """Forward keeping every stage's outputs, then the reversible backward stage by stage (what an autograd node per
-    stage does).  Returns (yi, ya, dx, dxa, [dW_l])."""
+    stage does).  `tables` is a list of one table per stage.  Returns (yi, ya, dx, dxa, [dW_l])."""
     outs = []
+    tab = lambda l: None if tables is None else tables[l]
     for l, W in enumerate(weights):
-        x, xa = stage_forward(x, xa, W, alpha, n, C, first_stage + l, m, activation)
+        x, xa = stage_forward(x, xa, W, alpha, n, C, first_stage + l, m, activation, table=tab(l), ctx_len=ctx_len)
         outs.append((x, xa))
     g, h = dy, dya
     dWs = [None] * len(weights)
     for l in range(len(weights) - 1, -1, -1):
         _, _, g, h, dWs[l] = stage_backward(outs[l][0], outs[l][1], g, h, weights[l], alpha, n, C, first_stage + l, m,
-                                            activation)
+                                            activation, table=tab(l), ctx_len=ctx_len)
     return outs[-1][0], outs[-1][1], g, h, dWs
 
 

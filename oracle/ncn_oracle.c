@@ -14,6 +14,11 @@
  *   backward           the closed form of ncn_triton/ncn_triton.py:176-246 (cross-checked with
  *                      ncn_cuda/ncn_bwd_cuda_kernel.cu:124-216): invert a step, recompute T, apply the step's
  *                      vector-Jacobian product; gradients of W summed over batch, groups and rows
+ *   tables, lengths    ncn_triton/ncn_triton_old.py:53-96: `table` [N] gives the position of slot o of group g at entry
+ *                      g n + o (instead of the stride map), `ctx_len` [batch] the live slots of a batch entry: groups
+ *                      below the length run as usual, the group it cuts runs on its live rows with as many steps,
+ *                      rows past the length pass through (y = x, dx = dy; this build's choice, the reference leaves
+ *                      them unwritten)
  *   activations        ncn_fwd_cuda_kernel.cu:86-95 (0 tanh, 1 relu, 2 sigmoid, other linear), 3 = leaky relu with
  *                      slope 0.01 (ncn_triton/ncn_triton.py:22-28)
  *
@@ -127,16 +132,34 @@ static void step_inverse(real* y, real* b, const real* wi, const real* wj, int n
     }
 }
 
-static void gather(const real* src, real* dst, int64_t base, int64_t g, int64_t stride, int64_t groups, int n, int ec,
-                   int64_t E) {
-    for (int o = 0; o < n; ++o)
-        memcpy(dst + (size_t)o * ec, src + base + row_of(g, o, stride, groups, n) * E, sizeof(real) * ec);
+/* positions of the n slots of group g, and how many of them are live for a batch entry of length len */
+static int group_rows(int64_t* pos, int64_t g, int64_t stride, int64_t groups, int n, const int32_t* table, int64_t len) {
+    for (int o = 0; o < n; ++o) pos[o] = table ? (int64_t)table[g * n + o] : row_of(g, o, stride, groups, n);
+    const int64_t live = len - g * n;
+    return live >= n ? n : (live > 0 ? (int)live : 0);
 }
 
-static void scatter(real* dst, const real* src, int64_t base, int64_t g, int64_t stride, int64_t groups, int n, int ec,
-                    int64_t E) {
-    for (int o = 0; o < n; ++o)
-        memcpy(dst + base + row_of(g, o, stride, groups, n) * E, src + (size_t)o * ec, sizeof(real) * ec);
+static void gather(const real* src, real* dst, int64_t base, const int64_t* pos, int rows, int ec, int64_t E) {
+    for (int o = 0; o < rows; ++o) memcpy(dst + (size_t)o * ec, src + base + pos[o] * E, sizeof(real) * ec);
+}
+
+static void scatter(real* dst, const real* src, int64_t base, const int64_t* pos, int rows, int ec, int64_t E) {
+    for (int o = 0; o < rows; ++o) memcpy(dst + base + pos[o] * E, src + (size_t)o * ec, sizeof(real) * ec);
+}
+
+/* slots rows .. n-1 of a group: dst = src (or zeros when src is NULL) */
+static void pass_through(real* dst, const real* src, int64_t base, const int64_t* pos, int rows, int n, int ec,
+                         int64_t E) {
+    for (int o = rows; o < n; ++o) {
+        if (src) memmove(dst + base + pos[o] * E, src + base + pos[o] * E, sizeof(real) * ec);
+        else memset(dst + base + pos[o] * E, 0, sizeof(real) * ec);
+    }
+}
+
+static int64_t entry_len(const int32_t* ctx_len, int64_t b, int64_t N) {
+    if (!ctx_len) return N;
+    const int64_t v = ctx_len[b];
+    return v < 0 ? 0 : (v > N ? N : v);
 }
 
 static int bad_shape(int64_t batch, int64_t N, int64_t E, int C, int n) {
@@ -146,7 +169,7 @@ static int bad_shape(int64_t batch, int64_t N, int64_t E, int C, int n) {
 /* One stage, x, xa -> y, ya (may alias).  Returns 0, or -1 for a shape this file does not handle. */
 int NAME(ncn_ref_stage_forward)(const real* x, const real* xa, real* y, real* ya, const real* W, int64_t batch,
                                 int64_t N, int64_t E, int C, int n, int64_t stage, real alpha, real m, int code,
-                                int inverse) {
+                                int inverse, const int32_t* table, const int32_t* ctx_len) {
     if (bad_shape(batch, N, E, C, n)) return -1;
     const int ec = (int)(E / C);
     const int64_t groups = N / n, stride = stage_stride(stage, groups);
@@ -156,16 +179,20 @@ int NAME(ncn_ref_stage_forward)(const real* x, const real* xa, real* y, real* ya
         const int64_t g = w % groups, c = (w / groups) % C, b = w / (groups * C);
         const int64_t base = b * N * E + c * ec;
         real gx[MAX_N * MAX_EC], ga[MAX_N * MAX_EC];
-        gather(x, gx, base, g, stride, groups, n, ec, E);
-        gather(xa, ga, base, g, stride, groups, n, ec, E);
+        int64_t pos[MAX_N];
+        const int rows = group_rows(pos, g, stride, groups, n, table, entry_len(ctx_len, b, N));
+        gather(x, gx, base, pos, rows, ec, E);
+        gather(xa, ga, base, pos, rows, ec, E);
         const real* wi = W + c * ec;
         const real* wj = W + E + c * ec;
         if (!inverse)
-            for (int j = 0; j < n; ++j) step_forward(gx, ga, wi, wj, n, ec, j, alpha, m, code);
+            for (int j = 0; j < rows; ++j) step_forward(gx, ga, wi, wj, rows, ec, j, alpha, m, code);
         else
-            for (int j = n - 1; j >= 0; --j) step_inverse(gx, ga, wi, wj, n, ec, j, alpha, m, code, 0, 0);
-        scatter(y, gx, base, g, stride, groups, n, ec, E);
-        scatter(ya, ga, base, g, stride, groups, n, ec, E);
+            for (int j = rows - 1; j >= 0; --j) step_inverse(gx, ga, wi, wj, rows, ec, j, alpha, m, code, 0, 0);
+        pass_through(y, x, base, pos, rows, n, ec, E);      /* before the scatter: y may be x */
+        pass_through(ya, xa, base, pos, rows, n, ec, E);
+        scatter(y, gx, base, pos, rows, ec, E);
+        scatter(ya, ga, base, pos, rows, ec, E);
     }
     return 0;
 }
@@ -174,7 +201,8 @@ int NAME(ncn_ref_stage_forward)(const real* x, const real* xa, real* y, real* ya
  * x_rec, xa_rec (may be NULL) get the stage's inputs, dx, dxa the gradients, dW[2E] (double) the weight gradient. */
 int NAME(ncn_ref_stage_backward)(const real* y, const real* ya, const real* dy, const real* dya, const real* W,
                                  real* x_rec, real* xa_rec, real* dx, real* dxa, double* dW, int64_t batch, int64_t N,
-                                 int64_t E, int C, int n, int64_t stage, real alpha, real m, int code) {
+                                 int64_t E, int C, int n, int64_t stage, real alpha, real m, int code,
+                                 const int32_t* table, const int32_t* ctx_len) {
     if (bad_shape(batch, N, E, C, n)) return -1;
     const int ec = (int)(E / C);
     const int64_t groups = N / n, stride = stage_stride(stage, groups);
@@ -198,21 +226,23 @@ int NAME(ncn_ref_stage_backward)(const real* y, const real* ya, const real* dy, 
             const int64_t base = b * N * E + c * ec;
             real gy[MAX_N * MAX_EC], gb[MAX_N * MAX_EC], gg[MAX_N * MAX_EC], gh[MAX_N * MAX_EC], df[MAX_N * MAX_EC];
             real s[MAX_N], r[MAX_N], dxj[MAX_EC];
-            gather(y, gy, base, g, stride, groups, n, ec, E);
-            gather(ya, gb, base, g, stride, groups, n, ec, E);
-            gather(dy, gg, base, g, stride, groups, n, ec, E);
-            if (dya) gather(dya, gh, base, g, stride, groups, n, ec, E);
+            int64_t pos[MAX_N];
+            const int rows = group_rows(pos, g, stride, groups, n, table, entry_len(ctx_len, b, N));
+            gather(y, gy, base, pos, rows, ec, E);
+            gather(ya, gb, base, pos, rows, ec, E);
+            gather(dy, gg, base, pos, rows, ec, E);
+            if (dya) gather(dya, gh, base, pos, rows, ec, E);
             else memset(gh, 0, sizeof(real) * n * ec);
             const real* wi = W + c * ec;
             const real* wj = W + E + c * ec;
             double* dwi = mine + c * ec;
             double* dwj = mine + E + c * ec;
-            for (int j = n - 1; j >= 0; --j) {
-                step_inverse(gy, gb, wi, wj, n, ec, j, alpha, m, code, s, df);   /* gy, gb: the step's inputs now */
+            for (int j = rows - 1; j >= 0; --j) {
+                step_inverse(gy, gb, wi, wj, rows, ec, j, alpha, m, code, s, df);   /* gy, gb: the step's inputs now */
                 const real* xj = gy + (size_t)j * ec;
                 for (int f = 0; f < ec; ++f) dxj[f] = 0;
                 real rsum = 0;
-                for (int i = 0; i < n; ++i) {
+                for (int i = 0; i < rows; ++i) {
                     const real* xi = gy + (size_t)i * ec;
                     real* gi = gg + (size_t)i * ec;
                     real* hi = gh + (size_t)i * ec;
@@ -237,10 +267,14 @@ int NAME(ncn_ref_stage_backward)(const real* y, const real* ya, const real* dy, 
                     gg[(size_t)j * ec + f] += dxj[f];
                 }
             }
-            scatter(dx, gg, base, g, stride, groups, n, ec, E);
-            scatter(dxa, gh, base, g, stride, groups, n, ec, E);
-            if (x_rec) scatter(x_rec, gy, base, g, stride, groups, n, ec, E);
-            if (xa_rec) scatter(xa_rec, gb, base, g, stride, groups, n, ec, E);
+            pass_through(dx, dy, base, pos, rows, n, ec, E);
+            pass_through(dxa, dya, base, pos, rows, n, ec, E);
+            if (x_rec) pass_through(x_rec, y, base, pos, rows, n, ec, E);
+            if (xa_rec) pass_through(xa_rec, ya, base, pos, rows, n, ec, E);
+            scatter(dx, gg, base, pos, rows, ec, E);
+            scatter(dxa, gh, base, pos, rows, ec, E);
+            if (x_rec) scatter(x_rec, gy, base, pos, rows, ec, E);
+            if (xa_rec) scatter(xa_rec, gb, base, pos, rows, ec, E);
         }
     }
     for (int64_t k = 0; k < 2 * E; ++k) {

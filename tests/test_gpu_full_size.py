@@ -164,3 +164,53 @@ def test_whole_tensor_against_the_c_oracle(M, name, entries):
     if entries is None:                                            # dW sums over the whole batch
         for l in range(L):
             assert O.rel_err(dW[l].cpu(), ref[4][l]) < gtol, l
+
+
+def test_headline_shape_with_table_and_lengths_against_the_c_oracle(M):
+    """cfg3 through the table / context-length entry points (a different length per batch entry, a radix-16 table on
+    stage 1), every element against the C oracle in float64."""
+    from oracle import c_oracle as CO
+    batch, N, E, C, n, L, dtype, _ = CONFIGS["cfg3"]
+    x, xa, dy, W = _inputs("cfg3")
+    tables = [O.stride_group_table(N, n, 0), O.radix_group_table(N, n, 1), O.stride_group_table(N, n, 2)]
+    lens = (N - 1 - 37 * torch.arange(batch)) % (N + 1)
+    lens[0], lens[1] = N, 0
+    gt = [t.to(torch.int32).cuda() for t in tables]
+    gl = lens.to(torch.int32).cuda()
+    saved, cx, cxa = [], x, xa
+    for l in range(L):
+        cx, cxa, y32, ya32 = M.forward_stages(cx, cxa, W[l], 0.9, 0, n, C, l, 1, save_fp32=True, group_index=gt[l],
+                                              ctx_len=gl)
+        saved.append((y32, ya32))
+    g, h, dWs = dy, None, [None] * L
+    for l in range(L - 1, -1, -1):
+        _, _, g, h, dWs[l] = M.backward_stages(saved[l][0], saved[l][1], g, h, W[l], 0.9, 0, n, C, l, 1, grad_dtype=dtype,
+                                               want_inputs=False, group_index=gt[l], ctx_len=gl)
+    d = torch.float64
+    ref = CO.net_forward_backward(x.cpu().to(d), xa.cpu().to(d), [w.cpu().to(d) for w in W], dy.cpu().to(d), None, 0.9, n,
+                                  C, tables=tables, ctx_len=lens)
+    tol = 2e-2
+    assert O.rel_err(cx.float().cpu(), ref[0]) < tol and O.rel_err(cxa.float().cpu(), ref[1]) < tol
+    assert O.rel_err(g.float().cpu(), ref[2]) < tol and O.rel_err(h.float().cpu(), ref[3]) < tol
+    for l in range(L):
+        assert O.rel_err(dWs[l][0].cpu(), ref[4][l]) < tol, l
+
+
+def test_deep_shape_radix_levels_against_the_c_oracle(M):
+    """cfg4's tensors through the 13 levels of the radix-2 grouping (two multi-level LDS passes each way), every element
+    against the C oracle in float64 on the radix tables."""
+    from oracle import c_oracle as CO
+    batch, N, E, C, n, L, dtype, _ = CONFIGS["cfg4"]
+    x, xa, dy, W = _inputs("cfg4")
+    y, ya = M.forward_radix(x, xa, W, 0.9, 0, n, C, 0, L)
+    xr, xar, dx, dxa, dW = M.backward_radix(y, ya, dy, None, W, 0.9, 0, n, C, 0, L)
+    tables = [O.radix_group_table(N, n, l) for l in range(L)]
+    d = torch.float64
+    ref = CO.net_forward_backward(x.cpu().to(d), xa.cpu().to(d), [w.cpu().to(d) for w in W], dy.cpu().to(d), None, 0.9, n,
+                                  C, tables=tables)
+    gtol = max(1e-5, 3e-6 * (1 / 0.9) ** (n * L))
+    assert O.rel_err(y.cpu(), ref[0]) < 1e-5 and O.rel_err(ya.cpu(), ref[1]) < 1e-5
+    assert O.rel_err(dx.cpu(), ref[2]) < gtol and O.rel_err(dxa.cpu(), ref[3]) < gtol
+    assert O.rel_err(xr.cpu(), x.cpu().to(d)) < gtol
+    for l in range(L):
+        assert O.rel_err(dW[l].cpu(), ref[4][l]) < gtol, l

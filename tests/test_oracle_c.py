@@ -101,3 +101,57 @@ def test_refuses_what_it_cannot_hold():
         CO.stage_forward(x, x, torch.zeros(8), 0.9, 65, 1, 0)      # more rows per group than the C arrays hold
     with pytest.raises(ValueError):
         CO.stage_forward(torch.zeros(1, 4, 6), torch.zeros(1, 4, 6), torch.zeros(12), 0.9, 3, 1, 0)   # N % n != 0
+
+
+@pytest.mark.parametrize("case", [(3, 32, 16, 2, 4, 2, 0), (2, 30, 12, 3, 5, 1, 3), (4, 64, 32, 1, 16, 2, 2), (2, 24, 8, 2, 3, 2, -1)],
+                         ids=lambda c: "b%d_N%d_E%d_C%d_n%d_L%d_a%d" % c)
+def test_tables_and_lengths_match_python_oracle(case):
+    batch, N, E, C, n, L, act = case
+    d = torch.float64
+    x, xa, Ws, dy, dya = O.make_inputs(batch, N, E, L, n, seed=8, xa_zero=False)
+    gen = torch.Generator().manual_seed(N)
+    tables = [torch.randperm(N, generator=gen) for _ in range(L)]
+    for lens in (None, [N] * batch, [int(v) for v in torch.randint(0, N + 1, (batch,), generator=gen)]):
+        ref = O.net_autograd_indexed(x.to(d), xa.to(d), [w.to(d) for w in Ws], dy.to(d), dya.to(d), 0.9, n, C, tables,
+                                     lens, activation=act)
+        got = CO.net_forward_backward(x.to(d), xa.to(d), [w.to(d) for w in Ws], dy.to(d), dya.to(d), 0.9, n, C,
+                                      activation=act, tables=tables, ctx_len=lens)
+        tol = 1e-12 * (1 / 0.9) ** n
+        for k in range(4):
+            assert O.rel_err(got[k], ref[k]) < tol, (lens, k)
+        for l in range(L):
+            assert O.rel_err(got[4][l], ref[4][l]) < tol, (lens, l)
+    # the stride map as a table is the closed form, bit for bit
+    st = [O.stride_group_table(N, n, l) for l in range(L)]
+    a = CO.net_forward_backward(x, xa, Ws, dy, dya, 0.9, n, C, activation=act)
+    b = CO.net_forward_backward(x, xa, Ws, dy, dya, 0.9, n, C, activation=act, tables=st)
+    assert all(torch.equal(p, q) for p, q in zip(a[:4], b[:4]))
+
+
+def test_tables_and_lengths_match_triton_vectors():
+    """The older Triton kernels' outputs (tests/golden/triton_tables_lengths.npz): whole-group lengths forward and
+    backward on the live rows, the cut group's live rows forward."""
+    g = load_npz("triton_tables_lengths")
+    batch, N, E, C, n = (int(v) for v in g["meta"])
+    alpha = float(g["alpha"])
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a))
+    codes = {"tanh": 0, "leaky-relu": 3}
+    for k in range(int(g["n_whole"])):
+        tag = f"whole{k}_"
+        table = t(g["table_" + str(g[tag + "table"])])
+        live = t(g[tag + "live"])[:, :, None].expand(batch, N, E)
+        if not bool(live.any()):
+            continue
+        x, W = t(g[tag + "x"]), t(g[tag + "W"])
+        got = CO.net_forward_backward(x, torch.zeros_like(x), [W], t(g[tag + "dyi"]), t(g[tag + "dya"]), alpha, n, C,
+                                      activation=codes[str(g[tag + "act"])], tables=[table], ctx_len=t(g[tag + "ctx_len"]))
+        for got_k, key in zip(got[:4], ("yi", "ya", "dx", "dxa")):
+            assert O.rel_err(got_k[live], t(g[tag + key])[live]) < 3e-6, (k, key)
+        assert O.rel_err(got[4][0], t(g[tag + "dW0"])) < 3e-6, k
+    for k in range(int(g["n_cut"])):
+        tag = f"cut{k}_"
+        table = t(g["table_" + str(g[tag + "table"])])
+        check = t(g[tag + "check"])[:, :, None].expand(batch, N, E)
+        x, W = t(g[tag + "x"]), t(g[tag + "W"])
+        yi, ya = CO.stage_forward(x, torch.zeros_like(x), W, alpha, n, C, 0, table=table, ctx_len=t(g[tag + "ctx_len"]))
+        assert O.rel_err(yi[check], t(g[tag + "yi"])[check]) < 3e-6 and O.rel_err(ya[check], t(g[tag + "ya"])[check]) < 3e-6
