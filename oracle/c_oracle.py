@@ -140,20 +140,25 @@ def stage_backward(Y, Ya, dY, dYa, W, alpha, n, C, stage, m=0.9, activation=0, t
 
 
 def net_forward_backward(x, xa, weights, dy, dya, alpha, n, C, m=0.9, activation=0, first_stage=0, tables=None,
-                         ctx_len=None):
+                         ctx_len=None, keep_outputs=True):
     """Forward keeping every stage's outputs, then the reversible backward stage by stage (what an autograd node per
-    stage does).  `tables` is a list of one table per stage.  Returns (yi, ya, dx, dxa, [dW_l])."""
+    stage does).  keep_outputs=False keeps only the last stage's outputs and lets each backward stage hand the
+    inputs it reconstructs to the one below (for float64 runs on tensors too large to keep L copies of).  `tables`
+    is a list of one table per stage.  Returns (yi, ya, dx, dxa, [dW_l])."""
     outs = []
     tab = lambda l: None if tables is None else tables[l]
     for l, W in enumerate(weights):
         x, xa = stage_forward(x, xa, W, alpha, n, C, first_stage + l, m, activation, table=tab(l), ctx_len=ctx_len)
-        outs.append((x, xa))
+        if keep_outputs:
+            outs.append((x, xa))
+    yi, ya = x, xa
     g, h = dy, dya
     dWs = [None] * len(weights)
     for l in range(len(weights) - 1, -1, -1):
-        _, _, g, h, dWs[l] = stage_backward(outs[l][0], outs[l][1], g, h, weights[l], alpha, n, C, first_stage + l, m,
-                                            activation, table=tab(l), ctx_len=ctx_len)
-    return outs[-1][0], outs[-1][1], g, h, dWs
+        cy, cya = outs.pop() if keep_outputs else (x, xa)
+        x, xa, g, h, dWs[l] = stage_backward(cy, cya, g, h, weights[l], alpha, n, C, first_stage + l, m, activation,
+                                             table=tab(l), ctx_len=ctx_len)
+    return yi, ya, g, h, dWs
 
 
 if __name__ == "__main__":

@@ -155,3 +155,15 @@ def test_tables_and_lengths_match_triton_vectors():
         x, W = t(g[tag + "x"]), t(g[tag + "W"])
         yi, ya = CO.stage_forward(x, torch.zeros_like(x), W, alpha, n, C, 0, table=table, ctx_len=t(g[tag + "ctx_len"]))
         assert O.rel_err(yi[check], t(g[tag + "yi"])[check]) < 3e-6 and O.rel_err(ya[check], t(g[tag + "ya"])[check]) < 3e-6
+
+
+def test_reversal_without_kept_outputs_is_the_same_in_float64():
+    d = torch.float64
+    x, xa, Ws, dy, dya = O.make_inputs(2, 64, 32, 4, 4, seed=2, xa_zero=False)
+    args = (x.to(d), xa.to(d), [w.to(d) for w in Ws], dy.to(d), dya.to(d), 0.9, 4, 2)
+    a = CO.net_forward_backward(*args)
+    b = CO.net_forward_backward(*args, keep_outputs=False)
+    for p, q in zip(a[:4], b[:4]):
+        assert O.rel_err(q, p) < 1e-12
+    for p, q in zip(a[4], b[4]):
+        assert O.rel_err(q, p) < 1e-12
