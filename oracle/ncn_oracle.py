@@ -26,14 +26,15 @@ The leaky-relu and linear activations (forward and closed-form backward), groupi
 radix tables and context lengths are pinned by tests/golden/triton_*.npz, which
 tests/golden/make_golden_triton.py wrote by running the reference's Triton kernels
 (ncn_triton/ncn_triton.py, ncn_triton_old.py) under Triton's CPU interpreter: whole groups below a
-length forward and backward, the group a length cuts forward only (the reference's backward of a cut
-group reads rows that alias position 0, an artefact).
+length and the group a length cuts, forward and backward (the reference's kernel lets the rows past the
+length alias position 0; the cut-group vectors use tables that keep position 0 among the dead rows,
+where that is harmless).
 Still parity unpinned:
   * the relu and sigmoid activations: they exist only in the reference's CUDA kernels
     (ncn_fwd_cuda_kernel.cu:86-95), which cannot be built here; pinned by autograd-vs-closed-form and
     special cases only;
-  * the backward of a cut group, and what happens to rows past a length: the reference leaves those rows
-    unwritten; stage_forward_indexed passes them through, which is this build's choice.
+  * what happens to rows past a length: the reference leaves those rows unwritten;
+    stage_forward_indexed passes them through, which is this build's choice.
 """
 import math
 

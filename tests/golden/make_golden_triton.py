@@ -26,7 +26,9 @@ What the older kernel's outputs mean (read off ncn_triton_old.py, and visible in
     fill is 0, so they alias position 0: they take part as ordinary rows and are stored over position 0.  The live
     rows never see them (a row's step only reads itself and the pivot, and only live rows are pivots), so the
     forward of live rows is well defined except at position 0; the backward sums over all rows of the group and
-    reads what the forward left at position 0, so with a cut group it is an artefact and is not recorded.
+    reads what the forward left at position 0, so with a cut group it is an artefact -- unless position 0 is itself a
+    dead row (a table that puts it in the last slot) and dead rows carry no upstream gradient: those cases are
+    recorded forward and backward (`cutbwd*`).
   * xa is ignored and starts from zeros (:79): the fixtures pass zeros.
 """
 import os
@@ -175,6 +177,38 @@ def tables_and_lengths(TO, G):
                          tag + "W": W.numpy(), tag + "yi": np.where(m, yi.numpy(), 0.0).astype(np.float32),
                          tag + "ya": np.where(m, ya.numpy(), 0.0).astype(np.float32)})
     blob["n_cut"] = np.array(k)
+    # lengths that cut a group, forward AND backward: with position 0 in the table's last slot it is a dead row for
+    # every length below N, so the rows that alias it disturb nobody live, and with no upstream gradient on dead rows
+    # (u = 0, r = 0 for them) they add nothing to the pivot row's gradient or to dW: the kernel's backward of the cut
+    # group is then well defined on the live rows
+    k = 0
+    for trial in range(2):
+        perm = torch.randperm(N, generator=gen)
+        at = int((perm == 0).nonzero()[0])
+        perm[at], perm[N - 1] = perm[N - 1].clone(), perm[at].clone()
+        table = perm.to(torch.int32)
+        for lens in ([7, 13, 30], [1, 18, 31], [5, 5, 22]):
+            x = _draw(gen, batch, N, E)
+            W = _draw(gen, 2 * E, scale=0.3)
+            ctx = torch.tensor(lens, dtype=torch.int32)
+            live = torch.zeros(batch, N, dtype=torch.bool)
+            for b in range(batch):
+                live[b, table[:lens[b]].long()] = True
+            dyi = _draw(gen, batch, N, E) * live[:, :, None]
+            dya = _draw(gen, batch, N, E) * live[:, :, None]
+            act = "tanh" if k % 2 == 0 else "leaky-relu"
+            out = _run(lambda a, b_, ws: TO.fused_chunk_linear_ncn(a, b_, ws[0], table, ctx, ALPHA, act, C, n, 0),
+                       x, torch.zeros(batch, N, E), [W], dyi, dya)
+            tag = f"cutbwd{k}_"
+            k += 1
+            blob[tag + "act"] = np.array(act)
+            blob.update({tag + "table": table.numpy(), tag + "ctx_len": ctx.numpy(), tag + "live": live.numpy(),
+                         tag + "x": x.numpy(), tag + "W": W.numpy(), tag + "dyi": dyi.numpy(), tag + "dya": dya.numpy()})
+            for key, v in out.items():
+                if key in ("yi", "ya", "dx", "dxa"):
+                    v = np.where(live.numpy()[:, :, None], v, 0.0).astype(np.float32)
+                blob[tag + key] = v
+    blob["n_cutbwd"] = np.array(k)
     return blob
 
 

@@ -108,3 +108,22 @@ def test_headline_tile_stack(surfaces, storage):
         assert O.rel_err(got.detach().float().cpu(), torch.from_numpy(g[key])) < tol, key
     for l in range(L):
         assert O.rel_err(Ws[l].grad.float().cpu(), torch.from_numpy(g[f"dW{l}"])) < tol, l
+
+
+@pytest.mark.parametrize("k", list(range(6)))
+def test_cut_group_forward_and_backward(surfaces, k):
+    """A length that cuts a group, both directions, against the reference's kernels (fixtures with position 0 among
+    the dead rows): forward, dx, dxa on the live rows and dW."""
+    _, CL = surfaces
+    g = load_npz("triton_tables_lengths")
+    batch, N, E, C, n = (int(v) for v in g["meta"])
+    tag = f"cutbwd{k}_"
+    live = torch.from_numpy(g[tag + "live"])[:, :, None].expand(batch, N, E)
+    x, W = _g(g[tag + "x"], True), _g(g[tag + "W"], True)
+    xa = torch.zeros_like(x).requires_grad_()
+    yi, ya = CL.fused_chunk_linear_ncn(x, xa, W, _g(g[tag + "table"]), _g(g[tag + "ctx_len"]), float(g["alpha"]),
+                                       str(g[tag + "act"]), C, n, 0)
+    torch.autograd.backward([yi, ya], [_g(g[tag + "dyi"]), _g(g[tag + "dya"])])
+    for got, key in ((yi, "yi"), (ya, "ya"), (x.grad, "dx"), (xa.grad, "dxa")):
+        assert O.rel_err(got.detach().cpu()[live], torch.from_numpy(g[tag + key])[live]) < TOL, key
+    assert O.rel_err(W.grad.cpu(), torch.from_numpy(g[tag + "dW0"])) < TOL

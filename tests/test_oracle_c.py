@@ -167,3 +167,20 @@ def test_reversal_without_kept_outputs_is_the_same_in_float64():
         assert O.rel_err(q, p) < 1e-12
     for p, q in zip(a[4], b[4]):
         assert O.rel_err(q, p) < 1e-12
+
+
+def test_cut_group_backward_matches_triton_vectors():
+    g = load_npz("triton_tables_lengths")
+    batch, N, E, C, n = (int(v) for v in g["meta"])
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a))
+    codes = {"tanh": 0, "leaky-relu": 3}
+    for k in range(int(g["n_cutbwd"])):
+        tag = f"cutbwd{k}_"
+        live = t(g[tag + "live"])[:, :, None].expand(batch, N, E)
+        x, W = t(g[tag + "x"]), t(g[tag + "W"])
+        got = CO.net_forward_backward(x, torch.zeros_like(x), [W], t(g[tag + "dyi"]), t(g[tag + "dya"]), float(g["alpha"]),
+                                      n, C, activation=codes[str(g[tag + "act"])], tables=[t(g[tag + "table"])],
+                                      ctx_len=t(g[tag + "ctx_len"]))
+        for got_k, key in zip(got[:4], ("yi", "ya", "dx", "dxa")):
+            assert O.rel_err(got_k[live], t(g[tag + key])[live]) < 3e-6, (k, key)
+        assert O.rel_err(got[4][0], t(g[tag + "dW0"])) < 3e-6, k

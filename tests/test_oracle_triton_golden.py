@@ -127,3 +127,25 @@ def test_headline_tile_stack():
         assert O.rel_err(got, _t(g[key])) < TOL, key
     for l in range(L):
         assert O.rel_err(dWs[l], _t(g[f"dW{l}"])) < TOL, l
+
+
+@pytest.mark.parametrize("k", list(range(6)))
+def test_cut_group_forward_and_backward(k):
+    """The group a length cuts, both directions (fixtures with position 0 among the dead rows, see the generator):
+    steps and pivots are the live rows, dead rows add nothing to dx or dW."""
+    g = load_npz("triton_tables_lengths")
+    assert int(g["n_cutbwd"]) == 6
+    batch, N, E, C, n = (int(v) for v in g["meta"])
+    tag = f"cutbwd{k}_"
+    table = _t(g[tag + "table"]).long()
+    ctx = _t(g[tag + "ctx_len"])
+    assert any(int(v) % n for v in ctx)                         # at least one batch entry has a cut group
+    live = _t(g[tag + "live"])[:, :, None].expand(batch, N, E)
+    x, W, dyi, dya = (_t(g[tag + key]) for key in ("x", "W", "dyi", "dya"))
+    d = torch.float64
+    yi, ya, dx, dxa, dWs = O.net_autograd_indexed(x.to(d), torch.zeros_like(x).to(d), [W.to(d)], dyi.to(d), dya.to(d),
+                                                  float(g["alpha"]), n, C, [table], ctx,
+                                                  activation=CODES[str(g[tag + "act"])])
+    for got, key in ((yi, "yi"), (ya, "ya"), (dx, "dx"), (dxa, "dxa")):
+        assert O.rel_err(got[live], _t(g[tag + key])[live]) < TOL, key
+    assert O.rel_err(dWs[0], _t(g[tag + "dW0"])) < TOL
