@@ -13,9 +13,8 @@ grouping is whatever the table says.
 Differences with that file, all deliberate:
   * xa is used (the reference's forward ignores its xa argument and starts from zeros, :79);
   * rows past the context length pass through (y = x, ya = xa, gradients likewise); the reference leaves them
-    unwritten in `torch.empty_like` outputs (:294-295) and, in the group the length cuts, reads position 0 for them;
-  * the reference's backward rebuilds only x, not xa, from the outputs (:197); here both are inverted, as in the
-    CUDA kernels (ncn_bwd_cuda_kernel.cu:88-115).
+    unwritten in `torch.empty_like` outputs (:294-295) and, in the group the length cuts, reads position 0 for them.
+The backward inverts the outputs step by step as the reference's does (:197-216), one step per live row.
 
 Tables: stride_group_table is the stride permutation of the current kernels (torch_ref/ncn_pytorch.py:12-41),
 radix_group_table the radix-n digit grouping of ncn_triton/group_tensors.py:8-18.
