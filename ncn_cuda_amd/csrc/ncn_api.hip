@@ -26,6 +26,19 @@ int kernel_path(const ncn_shape* sh, int /*activation*/) {
     return 0;
 }
 
+// The register kernels carry x times 2 log2(e) alpha and xa times that and (1-m) (StepTable): alpha, m and 1-m must
+// stay away from zero.  Other values go to the generic kernels, which use the plain formulas.
+bool scalars_fit_scaled_state(float alpha, float m) {
+    return alpha >= 1e-3f && alpha <= 1e3f && m >= 1e-3f && m <= 1.0f - 1e-3f;
+}
+
+// kernel_path() for a call with these scalars: 2, 1, or 0 when nothing can run it
+int kernel_path_for(const ncn_shape* sh, int activation, float alpha, float m) {
+    const int path = kernel_path(sh, activation);
+    if (path != 2 || scalars_fit_scaled_state(alpha, m)) return path;
+    return (sh->E / sh->n_head <= kGenericMaxHeadDim) ? 1 : 0;
+}
+
 int check_shape(const ncn_shape* sh, int first_stage, int n_stages, int activation) {
     if (!sh) return NCN_ERR_NULL;
     if (sh->batch <= 0 || sh->N <= 0 || sh->E <= 0 || sh->n_head <= 0 || sh->n_cache <= 0) return NCN_ERR_SHAPE;
@@ -61,10 +74,10 @@ struct Plan {
 };
 
 // reserve_rows: rows of the dW partial buffer kept free for another launch of the same stage
-Plan make_plan(const ncn_shape* sh, int activation, int reserve_rows = 0) {
+Plan make_plan(const ncn_shape* sh, int path, int reserve_rows = 0) {
     Plan p;
     const int max_rows = kMaxGridX - reserve_rows;
-    p.path = kernel_path(sh, activation);
+    p.path = path;
     const int ec = (int)(sh->E / sh->n_head);
     p.groups_per_tile = (p.path == 2) ? fast_groups_per_tile(sh->n_cache, ec) : generic_groups_per_tile(sh->n_cache);
     p.groups = (uint32_t)(sh->N / sh->n_cache);
@@ -100,7 +113,7 @@ Plan make_plan(const ncn_shape* sh, int activation, int reserve_rows = 0) {
 
 void fill_step_table(StepTable& t, int n_cache, float alpha, float m, int activation = NCN_ACT_TANH) {
     // a call fills the same table for every stage it launches, and callers repeat (alpha, m) step after step:
-    // keep the last one per thread (some 450 pow() otherwise)
+    // keep the last one per thread (some 70 pow() otherwise)
     thread_local StepTable cached;
     thread_local int cached_n = -1;
     if (cached_n == n_cache && cached.alpha == alpha && cached.m == m) {
@@ -108,23 +121,33 @@ void fill_step_table(StepTable& t, int n_cache, float alpha, float m, int activa
         t.activation = activation;
         return;
     }
-    const double md = m, al = alpha, k2l = 2.8853900817779268;
+    const double md = m, al = alpha, k2l = 2.8853900817779268, om = 1.0 - md, im = 1.0 / md;
+    // the generic kernels read alpha and m only; for scalars that do not fit the scaled state the rest stays finite
+    const bool fit = scalars_fit_scaled_state(alpha, m);
+    const double kappa = fit ? k2l * al : 1.0, ks = fit ? kappa * om : 1.0;
     t.alpha = alpha;
     t.m = m;
     t.activation = activation;
     t.reserved = 0;
+    t.kappa = (float)kappa;
+    t.inv_kappa = (float)(1.0 / kappa);
+    t.a_scale = (float)ks;
+    t.inv_a_scale = (float)(1.0 / ks);
+    t.b_scale = (float)(ks * im);
+    t.inv_b_scale = (float)(md / ks);
+    t.gamma = (float)(fit ? (1.0 - al) / (k2l * al * al) : 0.0);
+    t.om = (float)om;
+    t.im = (float)im;
+    const double k2 = kappa * om * om;
+    t.k2 = (float)k2;
+    t.m2k2 = (float)(-2.0 * k2);
+    t.bk0 = (float)(-k2 * im * im);
+    t.bk1 = (float)(2.0 * k2 * im * im);
+    t.ku = (float)(4.0 * om * al * im);
     t.m_pow_n = (float)std::pow(md, (double)n_cache);
     t.inv_m_pow_n = (float)std::pow(md, -(double)n_cache);
-    for (int k = 0; k < 64; ++k) {
-        const double im = std::pow(md, -(double)(k + 1)), mt = std::pow(md, (double)k);
-        t.step[k].lam = (float)(k2l * al * im);
-        t.step[k].kc2 = (float)(k2l * (1.0 - al) * im * im);
-        t.step[k].kap = (float)((1.0 - md) * mt);
-        t.step[k].krho = (float)(4.0 * (1.0 - md) / md * (1.0 - al) * im);
-        t.step[k].flam = (float)(k2l * al * mt);
-        t.step[k].fkc = (float)(k2l * (1.0 - al) * mt * mt);
-        t.step[k].fkap = (float)((1.0 - md) * im);
-    }
+    t.reserved2 = 0.f;
+    for (int k = 0; k < 64; ++k) t.krho[k] = (float)((1.0 - al) * 4.0 * om * std::pow(md, (double)k) / (kappa * kappa));
     cached = t;
     cached_n = n_cache;
 }
@@ -206,9 +229,10 @@ size_t base_workspace_bytes(const ncn_shape* sh) {
 }
 
 // the multi-stage plan of a stage range, or an empty vector when the one-stage loop should be used
-std::vector<FusedPass> multi_stage_plan(const ncn_shape* sh, int first_stage, int n_stages, int activation, bool backward) {
+std::vector<FusedPass> multi_stage_plan(const ncn_shape* sh, int first_stage, int n_stages, int activation, bool backward,
+                                        int path = 2) {
     std::vector<FusedPass> none;
-    if (n_stages < 2 || kernel_path(sh, activation) != 2 || !fused_supported(sh, activation)) return none;
+    if (n_stages < 2 || path != 2 || kernel_path(sh, activation) != 2 || !fused_supported(sh, activation)) return none;
     std::vector<FusedPass> passes = plan_fused(sh, first_stage, n_stages, backward);
     bool any = false;
     for (const FusedPass& p : passes) any = any || !p.single;
@@ -348,13 +372,15 @@ static int forward_impl(const void* x, const void* xa, int in_dtype, void* y, vo
     if (!aligned16(x) || !aligned16(xa) || !aligned16(y) || !aligned16(ya) || !aligned16(W) || !aligned16(y32) ||
         !aligned16(ya32) || !aligned16(workspace))
         return NCN_ERR_ALIGN;
-    const Plan p = make_plan(shape, activation);
+    const int path = kernel_path_for(shape, activation, alpha, m);
+    if (path == 0) return NCN_ERR_UNSUPPORTED;
+    const Plan p = make_plan(shape, path);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int64_t wstride = 2 * shape->E;
 
     // several stages: LDS-resident passes when the shape allows and the buffers permit the ping-pong
     std::vector<FusedPass> passes;
-    if (grouping.plain()) passes = multi_stage_plan(shape, first_stage, n_stages, activation, false);
+    if (grouping.plain()) passes = multi_stage_plan(shape, first_stage, n_stages, activation, false, path);
     const size_t np = passes.size();
     bool fused_ok = np > 0;
     if (np >= 2 && (out_dtype != NCN_F32 || !workspace || workspace_bytes < temp_bytes(shape, false))) fused_ok = false;
@@ -431,7 +457,9 @@ static int inverse_impl(const void* y, const void* ya, int in_dtype, void* x, vo
     if (!x || !xa || !y || !ya || !W) return NCN_ERR_NULL;
     if (!known_dtype(in_dtype) || !known_dtype(out_dtype)) return NCN_ERR_DTYPE;
     if (!aligned16(x) || !aligned16(xa) || !aligned16(y) || !aligned16(ya) || !aligned16(W)) return NCN_ERR_ALIGN;
-    const Plan p = make_plan(shape, activation);
+    const int path = kernel_path_for(shape, activation, alpha, m);
+    if (path == 0) return NCN_ERR_UNSUPPORTED;
+    const Plan p = make_plan(shape, path);
     hipStream_t s = static_cast<hipStream_t>(stream);
 
     // several stages: LDS-resident passes, last pass of the range first.  There is no scratch to ping-pong with: the
@@ -439,7 +467,7 @@ static int inverse_impl(const void* y, const void* ya, int in_dtype, void* x, vo
     // so the stages of such a pass are undone by one-stage launches (closed passes and one-stage launches may).
     std::vector<FusedPass> passes;
     if (grouping.plain() && (out_dtype == NCN_F32 || n_stages == 1))
-        passes = multi_stage_plan(shape, first_stage, n_stages, activation, false);
+        passes = multi_stage_plan(shape, first_stage, n_stages, activation, false, path);
     if (!passes.empty()) {
         const int64_t wstride = 2 * shape->E;
         const size_t np = passes.size();
@@ -508,8 +536,10 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
         !aligned16(x_rec) || !aligned16(xa_rec) || !aligned16(W) || !aligned16(dW) || !aligned16(workspace))
         return NCN_ERR_ALIGN;
     // partial rows of the generic kernel's second launch
-    const int extra_rows = (grouping.ctx_len && kernel_path(shape, activation) != 2) ? edge_rows(shape) : 0;
-    const Plan p = make_plan(shape, activation, extra_rows);
+    const int path = kernel_path_for(shape, activation, alpha, m);
+    if (path == 0) return NCN_ERR_UNSUPPORTED;
+    const int extra_rows = (grouping.ctx_len && path != 2) ? edge_rows(shape) : 0;
+    const Plan p = make_plan(shape, path, extra_rows);
     hipStream_t s = static_cast<hipStream_t>(stream);
     float* partials = static_cast<float*>(workspace);
     float* level1 = partials + (int64_t)kMaxGridX * 2 * shape->E;
@@ -518,7 +548,7 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
     // several stages: LDS-resident passes, last pass of the range first; the state ping-pongs between the
     // output arrays and four float32 arrays behind the dW scratch
     std::vector<FusedPass> passes;
-    if (grouping.plain()) passes = multi_stage_plan(shape, first_stage, n_stages, activation, true);
+    if (grouping.plain()) passes = multi_stage_plan(shape, first_stage, n_stages, activation, true, path);
     const size_t np = passes.size();
     bool fused_ok = np > 0;
     if (np >= 2 && workspace_bytes < base_workspace_bytes(shape) + temp_bytes(shape, true)) fused_ok = false;
@@ -667,10 +697,12 @@ int ncn_forward_radix(const void* x, const void* xa, int in_dtype, void* y, void
     if (!aligned16(x) || !aligned16(xa) || !aligned16(y) || !aligned16(ya) || !aligned16(W) || !aligned16(y32) ||
         !aligned16(ya32))
         return NCN_ERR_ALIGN;
-    const Plan p = make_plan(shape, activation);
+    const int path = kernel_path_for(shape, activation, alpha, m);
+    if (path == 0) return NCN_ERR_UNSUPPORTED;
+    const Plan p = make_plan(shape, path);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int64_t wstride = 2 * shape->E;
-    const std::vector<RadixPass> passes = plan_radix(shape, first_level, n_levels, false);
+    const std::vector<RadixPass> passes = plan_radix(shape, first_level, n_levels, false, path == 2);
     // every pass is closed: the first reads x, xa and the later ones run in place on y, ya; passes of several levels
     // keep their state in float32 LDS and convert on the way out
     for (size_t k = 0; k < passes.size(); ++k) {
@@ -717,12 +749,14 @@ int ncn_backward_radix(const void* y, const void* ya, int y_dtype, const void* d
     if (!aligned16(y) || !aligned16(ya) || !aligned16(dy) || !aligned16(dya) || !aligned16(dx) || !aligned16(dxa) ||
         !aligned16(x_rec) || !aligned16(xa_rec) || !aligned16(W) || !aligned16(dW) || !aligned16(workspace))
         return NCN_ERR_ALIGN;
-    const Plan p = make_plan(shape, activation);
+    const int path = kernel_path_for(shape, activation, alpha, m);
+    if (path == 0) return NCN_ERR_UNSUPPORTED;
+    const Plan p = make_plan(shape, path);
     hipStream_t s = static_cast<hipStream_t>(stream);
     float* partials = static_cast<float*>(workspace);
     float* level1 = partials + (int64_t)kMaxGridX * 2 * shape->E;
     const int64_t wstride = 2 * shape->E;
-    const std::vector<RadixPass> passes = plan_radix(shape, first_level, n_levels, true);
+    const std::vector<RadixPass> passes = plan_radix(shape, first_level, n_levels, true, path == 2);
     // last pass first; the first one to run reads y, ya, dy, dya, the others run in place on x_rec, xa_rec, dx, dxa
     DwReducer reducer(partials, level1, wstride, s);
     for (size_t e = 0; e < passes.size(); ++e) {
@@ -771,10 +805,12 @@ int ncn_inverse_radix(const void* y, const void* ya, int in_dtype, void* x, void
     if (!x || !xa || !y || !ya || !W) return NCN_ERR_NULL;
     if (!known_dtype(in_dtype) || !known_dtype(out_dtype)) return NCN_ERR_DTYPE;
     if (!aligned16(x) || !aligned16(xa) || !aligned16(y) || !aligned16(ya) || !aligned16(W)) return NCN_ERR_ALIGN;
-    const Plan p = make_plan(shape, activation);
+    const int path = kernel_path_for(shape, activation, alpha, m);
+    if (path == 0) return NCN_ERR_UNSUPPORTED;
+    const Plan p = make_plan(shape, path);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int64_t wstride = 2 * shape->E;
-    const std::vector<RadixPass> passes = plan_radix(shape, first_level, n_levels, false);
+    const std::vector<RadixPass> passes = plan_radix(shape, first_level, n_levels, false, path == 2);
     for (size_t e = 0; e < passes.size(); ++e) {   // last pass first; every pass is closed: in place after the first
         const RadixPass& ps = passes[passes.size() - 1 - e];
         const bool top = (e == 0);

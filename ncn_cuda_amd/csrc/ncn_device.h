@@ -8,21 +8,33 @@
 namespace ncn {
 
 // Scalars of the recurrence, made on the host in double precision and read by the kernels through scalar loads.
+//
+// The register kernels do not carry x and xa themselves but
+//     xs = kappa x,   as = kappa (1-m) xa          (forward)
+//     xs = kappa x,   bh = kappa (1-m)/m xa        (inverse and backward),
+// with kappa = 2 log2(e) alpha, and weights scaled by gamma = (1-alpha) / (2 log2(e) alpha^2).  Then
+//     z = 2 log2(e) T = xs_i + c_i xs_j,   c_i = <xs_i, gamma Wi> + <xs_j, gamma Wj>       (one FMA per element),
+//     forward:  as' = m as + k2 F,          xs' = m xs + as'                 (k2 = kappa (1-m)^2)
+//     inverse:  xs = xs'/m - bh',           bh = bh'/m - (k2/m^2) F
+// and with F = tanh T = 1 - 2r, r = 1/(1 + 2^z), the constant parts fold into the FMAs.
+// The backward carries its gradients divided by m^t after t inversion steps (G = g/m^t, P = p/m^t, p = (1-m) g + h),
+// which turns g <- m g + .. and p <- (1-m) g + m p into one FMA each; only dW needs the true scale, krho[t].
+// The scaling needs alpha and 1-m away from zero: the host sends other values to the generic kernels.
 struct StepTable {
     float alpha, m;
     int32_t activation;          // activation code (only read by kernels built for more than tanh)
     int32_t reserved;
+    float kappa, inv_kappa;      // 2 log2(e) alpha
+    float a_scale, inv_a_scale;  // kappa (1-m): xa -> as
+    float b_scale, inv_b_scale;  // kappa (1-m)/m: xa -> bh
+    float gamma;                 // (1-alpha) / (2 log2(e) alpha^2)
+    float om, im;                // 1-m, 1/m
+    float k2, m2k2;              // kappa (1-m)^2 and -2 k2
+    float bk0, bk1;              // -k2/m^2 and 2 k2/m^2
+    float ku;                    // 4 (1-m) alpha / m:  G += ku (U + rho Wi'),  U = P F'/4
     float m_pow_n, inv_m_pow_n;  // m^n_cache and its reciprocal
-    // Per-step scalars of the reversible backward / inverse, index t = number of inversion steps already done
-    // (t = 0 is the stage's last step):
-    //   im = m^-(t+1),  lam = 2 log2(e) alpha im,  kc2 = 2 log2(e) (1-alpha) im^2,
-    //   kap = (1-m) m^t,  krho = 4 (1-m)/m (1-alpha) im
-    // and of the forward, index t = number of steps already done:
-    //   flam = 2 log2(e) alpha m^t,  fkc = 2 log2(e) (1-alpha) m^2t,  fkap = (1-m) / m^(t+1)
-    struct StepScalars {
-        float lam, kc2, kap, krho;
-        float flam, fkc, fkap;
-    } step[64];
+    float reserved2;
+    float krho[64];              // (1-alpha) 4 (1-m) m^t / kappa^2: dW scale after t inversion steps
 };
 
 // Everything one stage launch needs.  Which pointer means what depends on the kernel:
@@ -176,6 +188,22 @@ __device__ __forceinline__ float lane_sum(float v) {
         return lane_sum<LO * 2, HI, ROWS, FROM1>(v);
     } else {
         return v;
+    }
+}
+
+// The same sums for N values at once, level by level over all of them: the N chains are independent, so their trips
+// across the lanes overlap (one wait per level instead of one per value and level).
+template <int LO, int HI, bool ROWS, int N, bool FROM1 = (LO == 1)>
+__device__ __forceinline__ void lane_sum_n(float (&v)[N]) {
+    if constexpr (LO < HI) {
+#pragma unroll
+        for (int k = 0; k < N; ++k) {
+            if constexpr (LO == 4 && FROM1 && ROWS)
+                v[k] += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v[k]), 0x141, 0xF, 0xF, true));
+            else
+                v[k] += lane_xor<LO, ROWS>(v[k]);
+        }
+        lane_sum_n<LO * 2, HI, ROWS, N, FROM1>(v);
     }
 }
 

@@ -20,9 +20,10 @@
 //
 // How.  Per stage each wave gathers R x F register tiles of whole groups from LDS (the tile shapes and the step
 // code are those of the one-stage kernels, ncn_stage_kernels.h), runs the n_cache steps and scatters the tile
-// back; one workgroup barrier separates stages.  The rows stay in the m-power-scaled form of the step code for the
-// whole pass (the step counter just keeps counting across stages; backward keeps p = (1-m) g + h in place of h),
-// so true values exist only in HBM.  The pass's weights sit in LDS.  Backward sums each wave's dW share of a stage into a per-wave LDS
+// back; one workgroup barrier separates stages.  The rows stay in the scaled form of the step code for the whole pass
+// (xs and as or bh, see StepTable; backward keeps G = g / m^t and P = p / m^t with the step counter counting across
+// the stages, p = (1-m) g + h in place of h), so true values exist only in HBM.  The pass's weights sit in LDS,
+// already scaled by gamma.  Backward sums each wave's dW share of a stage into a per-wave LDS
 // slot (one writer per slot, fixed order: deterministic) and leaves one partial row per workgroup and stage.
 //
 // RADIX builds of the same kernels run levels of the radix-n digit grouping (ncn_triton/group_tensors.py:8-18)
@@ -69,7 +70,7 @@ struct FusedArgs {
     uint32_t class_groups;    // closed: S0 / (window / ring) windows per batch entry; halo: S0
     uint32_t total_items;     // batch * class_groups * tiles_per_ring * n_head
     uint32_t sub_stride[kFusedMaxStages];  // s_l / S0 per stage of the pass
-    float scale_dn, scale_up;              // m^(n_cache * n_stages) and its reciprocal
+    float scale_dn, scale_up;              // m^(n_cache * n_stages) and its reciprocal (backward: gradients leave as G m^T)
     StepTable tab;
 };
 
@@ -204,7 +205,7 @@ __device__ __forceinline__ void fused_raw_to_float(const uint4& r, int dtype, fl
 }
 
 template <int EC, int NW, int K>
-__device__ __forceinline__ void fused_commit_rows(const uint4 (&raw)[K], int dtype, float* dst, uint32_t rows) {
+__device__ __forceinline__ void fused_commit_rows(const uint4 (&raw)[K], int dtype, float* dst, uint32_t rows, float scale) {
     constexpr uint32_t CPR = EC / 4;
 #pragma unroll
     for (int k = 0; k < K; ++k) {
@@ -212,6 +213,8 @@ __device__ __forceinline__ void fused_commit_rows(const uint4 (&raw)[K], int dty
         if (c < rows * CPR) {
             float v[4];
             fused_raw_to_float(raw[k], dtype, v);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] *= scale;
             lds_store_frag<4>(dst + c * 4, v);   // c * 4 == lr * EC + c4 * 4
         }
     }
@@ -235,12 +238,12 @@ __device__ __forceinline__ void fused_store_rows_scaled(const FusedArgs& A, cons
     }
 }
 
-// the pass's weights, [stage][Wi | Wj][EC] of this workgroup's head, into LDS
+// the pass's weights times gamma, [stage][Wi | Wj][EC] of this workgroup's head, into LDS
 template <int EC, int NW>
 __device__ __forceinline__ void fused_load_weights(const FusedArgs& A, int head, float* w_lds) {
     for (int k = threadIdx.x; k < A.n_stages * 2 * EC; k += 64 * NW) {
         const int st = k / (2 * EC), rem = k - st * 2 * EC, half = rem / EC, f = rem - half * EC;
-        w_lds[k] = A.W[(int64_t)st * 2 * A.E + (int64_t)half * A.E + (int64_t)head * EC + f];
+        w_lds[k] = A.tab.gamma * A.W[(int64_t)st * 2 * A.E + (int64_t)half * A.E + (int64_t)head * EC + f];
     }
 }
 
@@ -272,8 +275,8 @@ __global__ void __launch_bounds__(64 * kFusedWavesFwd) fused_forward_kernel(cons
     }
     for (uint32_t item = blockIdx.x; item < A.total_items; item += gridDim.x) {
         const FusedItem it = fused_item<NC, EC, RADIX>(A, item);
-        fused_commit_rows<EC, NW, K>(rx, A.in_dtype, xs, rows);
-        fused_commit_rows<EC, NW, K>(ra, A.in_dtype, as, rows);
+        fused_commit_rows<EC, NW, K>(rx, A.in_dtype, xs, rows, A.tab.kappa);
+        fused_commit_rows<EC, NW, K>(ra, A.in_dtype, as, rows, INVERSE ? A.tab.b_scale : A.tab.a_scale);
         __syncthreads();
         if (item + gridDim.x < A.total_items) {   // the next window travels while this one is computed
             int64_t off[K];
@@ -299,8 +302,8 @@ __global__ void __launch_bounds__(64 * kFusedWavesFwd) fused_forward_kernel(cons
                     lds_load_frag<F>(xs + row[rr], x[rr]);
                     lds_load_frag<F>(as + row[rr], a[rr]);
                 }
-                if (INVERSE) inverse_core<NC, EC, R, F, TANH_ONLY, false, true>(x, a, wi, wj, A.tab, sq * NC, lane, slots);
-                else forward_core<NC, EC, R, F, TANH_ONLY, false, true>(x, a, wi, wj, A.tab, sq * NC, lane, slots);
+                if (INVERSE) inverse_core<NC, EC, R, F, TANH_ONLY, false, true>(x, a, wi, wj, A.tab, lane, slots);
+                else forward_core<NC, EC, R, F, TANH_ONLY, false, true>(x, a, wi, wj, A.tab, lane, slots);
                 if (valid) {
 #pragma unroll
                     for (int rr = 0; rr < R; ++rr) {
@@ -311,9 +314,10 @@ __global__ void __launch_bounds__(64 * kFusedWavesFwd) fused_forward_kernel(cons
             }
             __syncthreads();
         }
-        const float back = INVERSE ? A.scale_up : A.scale_dn;   // out of the m-power-scaled form
-        fused_store_rows_scaled<NC, EC, NW, RADIX>(A, it, xs, back, A.out0, A.out_dtype, A.aux0);
-        fused_store_rows_scaled<NC, EC, NW, RADIX>(A, it, as, back, A.out1, A.out_dtype, A.aux1);
+        // out of the scaled form
+        fused_store_rows_scaled<NC, EC, NW, RADIX>(A, it, xs, A.tab.inv_kappa, A.out0, A.out_dtype, A.aux0);
+        fused_store_rows_scaled<NC, EC, NW, RADIX>(A, it, as, INVERSE ? A.tab.inv_b_scale : A.tab.inv_a_scale, A.out1,
+                                                   A.out_dtype, A.aux1);
         __syncthreads();
     }
 }
@@ -358,9 +362,9 @@ __global__ void __launch_bounds__(64 * kFusedWavesBwd, TANH_ONLY ? 4 : 1) fused_
         fused_fetch_rows<K>(A.g1, A.g_dtype, off, r.h);
     };
     auto commit = [&](const Raw& r) {
-        fused_commit_rows<EC, NW, K>(r.y, A.in_dtype, ys, rows);
-        fused_commit_rows<EC, NW, K>(r.b, A.in_dtype, bs, rows);
-        fused_commit_rows<EC, NW, K>(r.g, A.g_dtype, gs, rows);
+        fused_commit_rows<EC, NW, K>(r.y, A.in_dtype, ys, rows, A.tab.kappa);
+        fused_commit_rows<EC, NW, K>(r.b, A.in_dtype, bs, rows, A.tab.b_scale);
+        fused_commit_rows<EC, NW, K>(r.g, A.g_dtype, gs, rows, 1.0f);
         constexpr uint32_t CPR = EC / 4;   // p = (1-m) g + h  (h = 0 when dya is null: the fetch left zeros)
 #pragma unroll
         for (int k = 0; k < K; ++k) {
@@ -438,7 +442,7 @@ __global__ void __launch_bounds__(64 * kFusedWavesBwd, TANH_ONLY ? 4 : 1) fused_
             }
             __syncthreads();
         }
-        auto write_out = [&]() {   // owned rows back to true values: g = G m^T, h = P m^T - (1-m) g, x = Y / m^T, xa = B / m^T
+        auto write_out = [&]() {   // owned rows back to true values: g = G m^T, h = P m^T - (1-m) g, x = xs / kappa, xa = bh / b_scale
             constexpr uint32_t CPR = EC / 4;
             const uint32_t r0 = it.own_lo * NC, nrows = it.own_cnt * NC;
             for (uint32_t c = threadIdx.x; c < nrows * CPR; c += 64 * NW) {
@@ -456,8 +460,8 @@ __global__ void __launch_bounds__(64 * kFusedWavesBwd, TANH_ONLY ? 4 : 1) fused_
                 store_frag<4>(A.out1, A.out_dtype, off, true, h);
             }
             if (A.aux0) {
-                fused_store_rows_scaled<NC, EC, NW, RADIX>(A, it, ys, A.scale_up, A.aux0, NCN_F32, nullptr);
-                fused_store_rows_scaled<NC, EC, NW, RADIX>(A, it, bs, A.scale_up, A.aux1, NCN_F32, nullptr);
+                fused_store_rows_scaled<NC, EC, NW, RADIX>(A, it, ys, A.tab.inv_kappa, A.aux0, NCN_F32, nullptr);
+                fused_store_rows_scaled<NC, EC, NW, RADIX>(A, it, bs, A.tab.inv_b_scale, A.aux1, NCN_F32, nullptr);
             }
         };
         if (item + gridDim.x < A.total_items) {   // the same for the whole workgroup

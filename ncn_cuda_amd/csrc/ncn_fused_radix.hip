@@ -81,7 +81,7 @@ bool radix_fused_supported(const ncn_shape* sh) {
 
 // Levels [first, first + count) cut into passes of as many levels as fit the LDS budget (and the stage limits of the
 // kernels); a pass of one level is left to the one-stage kernel.  Every pass is closed.
-std::vector<RadixPass> plan_radix(const ncn_shape* sh, int first, int count, bool backward) {
+std::vector<RadixPass> plan_radix(const ncn_shape* sh, int first, int count, bool backward, bool fused) {
     std::vector<RadixPass> passes;
     const int nc = sh->n_cache, ec = (int)(sh->E / sh->n_head);
     const uint32_t cap_rows = floor_pow2((uint32_t)(kFusedStateBytes / ((backward ? 4 : 2) * ec * sizeof(float))));
@@ -93,15 +93,19 @@ std::vector<RadixPass> plan_radix(const ncn_shape* sh, int first, int count, boo
         RadixPass p{};
         p.first = a;
         p.count = (count - a < kmax) ? count - a : kmax;
-        p.single = (p.count < 2 || !radix_fused_supported(sh)) ? 1 : 0;
+        p.single = (p.count < 2 || !fused || !radix_fused_supported(sh)) ? 1 : 0;
         if (p.single) p.count = 1;
         p.s0 = (uint32_t)ipow(nc, first + a);
         p.span = (uint32_t)ipow(nc, p.count);
-        uint32_t rows = cap_rows;
+        // A workgroup holds a whole number of windows, and every workgroup-load of a batch entry holds the same
+        // number: the largest divisor of the window count that the LDS budget takes (N = odd * n^k leaves an odd
+        // factor in the window count; a count that does not divide would leave the last windows unprocessed).
         const uint32_t windows = (uint32_t)(sh->N / p.span);   // per batch entry and head
-        if (rows > windows * p.span) rows = windows * p.span;  // N smaller than the LDS budget
-        p.rows = rows;
-        p.loads = windows / (rows / p.span);
+        uint32_t per_load = cap_rows / p.span;
+        if (per_load > windows) per_load = windows;            // N smaller than the LDS budget
+        while (windows % per_load) --per_load;
+        p.rows = per_load * p.span;
+        p.loads = windows / per_load;
         passes.push_back(p);
         a += p.count;
     }

@@ -96,7 +96,8 @@ struct RadixPass {
     uint32_t loads;    // workgroup-loads per batch entry and head
 };
 bool radix_fused_supported(const ncn_shape* sh);
-std::vector<RadixPass> plan_radix(const ncn_shape* sh, int first, int count, bool backward);
+// fused = false: one level per pass whatever the shape (calls whose scalars only the generic kernels take)
+std::vector<RadixPass> plan_radix(const ncn_shape* sh, int first, int count, bool backward, bool fused = true);
 int radix_grid(const ncn_shape* sh, const RadixPass& p, bool backward);
 hipError_t launch_fused_radix(Pass pass, FusedArgs& a, const ncn_shape* sh, const RadixPass& p, hipStream_t s);
 

@@ -31,7 +31,6 @@ namespace ncn {
 
 constexpr int kWavesPerBlock = 4;
 constexpr int kBlockThreads = 64 * kWavesPerBlock;
-constexpr float kTwoLog2e = 2.8853900817779268f;  // exp(2T) = exp2(kTwoLog2e * T)
 
 template <int NC, int EC, int R, int F>
 struct Tile {
@@ -84,11 +83,10 @@ __device__ __forceinline__ void load_w(const float* W, int64_t E, int head, int 
 // Activation from z = 2 log2(e) T (the form the step code produces): F(T) and w = F'(T) / 4.
 //   tanh:    r = 1/(1 + 2^z), F = 1 - 2r, F'/4 = r - r^2                (ncn_fwd_cuda_kernel.cu:86-87)
 //   relu, sigmoid, linear: codes of ncn_fwd_cuda_kernel.cu:88-95 / ncn_bwd_cuda_kernel.cu:137-150
-// TANH_ONLY kernels have no branch; the others pick the activation with a wave-uniform branch on `code`.
+// TANH_ONLY kernels never come here: their step code works on r itself.
 constexpr float kHalfLn2 = 0.34657359027997264f;  // T = z * ln(2)/2
-template <bool TANH_ONLY>
 __device__ __forceinline__ void act_Fw(float z, int code, float& Fv, float& w) {
-    if (TANH_ONLY || code == NCN_ACT_TANH) {
+    if (code == NCN_ACT_TANH) {
         const float r = __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(z) + 1.0f);
         Fv = fmaf(-2.0f, r, 1.0f);
         w = fmaf(-r, r, r);
@@ -109,160 +107,110 @@ __device__ __forceinline__ void act_Fw(float z, int code, float& Fv, float& w) {
     }
 }
 
-template <int F>
-__device__ __forceinline__ float dot_frag(const float (&a)[F], const float (&b)[F]) {
-    float s0 = 0.f, s1 = 0.f;
+// The row sums c_i = <xs_i, Wi'> + <xs_j, Wj'> of a lane's R rows: a chain of FMAs per row that starts from the lane's
+// share e of <xs_j, Wj'>, then all R sums cross the LF lanes of a row together.
+template <int LF, int R, int F, bool ROWS>
+__device__ __forceinline__ void row_sums(const float (&x)[R][F], const float (&wi)[F], float e, float (&c)[R]) {
 #pragma unroll
-    for (int f = 0; f < F; f += 2) {
-        s0 = fmaf(a[f], b[f], s0);
-        if (f + 1 < F) s1 = fmaf(a[f + 1], b[f + 1], s1);
+    for (int rr = 0; rr < R; ++rr) {
+        c[rr] = e;
+#pragma unroll
+        for (int f = 0; f < F; ++f) c[rr] = fmaf(x[rr][f], wi[f], c[rr]);
     }
-    return s0 + s1;
+    lane_sum_n<1, LF, ROWS, R>(c);
+}
+
+template <int F>
+__device__ __forceinline__ float dot_chain(const float (&a)[F], const float (&b)[F]) {
+    float s = 0.f;
+#pragma unroll
+    for (int f = 0; f < F; ++f) s = fmaf(a[f], b[f], s);
+    return s;
 }
 
 // ---------------------------------------------------------------------------------------------
 // forward (torch_ref/ncn_pytorch.py:74-94), all n_cache steps on one register tile
 //   s_i = <x_i,Wi> + <x_j,Wj>      T = alpha x_i + (1-alpha) s_i x_j      F = tanh T = 1 - 2r,
 //   r = 1/(1 + exp(2T))            a' = m a + (1-m) F                     x' = m x + (1-m) a'
-// The registers hold X = x / m^t and A = xa / m^t after t steps, which turns the two updates into
-//   A <- A + (1-m)/m^(t+1) F   and   X <- X + (1-m) A   (the powers of m come from a host-made table).
-// ---------------------------------------------------------------------------------------------
-// forward_core runs the n_cache steps of one stage on registers that already hold x / m^t0, xa / m^t0 with
-// t0 = step_base steps done before (several stages in a row just keep counting) and leaves them scaled.
+// on the scaled state of StepTable: x holds xs, a holds as, wi / wj hold gamma Wi / gamma Wj.  Per element and step:
+// one FMA for the row sum, one for z, exp2, +1, rcp, two FMAs for as', one for xs'.
 // STEP_MASK builds take `live`, the live rows of the lane's group, and skip steps j >= live with the lanes of that
 // group switched off (a group that a context length cuts runs one step per live row,
 // ncn_triton/ncn_triton_old.py:93-96).  Every cross-lane exchange of a step stays inside one group.
+// ---------------------------------------------------------------------------------------------
 template <int NC, int EC, int R, int F, bool TANH_ONLY = true, bool STEP_MASK = false, bool ROWS = false>
 __device__ __forceinline__ void forward_core(float (&x)[R][F], float (&a)[R][F], const float (&wi)[F],
-                                             const float (&wj)[F], const StepTable& S, int step_base, int lane,
-                                             float4* slots, int live = NC) {
+                                             const float (&wj)[F], const StepTable& S, int lane, float4* slots,
+                                             int live = NC) {
     using T = Tile<NC, EC, R, F>;
-    const float om = 1.0f - S.m;
 #pragma unroll 1
     for (int jo = 0; jo < T::LR; ++jo) {
 #pragma unroll
         for (int jr = 0; jr < R; ++jr) {
             if (STEP_MASK && jo * R + jr >= live) continue;  // the lanes of a group agree: no lane it needs is off
-            const int ts = step_base + jo * R + jr;   // steps done so far
-            const float lam = S.step[ts].flam;     // z = lam X_i + c_i Xj
-            const float kc = S.step[ts].fkc;       // c_i = kc S_i
-            const float kap = S.step[ts].fkap;     // A <- A + kap F
-            float xj[F];
+            float xj[F], c[R];
             row_lane_broadcast<T::LF, T::LR, F>(x[jr], xj, jo, lane, slots);
-            const float e = dot_frag<F>(xj, wj);
-            // pivot row last: its registers are the source of xj when LR == 1
+            row_sums<T::LF, R, F, ROWS>(x, wi, dot_chain<F>(xj, wj), c);
 #pragma unroll
-            for (int k = 1; k <= R; ++k) {
-                const int rr = (jr + k) % R;
-                const float s = lane_sum<1, T::LF, ROWS>(dot_frag<F>(x[rr], wi) + e);
-                const float c = kc * s;
+            for (int rr = 0; rr < R; ++rr) {
 #pragma unroll
                 for (int f = 0; f < F; ++f) {
-                    const float z = fmaf(c, xj[f], lam * x[rr][f]);
-                    float Fv, w;
-                    act_Fw<TANH_ONLY>(z, S.activation, Fv, w);
-                    a[rr][f] = fmaf(kap, Fv, a[rr][f]);
-                    x[rr][f] = fmaf(om, a[rr][f], x[rr][f]);
+                    const float z = fmaf(c[rr], xj[f], x[rr][f]);
+                    if constexpr (TANH_ONLY) {
+                        const float r = __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(z) + 1.0f);
+                        a[rr][f] = fmaf(S.m2k2, r, fmaf(S.m, a[rr][f], S.k2));
+                    } else {
+                        float Fv, w;
+                        act_Fw(z, S.activation, Fv, w);
+                        a[rr][f] = fmaf(S.k2, Fv, S.m * a[rr][f]);
+                    }
+                    x[rr][f] = fmaf(S.m, x[rr][f], a[rr][f]);
                 }
             }
         }
     }
-}
-
-// one stage from true values to true values
-// m^k by repeated multiplication (k <= 64; only groups cut by a context length come here)
-__device__ __forceinline__ float pow_steps(float base, int k) {
-    float p = 1.0f;
-    for (int i = 0; i < k; ++i) p *= base;
-    return p;
-}
-
-template <int NC, int EC, int R, int F, bool TANH_ONLY, bool STEP_MASK = false>
-__device__ __forceinline__ void forward_steps(float (&x)[R][F], float (&a)[R][F], const float (&wi)[F],
-                                              const float (&wj)[F], const StepTable& S, int lane, float4* slots,
-                                              int live = NC) {
-    forward_core<NC, EC, R, F, TANH_ONLY, STEP_MASK>(x, a, wi, wj, S, 0, lane, slots, live);
-    // `live` steps were done: the registers hold x / m^live
-    const float dn = (!STEP_MASK || live == NC) ? S.m_pow_n : pow_steps(S.m, live);
-#pragma unroll
-    for (int rr = 0; rr < R; ++rr)
-#pragma unroll
-        for (int f = 0; f < F; ++f) {
-            x[rr][f] *= dn;
-            a[rr][f] *= dn;
-        }
 }
 
 // ---------------------------------------------------------------------------------------------
 // inverse (torch_ref/ncn_pytorch_invertible.py:87-113), steps j = n_cache-1 .. 0
 //   x = (y - (1-m) b)/m       recompute r from x        a = (b - (1-m) F)/m
-// with the same m^t scaling of the registers as the backward below (Y = m^t x, B = m^t xa).
+// on the scaled state: y holds xs, b holds bh (see StepTable).
+// STEP_MASK: a group with `live` < NC live rows only undoes its steps live-1 .. 0.
 // ---------------------------------------------------------------------------------------------
-// STEP_MASK: a group with `live` < NC live rows only undoes its steps live-1 .. 0.  The skipped steps come first in
-// the loop, so the registers are first scaled as if they had been done (m^(NC-live)): every later step then
-// finds the scaling its table entry assumes, and the final factor is the same for all groups.
-// inverse_core: the n_cache steps of one stage on registers that hold m^t0 x, m^t0 xa with t0 = step_base inversion
-// steps done before; leaves them scaled by t0 + n_cache steps (several stages in a row just keep counting).
 template <int NC, int EC, int R, int F, bool TANH_ONLY, bool STEP_MASK = false, bool ROWS = false>
 __device__ __forceinline__ void inverse_core(float (&y)[R][F], float (&b)[R][F], const float (&wi)[F],
-                                             const float (&wj)[F], const StepTable& S, int step_base, int lane,
-                                             float4* slots, int live = NC) {
+                                             const float (&wj)[F], const StepTable& S, int lane, float4* slots,
+                                             int live = NC) {
     using T = Tile<NC, EC, R, F>;
-    const float nom = S.m - 1.0f;
 #pragma unroll 1
     for (int jo = T::LR - 1; jo >= 0; --jo) {
 #pragma unroll
         for (int jr = R - 1; jr >= 0; --jr) {
             if (STEP_MASK && jo * R + jr >= live) continue;
-            const int ts = step_base + (T::LR - 1 - jo) * R + (R - 1 - jr);   // inversion steps done so far
-            const float lam = S.step[ts].lam, kc2 = S.step[ts].kc2, kap = S.step[ts].kap;
 #pragma unroll
             for (int rr = 0; rr < R; ++rr)
 #pragma unroll
-                for (int f = 0; f < F; ++f) y[rr][f] = fmaf(nom, b[rr][f], y[rr][f]);
-            float xj[F];
+                for (int f = 0; f < F; ++f) y[rr][f] = fmaf(S.im, y[rr][f], -b[rr][f]);
+            float xj[F], c[R];
             row_lane_broadcast<T::LF, T::LR, F>(y[jr], xj, jo, lane, slots);
-            const float e = dot_frag<F>(xj, wj);
+            row_sums<T::LF, R, F, ROWS>(y, wi, dot_chain<F>(xj, wj), c);
 #pragma unroll
             for (int rr = 0; rr < R; ++rr) {
-                const float s = lane_sum<1, T::LF, ROWS>(dot_frag<F>(y[rr], wi) + e);
-                const float c = kc2 * s;
 #pragma unroll
                 for (int f = 0; f < F; ++f) {
-                    const float z = fmaf(c, xj[f], lam * y[rr][f]);
-                    float Fv, w;
-                    act_Fw<TANH_ONLY>(z, S.activation, Fv, w);
-                    b[rr][f] = fmaf(-kap, Fv, b[rr][f]);
+                    const float z = fmaf(c[rr], xj[f], y[rr][f]);
+                    if constexpr (TANH_ONLY) {
+                        const float r = __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(z) + 1.0f);
+                        b[rr][f] = fmaf(S.bk1, r, fmaf(S.im, b[rr][f], S.bk0));
+                    } else {
+                        float Fv, w;
+                        act_Fw(z, S.activation, Fv, w);
+                        b[rr][f] = fmaf(S.bk0, Fv, S.im * b[rr][f]);
+                    }
                 }
             }
         }
     }
-}
-
-// one stage from true values to true values
-template <int NC, int EC, int R, int F, bool TANH_ONLY, bool STEP_MASK = false>
-__device__ __forceinline__ void inverse_steps(float (&y)[R][F], float (&b)[R][F], const float (&wi)[F],
-                                              const float (&wj)[F], const StepTable& S, int lane, float4* slots,
-                                              int live = NC) {
-    if (STEP_MASK && live != NC) {
-        const float sc = pow_steps(S.m, NC - live);
-#pragma unroll
-        for (int rr = 0; rr < R; ++rr)
-#pragma unroll
-            for (int f = 0; f < F; ++f) {
-                y[rr][f] *= sc;
-                b[rr][f] *= sc;
-            }
-    }
-    inverse_core<NC, EC, R, F, TANH_ONLY, STEP_MASK>(y, b, wi, wj, S, 0, lane, slots, live);
-    const float up = S.inv_m_pow_n;
-#pragma unroll
-    for (int rr = 0; rr < R; ++rr)
-#pragma unroll
-        for (int f = 0; f < F; ++f) {
-            y[rr][f] *= up;
-            b[rr][f] *= up;
-        }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -274,20 +222,23 @@ __device__ __forceinline__ void inverse_steps(float (&y)[R][F], float (&b)[R][F]
 //   g_i <- m g_i + a u_i + (1-a) r_i Wi   [+ sum_k ((1-a) r_k Wj + (1-a) s_k u_k) on the pivot row j]
 //   p_i <- (1-m) g_i(new) + m p_i          (equivalent to h_i <- m (1-m) g_i + m h_i)
 //
-// The divisions by m of the inversion and the multiplications by m of the gradient recurrences are
-// folded into per-step scalars: after t inversion steps the registers hold
-//   Y = m^t x,   B = m^t xa,   G = g / m^t,   P = p / m^t,
-// which turns  x <- (y - (1-m) b)/m  into  Y <- Y - (1-m) B,   g <- m g + ..  into  G <- G + ../m^(t+1)
-// and  p <- (1-m) g + m p  into  P <- P + (1-m) G  (one FMA each).
+// Registers: Y = xs, B = bh (scaled state, see StepTable), G = g / m^t, P = p / m^t after t inversion steps, which
+// turns  g <- m g + ..  into  G <- G + ../m^(t+1)  and  p <- (1-m) g + m p  into  P <- P + (1-m) G  (one FMA each).
+// With U = P F'/4 (so u = 4 (1-m) m^t U) and rh_i = <U_i, xs_j> every factor that is not a power of m is the one
+// constant ku = 4 (1-m) alpha / m:
+//   G_i += ku (U_i + rh_i Wi')           pivot row: G_j += ku sum_rows( (sum_i rh_i) Wj' + sum_i c_i U_i )
+// and only dW needs the true scale: dWi += krho[t] rh_i xs_i, dWj += krho[t] (sum_i rh_i) xs_j.
 //
-// On entry Y, B = stage outputs, G, H = their gradients; on exit G, H = gradients of the stage inputs and
-// Y, B = m^n_cache times the stage inputs (multiply by StepTable::inv_m_pow_n before storing them).
+// A step runs in phases over the lane's R rows, so that the cross-lane sums of the rows travel together:
+// invert xs; row sums c; [per element: z, r, bh, U, partial rh, v += c U, G += ku U]; sums rh; [G += ku rh Wi', dWi, P];
+// pivot row.  U is only needed inside the third phase.
+//
+// On entry Y, B = scaled stage outputs, G = g / m^t0, P = p / m^t0 with t0 = step_base inversion steps done before
+// (several stages in a row keep counting); on exit all four describe the stage inputs, t0 + n_cache steps done.
 // dwi, dwj accumulate this lane's share of dWi, dWj; with MASKED the share is weighted by `own` (1, or 0 for a
 // group whose dW another tile accounts for).
+// STEP_MASK: steps j >= live leave the registers as they are (the caller scales G, P as if they had been done).
 // ---------------------------------------------------------------------------------------------
-// backward_core: the n_cache steps of one stage on registers in the scaled form above with t0 = step_base
-// inversion steps done before (P holds p / m^t0, not h); leaves them scaled by t0 + n_cache steps.
-// STEP_MASK: steps j >= live leave the registers as they are (see inverse_steps for the scaling).
 template <int NC, int EC, int R, int F, bool MASKED, bool TANH_ONLY = true, bool STEP_MASK = false, bool ROWS = false>
 __device__ __forceinline__ void backward_core(float (&Y)[R][F], float (&B)[R][F], float (&G)[R][F], float (&P)[R][F],
                                               const float (&wi)[F], const float (&wj)[F], float (&dwi)[F],
@@ -295,106 +246,126 @@ __device__ __forceinline__ void backward_core(float (&Y)[R][F], float (&B)[R][F]
                                               float4* slots, int live = NC) {
     using T = Tile<NC, EC, R, F>;
     const int rl = (lane / T::LF) % T::LR;
-    const float om = 1.0f - S.m;
-    const float ku = 4.0f * om / S.m * S.alpha;  // G += ku * U        (U = P (r - r^2))
-    const float nom = -om;
 #pragma unroll 1
     for (int jo = T::LR - 1; jo >= 0; --jo) {
-        const float sel = (T::LR == 1 || rl == jo) ? 1.0f : 0.0f;  // this lane holds the pivot row
+        const float selku = (T::LR == 1 || rl == jo) ? S.ku : 0.0f;  // this lane holds the pivot row
 #pragma unroll
         for (int jr = R - 1; jr >= 0; --jr) {
             if (STEP_MASK && jo * R + jr >= live) continue;  // lanes of a group agree: no lane it needs is off
             const int ts = step_base + (T::LR - 1 - jo) * R + (R - 1 - jr);   // inversion steps done so far
-            const float lam = S.step[ts].lam;     // z = lam Y_i + chat_i Yj
-            const float kc2 = S.step[ts].kc2;     // chat_i = kc2 S_i
-            const float kap = S.step[ts].kap;     // B <- B - kap F
-            const float krho = S.step[ts].krho;   // rho_i = krho <U_i, Yj>
+            const float krho = MASKED ? S.krho[ts] * own : S.krho[ts];
 #pragma unroll
             for (int rr = 0; rr < R; ++rr)
 #pragma unroll
-                for (int f = 0; f < F; ++f) Y[rr][f] = fmaf(nom, B[rr][f], Y[rr][f]);  // m^(t+1) x of this step
-            float xj[F], v[F];
+                for (int f = 0; f < F; ++f) Y[rr][f] = fmaf(S.im, Y[rr][f], -B[rr][f]);  // xs before this step
+            float xj[F], v[F], c[R], rh[R];
             row_lane_broadcast<T::LF, T::LR, F>(Y[jr], xj, jo, lane, slots);
+            row_sums<T::LF, R, F, ROWS>(Y, wi, dot_chain<F>(xj, wj), c);
 #pragma unroll
             for (int f = 0; f < F; ++f) v[f] = 0.f;
-            const float e = dot_frag<F>(xj, wj);
+#pragma unroll
+            for (int rr = 0; rr < R; ++rr) {
+                rh[rr] = 0.f;
+#pragma unroll
+                for (int f = 0; f < F; ++f) {
+                    const float z = fmaf(c[rr], xj[f], Y[rr][f]);
+                    float w;
+                    if constexpr (TANH_ONLY) {
+                        const float r = __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(z) + 1.0f);
+                        B[rr][f] = fmaf(S.bk1, r, fmaf(S.im, B[rr][f], S.bk0));   // bh before this step
+                        w = fmaf(-r, r, r);
+                    } else {
+                        float Fv;
+                        act_Fw(z, S.activation, Fv, w);
+                        B[rr][f] = fmaf(S.bk0, Fv, S.im * B[rr][f]);
+                    }
+                    const float U = P[rr][f] * w;
+                    rh[rr] = fmaf(U, xj[f], rh[rr]);
+                    v[f] = fmaf(c[rr], U, v[f]);
+                    G[rr][f] = fmaf(S.ku, U, G[rr][f]);
+                }
+            }
+            lane_sum_n<1, T::LF, ROWS, R>(rh);
             float rhosum = 0.f;
 #pragma unroll
             for (int rr = 0; rr < R; ++rr) {
-                const float Ssum = lane_sum<1, T::LF, ROWS>(dot_frag<F>(Y[rr], wi) + e);
-                const float chat = kc2 * Ssum;
-                float u[F];
-                float rh = 0.f;
-#pragma unroll
-                for (int f = 0; f < F; ++f) {
-                    const float z = fmaf(chat, xj[f], lam * Y[rr][f]);
-                    float Fv, w;
-                    act_Fw<TANH_ONLY>(z, S.activation, Fv, w);
-                    B[rr][f] = fmaf(-kap, Fv, B[rr][f]);   // m^(t+1) xa of this step
-                    u[f] = P[rr][f] * w;
-                    rh = fmaf(u[f], xj[f], rh);
-                }
-                rh = lane_sum<1, T::LF, ROWS>(rh);
-                const float rho = krho * rh;       // (1-alpha) r_i / m^(t+1)
-                const float c4 = krho * Ssum;      // (1-alpha) s_i u-scale / m^(t+1)
-                const float rho_w = MASKED ? rho * own : rho;
-                rhosum += rho;
+                const float rho_w = krho * rh[rr];     // (1-alpha) r_i / kappa, weighted
+                const float kr = S.ku * rh[rr];
+                rhosum += rh[rr];
 #pragma unroll
                 for (int f = 0; f < F; ++f) {
                     dwi[f] = fmaf(rho_w, Y[rr][f], dwi[f]);
-                    v[f] = fmaf(c4, u[f], v[f]);
-                    G[rr][f] = fmaf(rho, wi[f], fmaf(ku, u[f], G[rr][f]));
-                    if (rr != jr) P[rr][f] = fmaf(om, G[rr][f], P[rr][f]);
+                    G[rr][f] = fmaf(kr, wi[f], G[rr][f]);
+                    if (rr != jr) P[rr][f] = fmaf(S.om, G[rr][f], P[rr][f]);
                 }
             }
-            const float rhosum_w = MASKED ? rhosum * own : rhosum;
+            const float rhosum_w = krho * rhosum;
+            float t[F];
 #pragma unroll
             for (int f = 0; f < F; ++f) {
                 dwj[f] = fmaf(rhosum_w, xj[f], dwj[f]);
-                const float vt = lane_sum<T::LF, T::LPG, ROWS>(fmaf(rhosum, wj[f], v[f]));  // over the group's row lanes
-                G[jr][f] = fmaf(sel, vt, G[jr][f]);
-                P[jr][f] = fmaf(om, G[jr][f], P[jr][f]);
+                t[f] = fmaf(rhosum, wj[f], v[f]);
+            }
+            lane_sum_n<T::LF, T::LPG, ROWS, F>(t);   // over the group's row lanes
+#pragma unroll
+            for (int f = 0; f < F; ++f) {
+                G[jr][f] = fmaf(selku, t[f], G[jr][f]);
+                P[jr][f] = fmaf(S.om, G[jr][f], P[jr][f]);
             }
             __builtin_amdgcn_sched_barrier(0);  // keep steps apart: interleaving them only costs registers
         }
     }
 }
 
-// one stage: G, H true gradients in and out; Y, B true outputs in, m^n_cache times the stage inputs out
+// m^k by repeated multiplication (k <= 64; only groups cut by a context length come here)
+__device__ __forceinline__ float pow_steps(float base, int k) {
+    float p = 1.0f;
+    for (int i = 0; i < k; ++i) p *= base;
+    return p;
+}
+
+// True values <-> scaled state, on a register tile.
+template <int R, int F>
+__device__ __forceinline__ void scale_tile(float (&x)[R][F], float (&a)[R][F], float sx, float sa) {
+#pragma unroll
+    for (int rr = 0; rr < R; ++rr)
+#pragma unroll
+        for (int f = 0; f < F; ++f) {
+            x[rr][f] *= sx;
+            a[rr][f] *= sa;
+        }
+}
+
+// one stage of the backward from true values to true values: G, H true gradients in and out; Y, B true outputs in,
+// true inputs out
 template <int NC, int EC, int R, int F, bool MASKED, bool TANH_ONLY, bool STEP_MASK = false>
 __device__ __forceinline__ void backward_steps(float (&Y)[R][F], float (&B)[R][F], float (&G)[R][F], float (&P)[R][F],
                                                const float (&wi)[F], const float (&wj)[F], float (&dwi)[F],
                                                float (&dwj)[F], float own, const StepTable& S, int lane,
                                                float4* slots, int live = NC) {
-    const float om = 1.0f - S.m;
-    const float nom = -om;
+    // as if the NC - live skipped steps of a cut group had been done: G, P carry m^-t
+    const float isc = (STEP_MASK && live != NC) ? pow_steps(S.im, NC - live) : 1.0f;
 #pragma unroll
     for (int rr = 0; rr < R; ++rr)
 #pragma unroll
-        for (int f = 0; f < F; ++f) P[rr][f] = fmaf(om, G[rr][f], P[rr][f]);  // h -> p
-    if (STEP_MASK && live != NC) {
-        // as if the NC - live skipped steps had been done: Y, B carry m^t, G, P carry m^-t
-        const float sc = pow_steps(S.m, NC - live), isc = pow_steps(1.0f / S.m, NC - live);
-#pragma unroll
-        for (int rr = 0; rr < R; ++rr)
-#pragma unroll
-            for (int f = 0; f < F; ++f) {
-                Y[rr][f] *= sc;
-                B[rr][f] *= sc;
+        for (int f = 0; f < F; ++f) {
+            Y[rr][f] *= S.kappa;
+            B[rr][f] *= S.b_scale;
+            P[rr][f] = fmaf(S.om, G[rr][f], P[rr][f]);  // h -> p
+            if (STEP_MASK) {
                 G[rr][f] *= isc;
                 P[rr][f] *= isc;
             }
-    }
+        }
     backward_core<NC, EC, R, F, MASKED, TANH_ONLY, STEP_MASK>(Y, B, G, P, wi, wj, dwi, dwj, own, S, 0, lane, slots,
                                                              live);
-    // undo the scaling of the gradients: NC steps done
-    const float dn = S.m_pow_n;       // m^NC
+    const float dn = S.m_pow_n;       // NC steps done: undo the scaling of the gradients
 #pragma unroll
     for (int rr = 0; rr < R; ++rr)
 #pragma unroll
         for (int f = 0; f < F; ++f) {
             G[rr][f] *= dn;
-            P[rr][f] = fmaf(P[rr][f], dn, nom * G[rr][f]);  // back to h = p - (1-m) g
+            P[rr][f] = fmaf(P[rr][f], dn, -S.om * G[rr][f]);  // back to h = p - (1-m) g
         }
 }
 
@@ -413,16 +384,17 @@ __device__ __forceinline__ void backward_steps(float (&Y)[R][F], float (&B)[R][F
     float4* slots = bcast_lds + (T::LR == 1 ? 0 : wave * (F / 4) * 64);                         \
     const int fl = lane % T::LF;                                                                \
     float wi[F], wj[F];                                                                         \
-    load_w<F>(A.W, A.E, head, EC, fl, wi, wj);
+    load_w<F>(A.W, A.E, head, EC, fl, wi, wj);                                                  \
+    _Pragma("unroll") for (int f = 0; f < F; ++f) {                                             \
+        wi[f] *= A.tab.gamma;                                                                   \
+        wj[f] *= A.tab.gamma;                                                                   \
+    }
 
 // Row rr of this lane is live when its slot is below the group's live rows (always, or never, without lengths).
 #define NCN_ROW_LIVE(rr) ((int)(((lane / T::LF) % T::LR) * R + (rr)) < live)
 
-// The 4 x 4 tanh build fits 72 VGPRs (7 waves per SIMD) when asked to, against the 78 (6 waves) the compiler picks by
-// itself: measured 5 % faster on the headline shape (a wave issues more often with more waves to pick from).  The
-// other builds would spill.
 template <int NC, int EC, int R, int F, bool TANH_ONLY = true, bool INDEXED = false>
-__global__ void __launch_bounds__(kBlockThreads, (TANH_ONLY && !INDEXED && R == 4 && F == 4) ? 7 : 1) stage_forward_kernel(const StageArgs A) {
+__global__ void __launch_bounds__(kBlockThreads, (TANH_ONLY && !INDEXED && R == 4 && F == 4) ? 6 : 1) stage_forward_kernel(const StageArgs A) {
     NCN_WAVE_PROLOGUE
     for (uint32_t t = gwave / A.n_head; t < A.total_tiles; t += tile_step) {
         int64_t off[R];
@@ -434,7 +406,9 @@ __global__ void __launch_bounds__(kBlockThreads, (TANH_ONLY && !INDEXED && R == 
             load_frag<F>(A.in0, A.in_dtype, off[rr], valid, x[rr]);
             load_frag<F>(A.in1, A.in_dtype, off[rr], valid, a[rr]);
         }
-        forward_steps<NC, EC, R, F, TANH_ONLY, INDEXED>(x, a, wi, wj, A.tab, lane, slots, live);
+        scale_tile<R, F>(x, a, A.tab.kappa, A.tab.a_scale);
+        forward_core<NC, EC, R, F, TANH_ONLY, INDEXED>(x, a, wi, wj, A.tab, lane, slots, live);
+        scale_tile<R, F>(x, a, A.tab.inv_kappa, A.tab.inv_a_scale);
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) {
             const bool valid = INDEXED ? NCN_ROW_LIVE(rr) : live != 0;
@@ -461,7 +435,9 @@ __global__ void __launch_bounds__(kBlockThreads) stage_inverse_kernel(const Stag
             load_frag<F>(A.in0, A.in_dtype, off[rr], valid, y[rr]);
             load_frag<F>(A.in1, A.in_dtype, off[rr], valid, b[rr]);
         }
-        inverse_steps<NC, EC, R, F, TANH_ONLY, INDEXED>(y, b, wi, wj, A.tab, lane, slots, live);
+        scale_tile<R, F>(y, b, A.tab.kappa, A.tab.b_scale);
+        inverse_core<NC, EC, R, F, TANH_ONLY, INDEXED>(y, b, wi, wj, A.tab, lane, slots, live);
+        scale_tile<R, F>(y, b, A.tab.inv_kappa, A.tab.inv_b_scale);
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) {
             const bool valid = INDEXED ? NCN_ROW_LIVE(rr) : live != 0;
@@ -471,9 +447,8 @@ __global__ void __launch_bounds__(kBlockThreads) stage_inverse_kernel(const Stag
     }
 }
 
-// Tiles of up to 16 elements per lane fit 128 VGPRs (4 waves per SIMD) when the compiler is asked to; measured 3-4 %
-// faster than the 136 it picks by itself.  Larger tiles, the multi-activation build and the builds that mask steps
-// would spill, so they are left alone.
+// Tiles of up to 16 elements per lane fit 128 VGPRs (4 waves per SIMD) when the compiler is asked to.  Larger tiles,
+// the multi-activation build and the builds that mask steps would spill, so they are left alone.
 template <int NC, int EC, int R, int F, bool TANH_ONLY = true, bool INDEXED = false>
 __global__ void __launch_bounds__(kBlockThreads, (TANH_ONLY && R * F <= 16 && F == 4) ? 4 : 1) stage_backward_kernel(const StageArgs A) {
     NCN_WAVE_PROLOGUE
@@ -503,8 +478,8 @@ __global__ void __launch_bounds__(kBlockThreads, (TANH_ONLY && R * F <= 16 && F 
             if (A.aux0) {
 #pragma unroll
                 for (int f = 0; f < F; ++f) {
-                    Y[rr][f] *= A.tab.inv_m_pow_n;
-                    B[rr][f] *= A.tab.inv_m_pow_n;
+                    Y[rr][f] *= A.tab.inv_kappa;
+                    B[rr][f] *= A.tab.inv_b_scale;
                 }
                 store_frag<F>(A.aux0, NCN_F32, off[rr], valid, Y[rr]);
                 store_frag<F>(A.aux1, NCN_F32, off[rr], valid, B[rr]);

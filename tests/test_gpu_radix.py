@@ -36,6 +36,9 @@ CASES = [
     (2, 256, 64, 4, 4, 0, 4),      # n = 4, head width 16
     (2, 4096, 128, 4, 4, 1, 5),    # n = 4: levels 1..5 of 4^6
     (2, 96, 32, 2, 2, 0, 5),       # N = 3 * 2^5: windows that do not fill the LDS budget evenly
+    (1, 640, 128, 4, 2, 0, 2),     # 160 windows of 4 rows forward, 64 fit a workgroup: 40 per load, 4 loads
+    (1, 384, 128, 4, 2, 0, 7),     # N = 3 * 2^7: three windows of 128 rows, the backward budget takes one per load
+    (2, 768, 64, 2, 4, 0, 3),      # n = 4, N = 12 * 4^3: 12 windows, 4 per load forward, 2 per load backward
     (2, 512, 32, 2, 8, 0, 3),      # n = 8: no LDS passes, closed-form positions in the one-stage register kernels
     (2, 81, 10, 2, 3, 0, 4),       # n = 3, head width 5: generic kernel
     (2, 128, 256, 2, 2, 2, 3),     # head width 128: register kernels, one level per launch

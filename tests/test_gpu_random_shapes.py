@@ -55,8 +55,10 @@ def test_random_problem(M, case):
     amp_stage = (1 / 0.9) ** n
     # float32 rounding of the inversion grows like (1/m)^n per stage: 5x at n = 16, 29x at n = 32, 850x at n = 64
     # (where the reference's own check uses atol = 1e-2, grad_test_bench.py:161)
-    gtol = max(1e-5, 3e-6 * amp_stage)
-    rtol = max(3e-5, 3e-6 * amp_stage) if n < 64 else 1e-1
+    # (every inversion step rounds twice, the product with 1/m and the difference: about 5e-6 relative per unit of
+    # amplification; n <= 16, the group sizes of the benchmark configurations, stay at the 1e-5 bar)
+    gtol = max(1e-5, 5e-6 * amp_stage)
+    rtol = max(3e-5, 5e-6 * amp_stage) if n < 64 else 1e-1
     # one call per stage, every stage saving its outputs
     outs, cx, cxa = [], gx, gxa
     for l in range(L):

@@ -134,6 +134,27 @@ def test_radix_plan_and_argument_checks(lib):
     assert h.ncn_plan_radix(ctypes.byref(_shape(lib, 2, 96, 32, 2, 2)), 0, 6, 0, 0, None, 0) == -2   # 64 does not divide 96
     assert h.ncn_plan_radix(ctypes.byref(_shape(lib, 2, 96, 32, 2, 2)), 0, 5, 0, 0, buf, 16) == 1
     assert list(buf[0:6]) == [0, 5, 1, 1, 32, 96]                                    # three windows per workgroup
+    # every plan covers every row: N = odd * n^k leaves a window count that the per-workgroup count must divide
+    for n, ec in ((2, 32), (4, 32), (2, 16), (4, 16), (8, 32)):
+        for N in [n ** k * odd for k in range(1, 9) for odd in (1, 3, 5, 7, 9, 15) if n ** k * odd <= 4096]:
+            kmax = 0
+            while N % n ** (kmax + 1) == 0:
+                kmax += 1
+            for first in range(kmax):
+                for count in range(1, kmax - first + 1):
+                    for backward in (0, 1):
+                        sh = _shape(lib, 1, N, 4 * ec, 4, n)
+                        k = h.ncn_plan_radix(ctypes.byref(sh), first, count, 0, backward, buf, 16)
+                        assert 0 < k <= 16, (n, N, first, count, backward, k)
+                        nxt = 0
+                        for q in range(k):
+                            f, c, multi, s0, span, rows = buf[6 * q:6 * q + 6]
+                            assert f == nxt and c >= 1 and s0 == n ** (first + f) and span == n ** c
+                            nxt = f + c
+                            if multi:   # a whole number of windows per workgroup, a whole number of workgroups per entry
+                                assert rows % span == 0 and N % rows == 0, (n, N, first, count, backward, q, rows)
+                                assert rows * ec * 4 * (4 if backward else 2) <= 64 * 1024
+                        assert nxt == count
     small = _shape(lib, 2, 64, 32, 4, 4)
     p = ctypes.c_void_p(4096)       # never dereferenced: every call below fails validation first
     z = ctypes.c_void_p(0)

@@ -176,3 +176,102 @@ def test_heads_use_disjoint_weight_slices():
     y2, _ = O.stage_forward(x, xa, W2, alpha, n, C, 1)
     assert torch.equal(y[..., :4], y2[..., :4])
     assert not torch.allclose(y[..., 4:], y2[..., 4:])
+
+
+# ---- relu / sigmoid / leaky relu / linear: codes of ncn_fwd_cuda_kernel.cu:86-95, ncn_bwd_cuda_kernel.cu:137-150 --------
+def _scalar_act(t, code):
+    if code == 0:
+        return math.tanh(t)
+    if code == 1:
+        return t if t > 0.0 else 0.0
+    if code == 2:
+        return 1.0 / (1.0 + math.exp(-t))
+    if code == 3:
+        return t if t >= 0.0 else 0.01 * t
+    return t
+
+
+@pytest.mark.parametrize("act", [0, 1, 2, 3, -1], ids=["tanh", "relu", "sigmoid", "leaky_relu", "linear"])
+def test_activations_against_scalar_loops(act):
+    """One stage on a tiny input, written out with Python floats only (no tensor op shared with the oracle)."""
+    B, N, E, C, n, stage, alpha, m = 2, 8, 4, 2, 4, 1, 0.8, 0.9
+    ce = E // C
+    X, Xa, W = _rand(B, N, E, seed=31), _rand(B, N, E, seed=32), _rand(2 * E, seed=33, scale=0.7)
+    y, ya = O.stage_forward(X, Xa, W, alpha, n, C, stage, m, activation=act)
+    groups = N // n
+    stride = 0 if stage == 0 else (1 << (stage - 1)) % groups
+    for b in range(B):
+        for c in range(C):
+            wi = [float(W[c * ce + f]) for f in range(ce)]
+            wj = [float(W[E + c * ce + f]) for f in range(ce)]
+            for g in range(groups):
+                pos = [((g + o * stride) % groups) * n + o for o in range(n)]
+                x = [[float(X[b, p, c * ce + f]) for f in range(ce)] for p in pos]
+                a = [[float(Xa[b, p, c * ce + f]) for f in range(ce)] for p in pos]
+                for j in range(n):
+                    xj = list(x[j])
+                    e = sum(xj[f] * wj[f] for f in range(ce))
+                    for i in range(n):
+                        sv = sum(x[i][f] * wi[f] for f in range(ce)) + e
+                        for f in range(ce):
+                            Fv = _scalar_act(alpha * x[i][f] + (1.0 - alpha) * sv * xj[f], act)
+                            a[i][f] = m * a[i][f] + (1.0 - m) * Fv
+                            x[i][f] = m * x[i][f] + (1.0 - m) * a[i][f]
+                for o, p in enumerate(pos):
+                    for f in range(ce):
+                        assert abs(float(y[b, p, c * ce + f]) - x[o][f]) < 1e-13
+                        assert abs(float(ya[b, p, c * ce + f]) - a[o][f]) < 1e-13
+
+
+def test_sigmoid_branch_is_the_pinned_tanh_branch_at_half_the_argument():
+    T = _rand(4, 50, seed=34, scale=3.0)
+    F, dF = O._act(T, O.ACT_SIGMOID)
+    Ft, dFt = O._act(T / 2, O.ACT_TANH)
+    assert torch.allclose(F, (1.0 + Ft) / 2.0, atol=1e-15)
+    assert torch.allclose(dF, dFt / 4.0, atol=1e-15)          # d/dT (1 + tanh(T/2))/2 = (1 - tanh^2(T/2))/4
+
+
+def test_relu_and_leaky_relu_slopes_by_hand():
+    T = torch.tensor([-2.0, -1e-9, 0.0, 1e-9, 3.0], dtype=D)
+    F, dF = O._act(T, O.ACT_RELU)
+    assert F.tolist() == [0.0, 0.0, 0.0, 1e-9, 3.0] and dF.tolist() == [0.0, 0.0, 0.0, 1.0, 1.0]
+    F, dF = O._act(T, O.ACT_LEAKY_RELU)
+    assert F.tolist() == pytest.approx([-0.02, -1e-11, 0.0, 1e-9, 3.0], rel=1e-14) and dF.tolist() == [0.01, 0.01, 1.0, 1.0, 1.0]
+
+
+@pytest.mark.parametrize("act", [1, 2, 3], ids=["relu", "sigmoid", "leaky_relu"])
+def test_closed_form_backward_against_finite_differences(act):
+    """dx, dxa and dW of a two-stage stack against central differences of the forward in float64, on a seed whose
+    every |T| stays above 1e-3 (so that no difference straddles the kink of relu / leaky relu)."""
+    batch, N, E, C, n, L, alpha = 1, 8, 4, 2, 2, 2, 0.8
+    for seed in range(100, 200):
+        x, xa, Ws, dy, dya = O.make_inputs(batch, N, E, L, n, seed=seed, xa_zero=False, dtype=D)
+        if O.net_min_abs_T(x, xa, Ws, alpha, n, C, activation=act) > 1e-3:
+            break
+    else:
+        pytest.fail("no seed keeps |T| away from zero")
+    _, _, dx, dxa, dWs = O.net_backward_checkpointed(x, xa, dy, dya, Ws, alpha, n, C, activation=act)
+
+    def loss(x_, xa_, Ws_):
+        y, ya = O.net_forward(x_, xa_, Ws_, alpha, n, C, activation=act)
+        return float((y * dy).sum() + (ya * dya).sum())
+
+    eps = 1e-6
+    gen = torch.Generator().manual_seed(5)
+    for which, grad in (("x", dx), ("xa", dxa), ("W0", dWs[0]), ("W1", dWs[1])):
+        for _ in range(12):
+            k = int(torch.randint(0, grad.numel(), (1,), generator=gen))
+            args = {"x": x.clone(), "xa": xa.clone(), "W0": Ws[0].clone(), "W1": Ws[1].clone()}
+            args[which].view(-1)[k] += eps
+            up = loss(args["x"], args["xa"], [args["W0"], args["W1"]])
+            args[which].view(-1)[k] -= 2 * eps
+            dn = loss(args["x"], args["xa"], [args["W0"], args["W1"]])
+            fd = (up - dn) / (2 * eps)
+            assert abs(fd - float(grad.view(-1)[k])) < 1e-7 * max(1.0, abs(fd)), (which, k, fd, float(grad.view(-1)[k]))
+
+
+def test_signed_regime_inputs_keep_away_from_the_kink():
+    x, xa, Ws, _, _ = O.make_inputs_signed_regimes(2, 64, 64, 3, 16, seed=3, dtype=D)
+    assert O.net_min_abs_T(x, xa, Ws, 0.9, 16, 2, activation=O.ACT_RELU) > 1e-3
+    y, _ = O.net_forward(x, xa, Ws, 0.9, 16, 2, activation=O.ACT_RELU)
+    assert (y[0] > 0).all() and (y[1] < 0).all()
