@@ -479,8 +479,18 @@ def make_inputs(batch, N, E, L, n, seed=0, xa_zero=True, w_scale=1.0, dtype=torc
 
 
 def rel_err(a, b):
-    """max |a-b| / max |b| : the relative error figure used for every parity claim in this repo."""
+    """max |a-b| / max |b| : the relative error figure used for every parity claim in this repo.  It is a statement
+    about the tensor as a whole, scaled by its largest entry: entries much smaller than that can be off by more than
+    the figure in their own terms (rms_err is the companion figure over all entries)."""
     a = a.detach().double().cpu()
     b = b.detach().double().cpu()
     denom = b.abs().max().item()
     return (a - b).abs().max().item() / (denom if denom > 0 else 1.0)
+
+
+def rms_err(a, b):
+    """sqrt(mean (a-b)^2) / sqrt(mean b^2): the root-mean-square error relative to the tensor's root mean square."""
+    a = a.detach().double().cpu()
+    b = b.detach().double().cpu()
+    denom = b.pow(2).mean().sqrt().item()
+    return (a - b).pow(2).mean().sqrt().item() / (denom if denom > 0 else 1.0)

@@ -2,6 +2,9 @@
 does not depend on size: (batch, head) instances are independent, hence the first batch entries of a full-size run
 must equal the oracle on just those entries; dW is a sum over batch entries, hence the full-size dW must equal the
 sum of the dW of batch chunks; inverse(forward(x)) must give x back; two runs must agree bit for bit."""
+import json
+import os
+
 import pytest
 import torch
 
@@ -36,9 +39,15 @@ def _inputs(name):
     return x, xa, dy, W
 
 
+def _segment(n):
+    """Stages per saved checkpoint, as bench.py and the whole-net autograd node choose it."""
+    from ncn_cuda_amd.modules import default_save_every
+    return default_save_every(n)
+
+
 def _run(M, x, xa, dy, W, C, n, L, dtype):
-    """Forward + reversible backward the way bench.py runs the configuration: segments of 26 // n stages."""
-    seg = max(1, 26 // n)
+    """Forward + reversible backward the way bench.py runs the configuration: segments of default_save_every(n) stages."""
+    seg = _segment(n)
     saved, spans = [], []
     cx, cxa = x, xa
     for a in range(0, L, seg):
@@ -73,7 +82,7 @@ def test_full_size_slice_parity_and_dw_additivity(M, name):
     d = torch.float64
     ref = O.net_autograd(x[:k].cpu().to(d), xa[:k].cpu().to(d), [w.cpu().to(d) for w in W], dy[:k].cpu().to(d),
                          torch.zeros(k, N, E, dtype=d), 0.9, n, C)
-    gtol = max(tol, 1e-6 * (1 / 0.9) ** (n * max(1, 26 // n)))     # rounding growth of the reversal per segment
+    gtol = tol                                                     # float32: 1e-5 on the gradients too
     assert O.rel_err(y[:k], ref[0]) < tol and O.rel_err(ya[:k], ref[1]) < tol
     assert O.rel_err(dx[:k], ref[2]) < gtol and O.rel_err(dxa[:k], ref[3]) < gtol
     # dW of the two entries alone (GPU) against the oracle, then additivity over batch chunks for the rest
@@ -95,7 +104,7 @@ def test_full_size_inverse_round_trip(M, name):
     batch, N, E, C, n, L, dtype, _ = CONFIGS[name]
     x, xa, _, W = _inputs(name)
     x, xa = x.float(), xa.float()
-    seg = max(1, 26 // n)
+    seg = _segment(n)
     for a in range(0, L, seg):            # reversal is only asked over what one saved checkpoint covers
         cnt = min(seg, L - a)
         y, ya = M.forward_stages(x, xa, W[a:a + cnt], 0.9, 0, n, C, a, cnt)
@@ -157,13 +166,22 @@ def test_whole_tensor_against_the_c_oracle(M, name, entries):
     d = torch.float64
     ref = CO.net_forward_backward(x[sel].cpu().to(d), xa[sel].cpu().to(d), [w.cpu().to(d) for w in W], dy[sel].cpu().to(d),
                                   None, 0.9, n, C, keep_outputs=False)   # float64: reversal costs nothing, L copies do
+    # 2e-2 with bf16 storage, 1e-5 in float32, for the outputs and for every gradient (max |diff| / max |ref| over the
+    # whole tensor; the root-mean-square figure is recorded beside it)
     tol = 2e-2 if dtype == torch.bfloat16 else 1e-5
-    gtol = max(tol, 3e-6 * (1 / 0.9) ** (n * max(1, 26 // n)))     # rounding growth of the reversal per segment
-    assert O.rel_err(y[sel].float().cpu(), ref[0]) < tol and O.rel_err(ya[sel].float().cpu(), ref[1]) < tol
-    assert O.rel_err(dx[sel].float().cpu(), ref[2]) < gtol and O.rel_err(dxa[sel].float().cpu(), ref[3]) < gtol
+    got = {"y": y[sel], "ya": ya[sel], "dx": dx[sel], "dxa": dxa[sel]}
+    want = {"y": ref[0], "ya": ref[1], "dx": ref[2], "dxa": ref[3]}
+    report = {k: {"max": O.rel_err(got[k].float().cpu(), want[k]), "rms": O.rms_err(got[k].float().cpu(), want[k])}
+              for k in got}
     if entries is None:                                            # dW sums over the whole batch
-        for l in range(L):
-            assert O.rel_err(dW[l].cpu(), ref[4][l]) < gtol, l
+        per_stage = [O.rel_err(dW[l].cpu(), ref[4][l]) for l in range(L)]
+        report["dW_worst"] = {"max": max(per_stage), "rms": max(O.rms_err(dW[l].cpu(), ref[4][l]) for l in range(L))}
+    print(f"measured errors {name} (segments of {_segment(n)} stages): " + json.dumps(report))
+    if os.environ.get("NCN_ERROR_REPORT"):                         # a file to read the figures from after a run
+        with open(os.environ["NCN_ERROR_REPORT"], "a") as fh:
+            fh.write(json.dumps({"config": name, "segment": _segment(n), **report}) + "\n")
+    for k, v in report.items():
+        assert v["max"] < tol, (k, v)
 
 
 def test_headline_shape_with_table_and_lengths_against_the_c_oracle(M):

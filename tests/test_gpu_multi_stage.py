@@ -90,15 +90,19 @@ def test_multi_stage_dya_none_and_bf16_input(M):
         assert O.rel_err(a[4][l], ref[4][l]) < 1e-4
 
 
-@pytest.mark.parametrize("act", [2, -1, 3], ids=["sigmoid", "linear", "leaky_relu"])
+@pytest.mark.parametrize("act", [1, 2, -1, 3], ids=["relu", "sigmoid", "linear", "leaky_relu"])
 @pytest.mark.parametrize("case", [(2, 1024, 64, 2, 2, 0, 9), (2, 512, 128, 4, 4, 1, 4)],
                          ids=["n2_halo_and_closed", "n4_from_stage1"])
 def test_multi_stage_other_activations(M, case, act):
-    """The LDS passes in their runtime-activation build (relu is left out as in the one-stage test: its kink makes
-    the reversible recomputation flip F' for |T| ~ eps)."""
+    """The LDS passes in their runtime-activation build.  relu and leaky relu have a kink at T = 0, where a float32
+    recomputation may pick the other slope: they run on inputs whose T keeps one sign per batch entry (both slopes,
+    never near the kink), so every gradient entry is compared."""
     batch, N, E, C, n, first, L = case
     alpha = 0.9
-    x, xa, Ws, dyi, dya = O.make_inputs(batch, N, E, L, n, seed=23, xa_zero=False)
+    if act in (1, 3):
+        x, xa, Ws, dyi, dya = O.make_inputs_signed_regimes(batch, N, E, L, n, seed=23)
+    else:
+        x, xa, Ws, dyi, dya = O.make_inputs(batch, N, E, L, n, seed=23, xa_zero=False)
     gx, gxa, gdy, gdya = x.cuda(), xa.cuda(), dyi.cuda(), dya.cuda()
     Wst = torch.stack(Ws).cuda()
     import ctypes
@@ -112,17 +116,9 @@ def test_multi_stage_other_activations(M, case, act):
     assert O.rel_err(y, ref[0]) < 1e-5 and O.rel_err(ya, ref[1]) < 1e-5
     xr, xar, dx, dxa, dW = M.backward_stages(y, ya, gdy, gdya, Wst, alpha, act, n, C, first, L)
     tol = max(1e-5, 5e-7 * (1 / 0.9) ** (n * L))
-    assert O.rel_err(xr, x) < tol and O.rel_err(xar, xa) < tol
-    if act == 3:
-        # a kink: where |T| is within rounding of 0 the recomputed slope flips between 1 and 0.01, which moves a
-        # handful of gradient entries (and, through them, dW a little); everything else must agree
-        def q999(a, b):
-            e = (a.detach().double().cpu() - b).abs().flatten() / b.abs().max()
-            return e.kthvalue(int(0.999 * e.numel())).values.item()
-        assert q999(dx, ref[2]) < tol and q999(dxa, ref[3]) < tol
-        for l in range(L):
-            assert O.rel_err(dW[l], ref[4][l]) < 1e-3
-        return
+    # (the sign-regime inputs of relu / leaky relu have xa in [0, 0.5] beside x in [0.5, 1.5]: the error of xa is
+    # measured against the smaller of the two scales)
+    assert O.rel_err(xr, x) < tol and O.rel_err(xar, xa) < (3 * tol if act in (1, 3) else tol)
     assert O.rel_err(dx, ref[2]) < tol and O.rel_err(dxa, ref[3]) < tol
     for l in range(L):
         assert O.rel_err(dW[l], ref[4][l]) < tol

@@ -99,8 +99,10 @@ def test_forward_backward_inverse_vs_oracle(M, shape):
     assert O.rel_err(outs[-1][1], ref_ya) < TOL_F32
     # the reversible backward divides by m at each of the n steps of a stage: float32 rounding grows like
     # (1/m)^n (5x at n = 16, 29x at n = 32, 850x at n = 64), which only matters above n = 16
-    tol_inv = max(TOL_F32, 3e-6 * (1 / 0.9) ** n)
-    tol_bwd = TOL_F32 if n <= 32 else tol_inv
+    # (n <= 16, the group sizes of the benchmark configurations, are held to 1e-5; every step rounds about 1e-7
+    # relative, which the steps that follow amplify: 5e-6 per unit of amplification covers n = 32 and 64)
+    tol_inv = max(TOL_F32, 5e-6 * (1 / 0.9) ** n)
+    tol_bwd = TOL_F32 if n <= 16 else tol_inv
     xr, xar, dx, dxa, dWs = _stack_backward(M, outs, gdyi, gdya, gWs, alpha, n, C)
     assert O.rel_err(dx, ref_dx) < tol_bwd
     assert O.rel_err(dxa, ref_dxa) < tol_bwd
@@ -157,11 +159,23 @@ def test_dya_none_equals_zeros(M):
 @pytest.mark.parametrize("act", [1, 2, -1, 3], ids=["relu", "sigmoid", "linear", "leaky_relu"])
 def test_other_activations_vs_oracle(M, act, shape):
     """relu / sigmoid / linear (codes of ncn_fwd_cuda_kernel.cu:86-95) and the Triton kernels' leaky relu
-    (ncn_triton.py:22-28) on the register kernels and on the generic kernel; the oracle for them is pinned by autograd only."""
+    (ncn_triton.py:22-28) on the register kernels and on the generic kernel; the oracle's branches for them are pinned by
+    scalar loops, identities and finite differences (tests/test_oracle_properties.py).
+    relu and leaky relu have a kink at T = 0, where a float32 recomputation may pick the other slope: the small shapes
+    use a seed whose every |T| stays above 1e-4 (checked in float64), the large one inputs whose T keeps one sign per
+    batch entry (both slopes, never near the kink)."""
     batch, N, E, C, n, L = shape
     alpha = 0.9
-    x, xa, Ws, dyi, dya = O.make_inputs(batch, N, E, L, n, seed=21, xa_zero=False)
     d = torch.float64
+    if act in (1, 3) and batch * N * E * n * L > 100000:
+        x, xa, Ws, dyi, dya = O.make_inputs_signed_regimes(batch, N, E, L, n, seed=21)
+    else:
+        for seed in range(21, 400):
+            x, xa, Ws, dyi, dya = O.make_inputs(batch, N, E, L, n, seed=seed, xa_zero=False)
+            if act not in (1, 3) or O.net_min_abs_T(x.to(d), xa.to(d), [w.to(d) for w in Ws], alpha, n, C, activation=act) > 1e-4:
+                break
+        else:
+            pytest.fail("no seed keeps |T| away from zero")
     ref_yi, ref_ya, ref_dx, ref_dxa, ref_dWs = O.net_autograd(x.to(d), xa.to(d), [w.to(d) for w in Ws], dyi.to(d),
                                                               dya.to(d), alpha, n, C, activation=act)
     gx, gxa, gdyi, gdya = _dev(x, xa, dyi, dya)
@@ -172,8 +186,6 @@ def test_other_activations_vs_oracle(M, act, shape):
     ix, ixa = M.inverse(outs[-1][0], outs[-1][1], gWs[-1], alpha, act, n, C, L - 1)
     prev = outs[-2]
     assert O.rel_err(ix, prev[0]) < 3e-5 and O.rel_err(ixa, prev[1]) < 3e-5
-    if act == 1:
-        return  # relu's kink makes the reversible recomputation flip F' for |T| ~ eps: gradients not compared
     _, _, dx, dxa, dWs = _stack_backward(M, outs, gdyi, gdya, gWs, alpha, n, C, act)
     assert O.rel_err(dx, ref_dx) < TOL_F32
     assert O.rel_err(dxa, ref_dxa) < TOL_F32

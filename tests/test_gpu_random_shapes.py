@@ -19,7 +19,7 @@ def M():
     return ncn_cuda_module
 
 
-def _cases(seed, count):
+def _cases(seed, count, acts=None):
     rng = random.Random(seed)
     out = []
     while len(out) < count:
@@ -35,18 +35,24 @@ def _cases(seed, count):
         L = rng.randint(1, 4 if n >= 8 else 6)
         first = rng.choice([0, 0, 1, 3])
         act = rng.choice([0, 0, 0, 2, -1, 3])
-        out.append((batch, n * groups, ec * C, C, n, first, L, act))
+        out.append((batch, n * groups, ec * C, C, n, first, L, act if acts is None else acts[len(out) % len(acts)]))
     return out
 
 
-CASES = _cases(2024, 40) + _cases(7, 40)
+# the last 16: relu and leaky relu (codes 1 and 3) on inputs that stay away from the kink
+CASES = _cases(2024, 40) + _cases(7, 40) + _cases(11, 16, acts=(1, 3))
 
 
 @pytest.mark.parametrize("case", CASES, ids=lambda c: "b%d_N%d_E%d_C%d_n%d_s%d_L%d_a%d" % c)
 def test_random_problem(M, case):
     batch, N, E, C, n, first, L, act = case
     alpha = 0.85
-    x, xa, Ws, dy, dya = O.make_inputs(batch, N, E, L, n, seed=sum(case) + 5, xa_zero=False)
+    if act in (1, 3):
+        # relu / leaky relu: a float32 recomputation picks the other slope where |T| ~ 1e-7; inputs whose T keeps its
+        # sign (positive in even batch entries, negative in odd ones) exercise both slopes and stay away from the kink
+        x, xa, Ws, dy, dya = O.make_inputs_signed_regimes(batch, N, E, L, n, seed=sum(case) + 5)
+    else:
+        x, xa, Ws, dy, dya = O.make_inputs(batch, N, E, L, n, seed=sum(case) + 5, xa_zero=False)
     d = torch.float64
     ref = O.net_autograd(x.to(d), xa.to(d), [w.to(d) for w in Ws], dy.to(d), dya.to(d), alpha, n, C, activation=act,
                          first_stage=first)
@@ -55,10 +61,10 @@ def test_random_problem(M, case):
     amp_stage = (1 / 0.9) ** n
     # float32 rounding of the inversion grows like (1/m)^n per stage: 5x at n = 16, 29x at n = 32, 850x at n = 64
     # (where the reference's own check uses atol = 1e-2, grad_test_bench.py:161)
-    # (every inversion step rounds twice, the product with 1/m and the difference: about 5e-6 relative per unit of
-    # amplification; n <= 16, the group sizes of the benchmark configurations, stay at the 1e-5 bar)
-    gtol = max(1e-5, 5e-6 * amp_stage)
-    rtol = max(3e-5, 5e-6 * amp_stage) if n < 64 else 1e-1
+    # (n <= 16, the group sizes of the benchmark configurations, are held to 1e-5 whatever the amplification; above,
+    # the sign-regime inputs of relu / leaky relu reach 9e-6 per unit of amplification at n = 64)
+    gtol = (2e-5 if n >= 64 else 1e-5) * amp_stage if n >= 32 else 1e-5
+    rtol = max(3e-5, 1e-5 * amp_stage) if n < 64 else 2e-1
     # one call per stage, every stage saving its outputs
     outs, cx, cxa = [], gx, gxa
     for l in range(L):
@@ -68,16 +74,14 @@ def test_random_problem(M, case):
     g, h = gdy, gdya
     for l in range(L - 1, -1, -1):
         xr, xar, g, h, dW = M.backward_stages(outs[l][0], outs[l][1], g, h, W[l], alpha, act, n, C, first + l, 1)
-        if act != 3:      # leaky relu: a slope flipped at |T| ~ eps moves single entries, see the activation tests
-            assert O.rel_err(dW[0], ref[4][l]) < gtol, f"dW{l}"
+        assert O.rel_err(dW[0], ref[4][l]) < gtol, f"dW{l}"
         prev = outs[l - 1] if l else (gx, gxa)
         assert O.rel_err(xr, prev[0]) < rtol and O.rel_err(xar, prev[1]) < rtol
-    if act != 3:
-        assert O.rel_err(g, ref[2]) < gtol and O.rel_err(h, ref[3]) < gtol
+    assert O.rel_err(g, ref[2]) < gtol and O.rel_err(h, ref[3]) < gtol
     # the same stages in one call (multi-stage passes where the shape allows), forward only compared tightly
     y, ya = M.forward_stages(gx, gxa, W, alpha, act, n, C, first, L)
     assert O.rel_err(y, ref[0]) < 1e-5 and O.rel_err(ya, ref[1]) < 1e-5
-    if (1 / 0.9) ** (n * L) < 50 and act != 3:
+    if (1 / 0.9) ** (n * L) < 50:
         _, _, dx, dxa, dWs = M.backward_stages(y, ya, gdy, gdya, W, alpha, act, n, C, first, L)
         tol = max(1e-5, 2e-6 * (1 / 0.9) ** (n * L))
         assert O.rel_err(dx, ref[2]) < tol and O.rel_err(dxa, ref[3]) < tol
@@ -95,9 +99,8 @@ def test_random_problem(M, case):
     ixr, ixar, idx, idxa, idW = M.backward_stages(iy, iya, gdy, gdya, W[0], alpha, act, n, C, 0, 1, group_index=gt,
                                                   ctx_len=gl)
     assert O.rel_err(ixr, x) < rtol
-    if act != 3:
-        assert O.rel_err(idx, iref[2]) < gtol and O.rel_err(idxa, iref[3]) < gtol
-        assert O.rel_err(idW[0], iref[4][0]) < gtol
+    assert O.rel_err(idx, iref[2]) < gtol and O.rel_err(idxa, iref[3]) < gtol
+    assert O.rel_err(idW[0], iref[4][0]) < gtol
     # the first levels of the radix-n grouping that N admits, without tables
     levels = 0
     while n > 1 and levels < L and N % n ** (levels + 1) == 0:
@@ -108,7 +111,7 @@ def test_random_problem(M, case):
                                       rtables, activation=act)
         ry, rya = M.forward_radix(gx, gxa, W[:levels], alpha, act, n, C, 0, levels)
         assert O.rel_err(ry, rref[0]) < 1e-5 and O.rel_err(rya, rref[1]) < 1e-5
-        if (1 / 0.9) ** (n * levels) < 50 and act != 3:
+        if (1 / 0.9) ** (n * levels) < 50:
             rxr, _, rdx, rdxa, rdW = M.backward_radix(ry, rya, gdy, gdya, W[:levels], alpha, act, n, C, 0, levels)
             tol = max(1e-5, 2e-6 * (1 / 0.9) ** (n * levels))
             assert O.rel_err(rdx, rref[2]) < tol and O.rel_err(rdxa, rref[3]) < tol and O.rel_err(rxr, x) < tol
