@@ -62,6 +62,7 @@ extern "C" {
 #define NCN_ERR_UNSUPPORTED (-6) /* n_cache > 64, or head width too large for the generic kernel */
 #define NCN_ERR_ALIGN (-7)       /* a pointer is not 16-byte aligned (4-byte for the int32 tables) */
 #define NCN_ERR_ALIAS (-8)       /* n_stages > 1 needs the state buffers the call would carry it in */
+#define NCN_ERR_STATIC_LIMIT (-9) /* ncn_backward_static: the shape needs more scratch than the library holds */
 
 /* Shape of one problem; shared by all entry points. */
 typedef struct ncn_shape {
@@ -124,6 +125,30 @@ int ncn_backward(const void* y, const void* ya, int y_dtype,
                  void* workspace, size_t workspace_bytes,
                  const ncn_shape* shape, int first_stage, int n_stages,
                  float alpha, float m, int activation, void* stream);
+
+/*
+ * ncn_backward without a workspace argument and without any allocation, for callers that cannot allocate device
+ * memory (code under HIP graph capture, serving loops, harnesses that forbid it).  No counterpart in the reference,
+ * whose host functions allocate every output and the [batch, N, 2E] dW partial tensor themselves
+ * (ncn_bwd_cuda_kernel.cu:247-251).  The dW partial rows live in an array inside the library
+ * (ncn_static_scratch_bytes() bytes, about 9 MiB, held by every GPU the library runs on until the process ends).
+ * Limits: E <= 256 (NCN_ERR_STATIC_LIMIT above that); always one launch per stage, also where ncn_backward would use
+ * its multi-stage passes, so with n_stages > 1 the two agree to rounding, not bit for bit; dx, dxa, x_rec, xa_rec of
+ * one stage are bit-identical to ncn_backward's, dW sums the same terms over fewer partial rows.
+ * Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (different streams or threads) race;
+ * calls on one stream are ordered.  Nothing in the array has to be cleared between calls.
+ * Arguments as ncn_backward.
+ */
+int ncn_backward_static(const void* y, const void* ya, int y_dtype,
+                        const void* dy, const void* dya, int dy_dtype,
+                        void* dx, void* dxa, int dx_dtype,
+                        float* x_rec, float* xa_rec,
+                        const float* W, float* dW,
+                        const ncn_shape* shape, int first_stage, int n_stages,
+                        float alpha, float m, int activation, void* stream);
+
+/* Size in bytes of the library's own scratch array per GPU (see ncn_backward_static). */
+size_t ncn_static_scratch_bytes(void);
 
 /*
  * Inverse of stages first_stage+n_stages-1 .. first_stage: x, xa such that ncn_forward(x, xa) = y, ya.

@@ -14,7 +14,7 @@ ACT_TANH, ACT_RELU, ACT_SIGMOID, ACT_LEAKY_RELU, ACT_LINEAR = 0, 1, 2, 3, -1
 EXPORTS = ("ncn_forward", "ncn_backward", "ncn_inverse", "ncn_forward_indexed", "ncn_backward_indexed",
            "ncn_inverse_indexed", "ncn_forward_radix", "ncn_backward_radix", "ncn_inverse_radix", "ncn_plan_radix", "ncn_workspace_bytes", "ncn_workspace_bytes_stages",
            "ncn_plan_passes", "ncn_kernel_path",
-           "ncn_check_shape", "ncn_error_string", "ncn_version")
+           "ncn_check_shape", "ncn_error_string", "ncn_version", "ncn_backward_static", "ncn_static_scratch_bytes")
 
 
 class NcnShape(ctypes.Structure):
@@ -42,6 +42,10 @@ def load():
     lib.ncn_backward.restype = i
     lib.ncn_backward.argtypes = [vp, vp, i, vp, vp, i, vp, vp, i, f32p, f32p, f32p, f32p, vp, ctypes.c_size_t,
                                  shp, i, i, fl, fl, i, vp]
+    lib.ncn_backward_static.restype = i
+    lib.ncn_backward_static.argtypes = [vp, vp, i, vp, vp, i, vp, vp, i, f32p, f32p, f32p, f32p, shp, i, i, fl, fl, i, vp]
+    lib.ncn_static_scratch_bytes.restype = ctypes.c_size_t
+    lib.ncn_static_scratch_bytes.argtypes = []
     lib.ncn_inverse.restype = i
     lib.ncn_inverse.argtypes = [vp, vp, i, vp, vp, i, f32p, shp, i, i, fl, fl, i, vp]
     lib.ncn_forward_indexed.restype = i

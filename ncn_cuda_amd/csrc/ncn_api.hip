@@ -2,6 +2,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cmath>
+#include <mutex>
 
 #include "../../include/ncn_hip.h"
 #include "ncn_fused_kernels.h"
@@ -74,9 +75,10 @@ struct Plan {
 };
 
 // reserve_rows: rows of the dW partial buffer kept free for another launch of the same stage
-Plan make_plan(const ncn_shape* sh, int path, int reserve_rows = 0) {
+// row_cap: rows of the dW partial buffer the caller has (kMaxGridX in a workspace of ncn_workspace_bytes)
+Plan make_plan(const ncn_shape* sh, int path, int reserve_rows = 0, int row_cap = kMaxGridX) {
     Plan p;
-    const int max_rows = kMaxGridX - reserve_rows;
+    const int max_rows = row_cap - reserve_rows;
     p.path = path;
     const int ec = (int)(sh->E / sh->n_head);
     p.groups_per_tile = (p.path == 2) ? fast_groups_per_tile(sh->n_cache, ec) : generic_groups_per_tile(sh->n_cache);
@@ -224,9 +226,11 @@ int edge_rows(const ncn_shape* sh) { return (int)(sh->batch < kEdgeGridX ? sh->b
 
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
-size_t base_workspace_bytes(const ncn_shape* sh) {
-    return align256((size_t)(kMaxGridX + kReduceLevel1Rows) * 2 * (size_t)sh->E * sizeof(float));
+// dW partial rows of the backward launches of a call, then the chunk sums of the first reduction level
+size_t partial_buffer_bytes(const ncn_shape* sh, int row_cap) {
+    return align256((size_t)(row_cap + kReduceLevel1Rows) * 2 * (size_t)sh->E * sizeof(float));
 }
+size_t base_workspace_bytes(const ncn_shape* sh) { return partial_buffer_bytes(sh, kMaxGridX); }
 
 // the multi-stage plan of a stage range, or an empty vector when the one-stage loop should be used
 std::vector<FusedPass> multi_stage_plan(const ncn_shape* sh, int first_stage, int n_stages, int activation, bool backward,
@@ -248,14 +252,14 @@ size_t temp_bytes(const ncn_shape* sh, bool backward) {
 // and the job (kReduceMaxSegments launches, kReduceMaxStages stages) hold them.
 class DwReducer {
   public:
-    DwReducer(float* partials, float* level1, int64_t two_e, hipStream_t s)
-        : partials_(partials), level1_(level1), two_e_(two_e), stream_(s) { job_.n = 0; }
+    DwReducer(float* partials, float* level1, int64_t two_e, hipStream_t s, int row_cap = kMaxGridX)
+        : partials_(partials), level1_(level1), two_e_(two_e), stream_(s), row_cap_(row_cap) { job_.n = 0; }
     // Where a launch of `rows` partial rows of `stages` stages each may write; earlier launches are summed first
     // if it would not fit behind them.
     hipError_t reserve(int rows, int stages, float** region) {
         hipError_t err = hipSuccess;
         if (job_.n == kReduceMaxSegments || stages_ + stages > kReduceMaxStages ||
-            used_rows_ + (int64_t)rows * stages > kMaxGridX)
+            used_rows_ + (int64_t)rows * stages > row_cap_)
             err = flush();
         *region = partials_ + used_rows_ * two_e_;
         return err;
@@ -290,9 +294,44 @@ class DwReducer {
     int64_t two_e_;
     hipStream_t stream_;
     ReduceJob job_;
+    int row_cap_;
     int64_t used_rows_ = 0, level1_floats_ = 0;
     int stages_ = 0, chunks_ = 0;
 };
+
+// ---- scratch of ncn_backward_static: device memory that belongs to the library, one copy per GPU -----------------
+// Holds the dW partial rows and chunk sums that ncn_backward takes from its workspace argument.  kStaticRowCap partial
+// rows (a quarter of what a workspace gives: large problems loop over them) of up to kStaticMaxTwoE floats.
+constexpr int kStaticRowCap = 4096;
+constexpr int kStaticMaxTwoE = 512;
+constexpr size_t kStaticScratchFloats = (size_t)(kStaticRowCap + kReduceLevel1Rows) * kStaticMaxTwoE;   // 9.0 MiB
+constexpr int kStaticMaxDevices = 64;
+
+}  // namespace
+
+static __device__ __align__(256) float ncn_static_scratch[kStaticScratchFloats];
+
+namespace {
+
+// Address of the array on the current device.  The array's name is only a host-side handle: the address a kernel
+// can use comes from hipGetSymbolAddress, once per device (every GPU holds its own copy at its own address).
+hipError_t static_scratch(float** out) {
+    static float* ptrs[kStaticMaxDevices] = {};
+    static std::mutex lock;
+    int dev = -1;
+    hipError_t err = hipGetDevice(&dev);
+    if (err != hipSuccess) return err;
+    if (dev < 0 || dev >= kStaticMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> guard(lock);
+    if (!ptrs[dev]) {
+        void* p = nullptr;
+        err = hipGetSymbolAddress(&p, HIP_SYMBOL(ncn_static_scratch));
+        if (err != hipSuccess) return err;
+        ptrs[dev] = static_cast<float*>(p);
+    }
+    *out = ptrs[dev];
+    return hipSuccess;
+}
 
 }  // namespace
 
@@ -329,6 +368,7 @@ const char* ncn_error_string(int code) {
         case NCN_ERR_UNSUPPORTED: return "unsupported shape: n_cache must be <= 64 and the head width <= 64 (128 for power-of-two n_cache <= 16)";
         case NCN_ERR_ALIGN: return "a pointer is not 16-byte aligned (4-byte for group_index and ctx_len)";
         case NCN_ERR_ALIAS: return "n_stages > 1 needs float32 x_rec, xa_rec, dx, dxa to carry the state";
+        case NCN_ERR_STATIC_LIMIT: return "ncn_backward_static: E is above 256, the limit of the library's own scratch";
         default: break;
     }
     if (code > 0) return hipGetErrorString((hipError_t)code);
@@ -522,7 +562,8 @@ static int inverse_impl(const void* y, const void* ya, int in_dtype, void* x, vo
 static int backward_impl(const void* y, const void* ya, int y_dtype, const void* dy, const void* dya, int dy_dtype,
                          void* dx, void* dxa, int dx_dtype, float* x_rec, float* xa_rec, const float* W, float* dW,
                          void* workspace, size_t workspace_bytes, const Grouping& grouping, const ncn_shape* shape,
-                         int first_stage, int n_stages, float alpha, float m, int activation, void* stream) {
+                         int first_stage, int n_stages, float alpha, float m, int activation, void* stream,
+                         int row_cap = kMaxGridX) {
     int rc = check_shape(shape, first_stage, n_stages, activation);
     if (rc != NCN_OK) return rc;
     rc = check_grouping(grouping, shape);
@@ -531,7 +572,7 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
     if ((x_rec == nullptr) != (xa_rec == nullptr)) return NCN_ERR_NULL;
     if (!known_dtype(y_dtype) || !known_dtype(dy_dtype) || !known_dtype(dx_dtype)) return NCN_ERR_DTYPE;
     if (n_stages > 1 && (!x_rec || dx_dtype != NCN_F32)) return NCN_ERR_ALIAS;
-    if (!workspace || workspace_bytes < ncn_workspace_bytes(shape)) return NCN_ERR_WORKSPACE;
+    if (!workspace || workspace_bytes < partial_buffer_bytes(shape, row_cap)) return NCN_ERR_WORKSPACE;
     if (!aligned16(y) || !aligned16(ya) || !aligned16(dy) || !aligned16(dya) || !aligned16(dx) || !aligned16(dxa) ||
         !aligned16(x_rec) || !aligned16(xa_rec) || !aligned16(W) || !aligned16(dW) || !aligned16(workspace))
         return NCN_ERR_ALIGN;
@@ -539,16 +580,17 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
     const int path = kernel_path_for(shape, activation, alpha, m);
     if (path == 0) return NCN_ERR_UNSUPPORTED;
     const int extra_rows = (grouping.ctx_len && path != 2) ? edge_rows(shape) : 0;
-    const Plan p = make_plan(shape, path, extra_rows);
+    const Plan p = make_plan(shape, path, extra_rows, row_cap);
     hipStream_t s = static_cast<hipStream_t>(stream);
     float* partials = static_cast<float*>(workspace);
-    float* level1 = partials + (int64_t)kMaxGridX * 2 * shape->E;
+    float* level1 = partials + (int64_t)row_cap * 2 * shape->E;
     const int64_t wstride = 2 * shape->E;
 
     // several stages: LDS-resident passes, last pass of the range first; the state ping-pongs between the
-    // output arrays and four float32 arrays behind the dW scratch
+    // output arrays and four float32 arrays behind the dW scratch (their grids count on kMaxGridX partial rows)
     std::vector<FusedPass> passes;
-    if (grouping.plain()) passes = multi_stage_plan(shape, first_stage, n_stages, activation, true, path);
+    if (grouping.plain() && row_cap == kMaxGridX)
+        passes = multi_stage_plan(shape, first_stage, n_stages, activation, true, path);
     const size_t np = passes.size();
     bool fused_ok = np > 0;
     if (np >= 2 && workspace_bytes < base_workspace_bytes(shape) + temp_bytes(shape, true)) fused_ok = false;
@@ -605,7 +647,7 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
         return (int)reducer.flush();
     }
 
-    DwReducer reducer(partials, level1, wstride, s);
+    DwReducer reducer(partials, level1, wstride, s, row_cap);
     for (int k = n_stages - 1; k >= 0; --k) {
         float* region;
         hipError_t err = reducer.reserve(p.partial_rows + extra_rows, 1, &region);
@@ -672,6 +714,23 @@ int ncn_backward(const void* y, const void* ya, int y_dtype, const void* dy, con
     return backward_impl(y, ya, y_dtype, dy, dya, dy_dtype, dx, dxa, dx_dtype, x_rec, xa_rec, W, dW, workspace,
                          workspace_bytes, Grouping{nullptr, nullptr}, shape, first_stage, n_stages, alpha, m, activation,
                          stream);
+}
+
+size_t ncn_static_scratch_bytes(void) { return kStaticScratchFloats * sizeof(float); }
+
+int ncn_backward_static(const void* y, const void* ya, int y_dtype, const void* dy, const void* dya, int dy_dtype,
+                        void* dx, void* dxa, int dx_dtype, float* x_rec, float* xa_rec, const float* W, float* dW,
+                        const ncn_shape* shape, int first_stage, int n_stages, float alpha, float m, int activation,
+                        void* stream) {
+    int rc = check_shape(shape, first_stage, n_stages, activation);
+    if (rc != NCN_OK) return rc;
+    if (2 * shape->E > kStaticMaxTwoE) return NCN_ERR_STATIC_LIMIT;
+    float* scratch = nullptr;
+    const hipError_t err = static_scratch(&scratch);
+    if (err != hipSuccess) return (int)err;
+    return backward_impl(y, ya, y_dtype, dy, dya, dy_dtype, dx, dxa, dx_dtype, x_rec, xa_rec, W, dW, scratch,
+                         partial_buffer_bytes(shape, kStaticRowCap), Grouping{nullptr, nullptr}, shape, first_stage,
+                         n_stages, alpha, m, activation, stream, kStaticRowCap);
 }
 
 int ncn_backward_indexed(const void* y, const void* ya, int y_dtype, const void* dy, const void* dya, int dy_dtype,

@@ -1,0 +1,88 @@
+"""ncn_backward_static: the backward without workspace argument or allocation, against ncn_backward.
+
+Two calls in a row through the C ABI, the second on a smaller problem: the library's own scratch keeps what the first
+call left there, and nothing of it may leak into the second result."""
+import ctypes
+
+import pytest
+import torch
+
+from oracle import ncn_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _call_both(lib, _lib, shape5, n_stages, seed, dtype=torch.float32):
+    batch, N, E, C, n = shape5
+    x, xa, Ws, dy, dya = O.make_inputs(batch, N, E, n_stages, n, seed=seed, xa_zero=False)
+    dev = torch.device("cuda:0")
+    W = torch.stack(Ws).to(dev)
+    sh = _lib.NcnShape(batch, N, E, C, n)
+    f32 = torch.float32
+    # outputs of the stages: the saved tensors a backward starts from (float32, as the autograd node keeps them)
+    y, ya = x.to(dev), xa.to(dev)
+    for l in range(n_stages):
+        y2, ya2 = torch.empty_like(y), torch.empty_like(ya)
+        rc = lib.ncn_forward(y.data_ptr(), ya.data_ptr(), 0, y2.data_ptr(), ya2.data_ptr(), 0, None, None,
+                             W[l].data_ptr(), None, 0, ctypes.byref(sh), l, 1, 0.9, 0.9, 0, None)
+        assert rc == 0
+        y, ya = y2, ya2
+    gdy, gdya = dy.to(dev).to(dtype), dya.to(dev).to(dtype)
+    code = 0 if dtype == f32 else 1
+    gcode = code if n_stages == 1 else 0
+
+    def outputs():
+        gd = dtype if n_stages == 1 else f32
+        return (torch.full((batch, N, E), float("nan"), device=dev, dtype=gd), torch.full((batch, N, E), float("nan"), device=dev, dtype=gd),
+                torch.full((batch, N, E), float("nan"), device=dev), torch.full((batch, N, E), float("nan"), device=dev),
+                torch.full((n_stages, 2 * E), float("nan"), device=dev))
+
+    ws_bytes = lib.ncn_workspace_bytes(ctypes.byref(sh))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    a = outputs()
+    rc = lib.ncn_backward(y.data_ptr(), ya.data_ptr(), 0, gdy.data_ptr(), gdya.data_ptr(), code, a[0].data_ptr(), a[1].data_ptr(),
+                          gcode, a[2].data_ptr(), a[3].data_ptr(), W.data_ptr(), a[4].data_ptr(), ws.data_ptr(),
+                          ctypes.c_size_t(ws_bytes), ctypes.byref(sh), 0, n_stages, 0.9, 0.9, 0, None)
+    assert rc == 0, _lib.error_string(rc)
+    b = outputs()
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()
+    rc = lib.ncn_backward_static(y.data_ptr(), ya.data_ptr(), 0, gdy.data_ptr(), gdya.data_ptr(), code, b[0].data_ptr(),
+                                 b[1].data_ptr(), gcode, b[2].data_ptr(), b[3].data_ptr(), W.data_ptr(), b[4].data_ptr(),
+                                 ctypes.byref(sh), 0, n_stages, 0.9, 0.9, 0, None)
+    assert rc == 0, _lib.error_string(rc)
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() == before
+    return a, b
+
+
+def test_backward_static_matches_backward_on_two_calls_in_a_row():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from ncn_cuda_amd import _lib
+    lib = _lib.load()
+    assert 0 < lib.ncn_static_scratch_bytes() <= 16 << 20
+    # first call: more tiles than the scratch has partial rows (a persistent loop over 4096 blocks), bf16 gradients
+    a, b = _call_both(lib, _lib, (24, 4096, 128, 4, 16), 1, seed=3, dtype=torch.bfloat16)
+    for u, v in zip(a[:4], b[:4]):
+        assert torch.equal(u, v)                         # dx, dxa, x_rec, xa_rec do not depend on the grid
+    assert O.rel_err(b[4], a[4]) < 1e-5 and torch.isfinite(b[4]).all()   # the same terms summed over fewer partial rows
+    # second call, smaller, three stages: what the first call left in the scratch must not show
+    a, b = _call_both(lib, _lib, (2, 96, 32, 4, 4), 3, seed=4)
+    for u, v in zip(a, b):
+        assert torch.isfinite(v).all() and O.rel_err(v, u) < 1e-5
+    # generic kernels (n_cache = 3) use the scratch too
+    a, b = _call_both(lib, _lib, (2, 36, 20, 2, 3), 1, seed=5)
+    for u, v in zip(a, b):
+        assert torch.isfinite(v).all() and O.rel_err(v, u) < 1e-5
+
+
+def test_backward_static_rejects_what_its_scratch_cannot_hold():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from ncn_cuda_amd import _lib
+    lib = _lib.load()
+    sh = _lib.NcnShape(1, 16, 512, 4, 4)                  # E = 512: a partial row of 1024 floats
+    p = ctypes.c_void_p(4096)                             # never dereferenced: the size check comes first
+    rc = lib.ncn_backward_static(p, p, 0, p, p, 0, p, p, 0, None, None, p, p, ctypes.byref(sh), 0, 1, 0.9, 0.9, 0, None)
+    assert rc == -9 and "scratch" in _lib.error_string(rc)
