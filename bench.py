@@ -10,10 +10,15 @@ already resident in HBM.  The default workload is the configuration the metric i
 B=16384, D=4096, g=16, bf16 storage / float32 arithmetic, i.e. [batch=128, N=4096, E=128],
 4 heads of 32, n_cache=16, 3 stages.
 
-Prints ONE JSON line.  `roofline` describes the dominant kernel (the backward stage kernel):
-algorithmic bytes of one launch divided by its average duration, measured with HIP events on the
-launch stream inside the timed region.  `cpu_baseline` times the checker's plain C restatement (and, beside it,
-the PyTorch one) on a bounded batch slice of the same workload on the host cores.
+Prints ONE JSON line.  `roofline` describes the dominant kernel (the backward stage kernel, or the
+backward call over a segment of stages where several stages run per launch) against the roof that binds
+it: float32 vector arithmetic for groups of 8 rows and more (each element takes n_cache sequential tanh
+steps per stage), HBM bandwidth for smaller groups.  Its duration is measured with HIP events on the
+launch stream inside the timed region; the figures for the other roof ride along as hbm_* / valu_*.
+`roofline.traffic` is read from profiles/traffic.json (rocprofv3 FETCH_SIZE + WRITE_SIZE of that kernel,
+recorded for one library version) and is null when that file has no entry for this library version.
+`cpu_baseline` times the checker's plain C restatement (and, beside it, the PyTorch one) on a bounded
+batch slice of the same workload on the host cores.
 """
 import argparse
 import json
@@ -34,16 +39,29 @@ CONFIGS = {
     "cfg5": dict(batch=64, N=2048, E=128, C=4, n=8, L=4, dtype="f32", w_scale=0.1),
 }
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
-VALU_PEAK_TFLOPS = 157.3   # MI355X FP32 vector peak (packed); 78.6 without packed FP32
+VALU_PEAK_TFLOPS = 157.3   # MI355X FP32 vector peak, which counts packed FP32 instructions
+VALU_PEAK_TFLOPS_UNPACKED = 78.6   # the same without them (this build does not use packed FP32)
 # float32 operations per element and step of the kernels as written in ncn_stage_kernels.h (FMA = 2, exp2 and
-# rcp = 1 each), without the per-row and per-lane bookkeeping: forward 1 FMA (dot) + 2 (z) + 1 (t+1) + 2 FMA (xa)
-# + 2 (x) + exp2 + rcp = 13; backward 11 FMA + 4 mul/add + exp2 + rcp = 28.
-# HBM bytes of one backward-stage launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (calibrated on a
-# 1 GiB copy; see profiles/stage_kernels_cfg3.md); for cfg4 the three passes of one backward call over the 13 stages
-# (profiles/fused_kernels_cfg4.md: 7.19 GB read + 6.46 GB written).
-MEASURED_BWD_TRAFFIC_BYTES = {"cfg3": 1.1128e9, "cfg4": 13.65e9}
+# rcp = 1 each), without the per-row and per-lane bookkeeping: forward 5 FMA (row sum, z, two for xa, x) + the
+# +1 before the reciprocal + exp2 + rcp = 13; backward 12 FMA (inversion of x, row sum, z, two for xa, F'/4, the
+# row's <U, x_j>, the pivot row's sum, two for G, dWi, P) + the +1 + P F'/4 + exp2 + rcp = 28.
 FLOPS_FWD_PER_ELEM_STEP = 13.0
 FLOPS_BWD_PER_ELEM_STEP = 28.0
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
+
+
+def measured_traffic(config, grouping, version):
+    """HBM bytes per launch (or per backward call over a segment) of the dominant kernel, from the profile record of
+    this library version; None when there is none."""
+    try:
+        with open(TRAFFIC_FILE) as fh:
+            rec = json.load(fh)
+    except (OSError, ValueError):
+        return None
+    entry = rec.get("entries", {}).get(f"{config}/{grouping}")
+    if not entry or entry.get("ncn_version") != version:
+        return None
+    return entry.get("bytes")
 
 
 def main():
@@ -127,8 +145,9 @@ def main():
                                                       group_index=tables[a], ctx_len=lens, check_tables=False)
                 saved.append((y32, ya32))
             elif bf16 and cnt == 1:
-                cx, cxa, y32, ya32 = M.forward_stages(cx, cxa, Wst[a], alpha, 0, n, C, a, 1, save_fp32=True)
-                saved.append((y32, ya32))
+                # bf16 outputs plus what their rounding took away (a second bf16 plane): what the backward inverts
+                cx, cxa, ys, yas = M.forward_stages(cx, cxa, Wst[a], alpha, 0, n, C, a, 1, save_residual=True)
+                saved.append((ys, yas))
             else:
                 cx, cxa = M.forward_stages(cx, cxa, Wst[a:a + cnt], alpha, 0, n, C, a, cnt, out_dtype=torch.float32)
                 saved.append((cx, cxa))
@@ -163,13 +182,18 @@ def main():
         step()
     torch.cuda.synchronize()
     events = []
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    marks[0].record()
+    for k in range(args.steps):
         out = step(events)
+        marks[k + 1].record()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / args.steps
     value = tokens / (ms_per_step * 1e-3)
+    per_step_ms = sorted(marks[k].elapsed_time(marks[k + 1]) for k in range(args.steps))
+    median_step_ms = per_step_ms[len(per_step_ms) // 2]
 
     # what a plain device-to-device copy reaches on this GPU (reads 1 GiB and writes 1 GiB per copy): quoted beside
     # the published 8 TB/s peak, outside the timed region
@@ -222,13 +246,39 @@ def main():
     # stay per stage launch there)
     lds_passes = save_every > 1 and n in (2, 4)
     bracket_ms = sum(e0.elapsed_time(e1) for e0, e1, _ in events)
-    bwd_ms = bracket_ms / len(events) if lds_passes else bracket_ms / sum(cnt for _, _, cnt in events)
+    stages_in_brackets = sum(cnt for _, _, cnt in events)
+    bwd_ms = bracket_ms / len(events) if lds_passes else bracket_ms / stages_in_brackets
+    stages_per_unit = stages_in_brackets / len(events) if lds_passes else 1.0
+    # saved outputs of a stage are read as 4 bytes per value in either storage (float32, or two bf16 planes)
     bytes_bwd_launch = 6.0 * P * (sbytes if save_every == 1 else 4)   # read y, ya, dy, dya; write dx, dxa
-    achieved = bytes_bwd_launch / (bwd_ms * 1e-3) / 1e9
+    hbm_achieved = bytes_bwd_launch / (bwd_ms * 1e-3) / 1e9
     elem_steps_stage = float(P) * n
+    flops_bwd_unit = FLOPS_BWD_PER_ELEM_STEP * elem_steps_stage * stages_per_unit
+    valu_achieved = flops_bwd_unit / (bwd_ms * 1e-3) / 1e12
     flops_step = (FLOPS_FWD_PER_ELEM_STEP + FLOPS_BWD_PER_ELEM_STEP) * elem_steps_stage * L
+    # which roof binds the dominant kernel: at the two peaks, n_cache tanh steps per element cost more time than its
+    # bytes from 8 rows per group on (one launch per stage); the multi-stage passes of small groups are built to be
+    # limited by their HBM round trips
+    valu_bound = n >= 8
+    version = M._lib.load().ncn_version().decode()
+    kernel = (f"stage_backward_kernel<{n},{E // C}>" + (" (indexed build)" if tables else "") if not lds_passes else
+              f"backward call over a segment of up to {save_every} stages (multi-stage passes)")
+    roof = {"bound": "fp32_valu" if valu_bound else "hbm",
+            "achieved": valu_achieved if valu_bound else hbm_achieved,
+            "peak": VALU_PEAK_TFLOPS if valu_bound else HBM_PEAK_GBS,
+            "unit": "TFLOP/s" if valu_bound else "GB/s",
+            "frac": (valu_achieved / VALU_PEAK_TFLOPS) if valu_bound else (hbm_achieved / HBM_PEAK_GBS),
+            "traffic": measured_traffic(args.config, args.grouping, version),
+            "kernel": kernel, "avg_launch_ms": bwd_ms,
+            "algorithmic_flops_per_launch": flops_bwd_unit,
+            "algorithmic_bytes_per_launch": bytes_bwd_launch,
+            "valu_achieved_TFLOPs": valu_achieved, "valu_frac_of_packed_peak": valu_achieved / VALU_PEAK_TFLOPS,
+            "valu_frac_of_unpacked_peak": valu_achieved / VALU_PEAK_TFLOPS_UNPACKED,
+            "hbm_achieved_GBps": hbm_achieved, "hbm_frac": hbm_achieved / HBM_PEAK_GBS,
+            "attainable_copy_GBps": copy_gbps, "hbm_frac_of_attainable_copy": hbm_achieved / copy_gbps,
+            "ncn_version": version}
     result = {
-        "metric": "NCN fwd+bwd tokens/sec and achieved HBM GB/s (% roofline), B=16384 D=4096 g=16",
+        "metric": f"NCN fwd+bwd tokens/sec and achieved HBM GB/s (% roofline), B={tokens} D={N} g={n}",
         "value": value,
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -244,25 +294,19 @@ def main():
                                f"{C} heads of {E // C}, n_cache={n}, {L} stages, alpha=0.9, m=0.9, tanh, "
                                f"{cfg['dtype']} storage, outputs saved every {save_every} stage(s), "
                                f"grouping {args.grouping}", "positions_per_s": batch * N / (ms_per_step * 1e-3)},
-        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_BWD_TRAFFIC_BYTES.get(args.config) if args.grouping == "closed" else None,
-                     "kernel": (f"stage_backward_kernel<{n},{E // C}>" + (" (indexed build)" if tables else "")
-                                if not lds_passes else
-                                f"backward call over a segment of up to {save_every} stages (multi-stage passes)"),
-                     "avg_launch_ms": bwd_ms,
-                     "attainable_copy_GBps": copy_gbps, "frac_of_attainable_copy": achieved / copy_gbps,
-                     "algorithmic_bytes_per_launch": bytes_bwd_launch},
-        "stack": {"algorithmic_bytes_fused": 10.0 * P * sbytes,
+        "roofline": roof,
+        "stack": {"median_ms_per_step": median_step_ms,
+                  "min_ms_per_step": per_step_ms[0], "max_ms_per_step": per_step_ms[-1],
+                  "algorithmic_bytes_fused": 10.0 * P * sbytes,
                   "achieved_GBps_fused_bytes": 10.0 * P * sbytes / (ms_per_step * 1e-3) / 1e9,
                   "algorithmic_bytes_per_stage_launches": 10.0 * P * sbytes * L,
                   "achieved_GBps_per_stage_bytes": 10.0 * P * sbytes * L / (ms_per_step * 1e-3) / 1e9,
                   "fp32_flops_per_step": flops_step,
                   "achieved_TFLOPs": flops_step / (ms_per_step * 1e-3) / 1e12,
                   "frac_of_fp32_vector_peak": flops_step / (ms_per_step * 1e-3) / 1e12 / VALU_PEAK_TFLOPS,
+                  "frac_of_fp32_vector_peak_unpacked": flops_step / (ms_per_step * 1e-3) / 1e12 / VALU_PEAK_TFLOPS_UNPACKED,
                   "inverse_ms_per_stack": inverse_ms,
-                  "inverse_reconstruction_rel_err": recon_err if inverse_ms is not None else None,
-                  "note": "the step is bound by float32 VALU + exp2/rcp issue, not by HBM or MFMA: "
-                          "each element takes n_cache sequential tanh steps per stage"},
+                  "inverse_reconstruction_rel_err": recon_err if inverse_ms is not None else None},
     }
 
     if not args.no_cpu:

@@ -40,6 +40,14 @@ extern "C" {
 /* element types of activation / gradient buffers */
 #define NCN_F32 0
 #define NCN_BF16 1
+/* A value kept as two bfloat16: buffer [2, batch, N, E], plane 0 = the value rounded to bfloat16, plane 1 = what
+ * the rounding took away, rounded to bfloat16 again (16 significant bits in all).  What a bf16 caller saves for the
+ * reversible backward: plane 0 alone is the ordinary bf16 tensor [batch, N, E] (the next stage reads it as NCN_BF16),
+ * so a forward writes 4 bytes per value instead of the 2 + 4 of a bf16 output plus a float32 copy.  Accepted as
+ * out_dtype of ncn_forward / ncn_forward_indexed, y_dtype of ncn_backward / ncn_backward_indexed / ncn_backward_static
+ * and in_dtype of ncn_inverse / ncn_inverse_indexed, for one stage per call (n_stages == 1) on the register kernels
+ * (ncn_kernel_path() == 2); NCN_ERR_DTYPE elsewhere. */
+#define NCN_BF16X2 2
 
 /* activation codes: those of the reference's CUDA surface (ncn_pytorch_wrapper_v2.py:111,
  * ncn_fwd_cuda_kernel.cu:86-95): 0 tanh, 1 relu, 2 sigmoid, anything else the reference treats as
@@ -274,6 +282,11 @@ int ncn_plan_passes(const ncn_shape* shape, int first_stage, int n_stages, int a
 /* 2: hand-tuned register kernel, 1: generic LDS kernel, 0: not supported (n_cache > 64, or the
  * head width does not fit the generic kernel's LDS).  No reference counterpart. */
 int ncn_kernel_path(const ncn_shape* shape);
+
+/* The same for a call with these scalars: the register kernels carry their state times alpha and 1 - m, so values
+ * of alpha or 1 - m next to zero (below 1e-3) run on the generic kernels (1), or nowhere (0) when the head is wider
+ * than those take. */
+int ncn_kernel_path_scalars(const ncn_shape* shape, float alpha, float m);
 
 /* Validates arguments exactly as the entry points do, without touching the GPU.  Returns NCN_OK or
  * the error the corresponding call would return before launching.  No reference counterpart (the

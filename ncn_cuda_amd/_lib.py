@@ -8,13 +8,13 @@ import os
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG_DIR, "libncn_hip.so")
 
-NCN_F32, NCN_BF16 = 0, 1
+NCN_F32, NCN_BF16, NCN_BF16X2 = 0, 1, 2
 ACT_TANH, ACT_RELU, ACT_SIGMOID, ACT_LEAKY_RELU, ACT_LINEAR = 0, 1, 2, 3, -1
 
 EXPORTS = ("ncn_forward", "ncn_backward", "ncn_inverse", "ncn_forward_indexed", "ncn_backward_indexed",
            "ncn_inverse_indexed", "ncn_forward_radix", "ncn_backward_radix", "ncn_inverse_radix", "ncn_plan_radix", "ncn_workspace_bytes", "ncn_workspace_bytes_stages",
            "ncn_plan_passes", "ncn_kernel_path",
-           "ncn_check_shape", "ncn_error_string", "ncn_version", "ncn_backward_static", "ncn_static_scratch_bytes")
+           "ncn_check_shape", "ncn_error_string", "ncn_version", "ncn_backward_static", "ncn_static_scratch_bytes", "ncn_kernel_path_scalars")
 
 
 class NcnShape(ctypes.Structure):
@@ -72,6 +72,8 @@ def load():
     lib.ncn_plan_passes.argtypes = [shp, i, i, i, i, ctypes.POINTER(ctypes.c_int32), i]
     lib.ncn_kernel_path.restype = i
     lib.ncn_kernel_path.argtypes = [shp]
+    lib.ncn_kernel_path_scalars.restype = i
+    lib.ncn_kernel_path_scalars.argtypes = [shp, fl, fl]
     lib.ncn_check_shape.restype = i
     lib.ncn_check_shape.argtypes = [shp, i, i, i]
     lib.ncn_error_string.restype = ctypes.c_char_p

@@ -63,16 +63,18 @@ def radix_group_table(N, n_cache, level, device=None):
 
 class FusedLinearChunkNCNFunction(torch.autograd.Function):
     """Autograd node of one table-grouped stage (ncn_triton_old.py:287-357): saves the outputs and inverts them in
-    backward."""
+    backward.  bfloat16 outputs are saved with what their rounding took away (two bfloat16 planes, or float32 copies
+    on the generic kernels): the inversion would amplify bare bfloat16 rounding by (1/m)^n_cache."""
 
     @staticmethod
     def forward(ctx, x, xa, W, group_tensor, ctxlen_tensor, ALPHA, ACTIVATION, NUM_HEADS, CACHE, l):
         code = _activation_code(ACTIVATION)
-        yi, ya = ncn_cuda_module.forward_stages(x, xa, W, ALPHA, code, CACHE, NUM_HEADS, 0, 1,
-                                                group_index=group_tensor, ctx_len=ctxlen_tensor)
-        ctx.save_for_backward(yi, ya, W)
+        yi, ya, sy, sya = ncn_cuda_module.forward_stages_saving(x, xa, W, ALPHA, code, CACHE, NUM_HEADS, 0,
+                                                                group_index=group_tensor, ctx_len=ctxlen_tensor)
+        ctx.save_for_backward(sy, sya, W)
         ctx.group_tensor, ctx.ctxlen_tensor = group_tensor, ctxlen_tensor
         ctx.args = (ALPHA, code, CACHE, NUM_HEADS)
+        ctx.io_dtype = x.dtype
         return yi, ya
 
     @staticmethod
@@ -81,7 +83,8 @@ class FusedLinearChunkNCNFunction(torch.autograd.Function):
         alpha, code, cache, heads = ctx.args
         _, _, dx, dxa, dW = ncn_cuda_module.backward_stages(
             yi, ya, dyi.contiguous(), dya.contiguous() if dya is not None else None, W, alpha, code, cache, heads, 0, 1,
-            want_inputs=False, group_index=ctx.group_tensor, ctx_len=ctx.ctxlen_tensor, check_tables=False)
+            grad_dtype=ctx.io_dtype, want_inputs=False, group_index=ctx.group_tensor, ctx_len=ctx.ctxlen_tensor,
+            check_tables=False)
         return dx, dxa, dW.reshape(W.shape).to(W.dtype), None, None, None, None, None, None, None
 
 

@@ -16,6 +16,8 @@ bool known_activation(int a) {
     return a == NCN_ACT_TANH || a == NCN_ACT_RELU || a == NCN_ACT_SIGMOID || a == NCN_ACT_LEAKY_RELU || a == NCN_ACT_LINEAR;
 }
 bool known_dtype(int d) { return d == NCN_F32 || d == NCN_BF16; }
+// the arguments that also take a value kept as two bfloat16 planes (one stage per call, register kernels)
+bool known_dtype_or_x2(int d, int n_stages, int path) { return known_dtype(d) || (d == NCN_BF16X2 && n_stages == 1 && path == 2); }
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // 2 = register kernels, 1 = generic LDS kernels, 0 = unsupported
@@ -193,6 +195,7 @@ void fill_common(StageArgs& a, const ncn_shape* sh, const Plan& p, int stage, fl
     a.radix_stride = g.radix_first >= 0 ? upow((uint32_t)sh->n_cache, g.radix_first + rel_stage) : 0u;
     a.N = sh->N;
     a.E = sh->E;
+    a.plane = sh->batch * sh->N * sh->E;
     a.total_tiles = p.total_tiles;
     a.tiles_per_inst = p.tiles_per_inst;
     a.groups = p.groups;
@@ -337,7 +340,7 @@ hipError_t static_scratch(float** out) {
 
 extern "C" {
 
-const char* ncn_version(void) { return "0.4"; }
+const char* ncn_version(void) { return "0.5"; }
 
 int ncn_plan_passes(const ncn_shape* shape, int first_stage, int n_stages, int activation, int backward, int32_t* out,
                     int max_passes) {
@@ -362,7 +365,7 @@ const char* ncn_error_string(int code) {
         case NCN_OK: return "ok";
         case NCN_ERR_NULL: return "a required pointer is NULL";
         case NCN_ERR_SHAPE: return "bad shape: sizes must be positive, N % n_cache == 0, E % n_head == 0, n_stages >= 1";
-        case NCN_ERR_DTYPE: return "unknown element type (0 = float32, 1 = bfloat16)";
+        case NCN_ERR_DTYPE: return "unknown element type (0 = float32, 1 = bfloat16; 2 = two bfloat16 planes, only for the saved outputs of one stage on the register kernels)";
         case NCN_ERR_ACTIVATION: return "unknown activation code (0 tanh, 1 relu, 2 sigmoid, 3 leaky relu, -1 linear)";
         case NCN_ERR_WORKSPACE: return "workspace is NULL or smaller than ncn_workspace_bytes()";
         case NCN_ERR_UNSUPPORTED: return "unsupported shape: n_cache must be <= 64 and the head width <= 64 (128 for power-of-two n_cache <= 16)";
@@ -384,6 +387,10 @@ int ncn_kernel_path(const ncn_shape* shape) {
         return 0;
     if (shape->E % shape->n_head != 0) return 0;
     return kernel_path(shape, NCN_ACT_TANH);
+}
+
+int ncn_kernel_path_scalars(const ncn_shape* shape, float alpha, float m) {
+    return ncn_kernel_path(shape) ? kernel_path_for(shape, NCN_ACT_TANH, alpha, m) : 0;
 }
 
 size_t ncn_workspace_bytes(const ncn_shape* shape) {
@@ -408,12 +415,12 @@ static int forward_impl(const void* x, const void* xa, int in_dtype, void* y, vo
     if (rc != NCN_OK) return rc;
     if (!x || !xa || !y || !ya || !W) return NCN_ERR_NULL;
     if ((y32 == nullptr) != (ya32 == nullptr)) return NCN_ERR_NULL;
-    if (!known_dtype(in_dtype) || !known_dtype(out_dtype)) return NCN_ERR_DTYPE;
+    const int path = kernel_path_for(shape, activation, alpha, m);
+    if (path == 0) return NCN_ERR_UNSUPPORTED;
+    if (!known_dtype(in_dtype) || !known_dtype_or_x2(out_dtype, n_stages, path)) return NCN_ERR_DTYPE;
     if (!aligned16(x) || !aligned16(xa) || !aligned16(y) || !aligned16(ya) || !aligned16(W) || !aligned16(y32) ||
         !aligned16(ya32) || !aligned16(workspace))
         return NCN_ERR_ALIGN;
-    const int path = kernel_path_for(shape, activation, alpha, m);
-    if (path == 0) return NCN_ERR_UNSUPPORTED;
     const Plan p = make_plan(shape, path);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int64_t wstride = 2 * shape->E;
@@ -495,10 +502,10 @@ static int inverse_impl(const void* y, const void* ya, int in_dtype, void* x, vo
     rc = check_grouping(grouping, shape);
     if (rc != NCN_OK) return rc;
     if (!x || !xa || !y || !ya || !W) return NCN_ERR_NULL;
-    if (!known_dtype(in_dtype) || !known_dtype(out_dtype)) return NCN_ERR_DTYPE;
-    if (!aligned16(x) || !aligned16(xa) || !aligned16(y) || !aligned16(ya) || !aligned16(W)) return NCN_ERR_ALIGN;
     const int path = kernel_path_for(shape, activation, alpha, m);
     if (path == 0) return NCN_ERR_UNSUPPORTED;
+    if (!known_dtype_or_x2(in_dtype, n_stages, path) || !known_dtype(out_dtype)) return NCN_ERR_DTYPE;
+    if (!aligned16(x) || !aligned16(xa) || !aligned16(y) || !aligned16(ya) || !aligned16(W)) return NCN_ERR_ALIGN;
     const Plan p = make_plan(shape, path);
     hipStream_t s = static_cast<hipStream_t>(stream);
 
@@ -570,15 +577,15 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
     if (rc != NCN_OK) return rc;
     if (!y || !ya || !dy || !dx || !dxa || !W || !dW) return NCN_ERR_NULL;
     if ((x_rec == nullptr) != (xa_rec == nullptr)) return NCN_ERR_NULL;
-    if (!known_dtype(y_dtype) || !known_dtype(dy_dtype) || !known_dtype(dx_dtype)) return NCN_ERR_DTYPE;
+    const int path = kernel_path_for(shape, activation, alpha, m);
+    if (path == 0) return NCN_ERR_UNSUPPORTED;
+    if (!known_dtype_or_x2(y_dtype, n_stages, path) || !known_dtype(dy_dtype) || !known_dtype(dx_dtype)) return NCN_ERR_DTYPE;
     if (n_stages > 1 && (!x_rec || dx_dtype != NCN_F32)) return NCN_ERR_ALIAS;
     if (!workspace || workspace_bytes < partial_buffer_bytes(shape, row_cap)) return NCN_ERR_WORKSPACE;
     if (!aligned16(y) || !aligned16(ya) || !aligned16(dy) || !aligned16(dya) || !aligned16(dx) || !aligned16(dxa) ||
         !aligned16(x_rec) || !aligned16(xa_rec) || !aligned16(W) || !aligned16(dW) || !aligned16(workspace))
         return NCN_ERR_ALIGN;
     // partial rows of the generic kernel's second launch
-    const int path = kernel_path_for(shape, activation, alpha, m);
-    if (path == 0) return NCN_ERR_UNSUPPORTED;
     const int extra_rows = (grouping.ctx_len && path != 2) ? edge_rows(shape) : 0;
     const Plan p = make_plan(shape, path, extra_rows, row_cap);
     hipStream_t s = static_cast<hipStream_t>(stream);

@@ -61,6 +61,7 @@ struct StageArgs {
     const int32_t* table;    // [N] slot -> position, or null
     const int32_t* ctx_len;  // [batch] live slots per batch entry, or null
     int64_t N, E;
+    int64_t plane;            // batch * N * E: elements between the two planes of an NCN_BF16X2 buffer
     uint32_t total_tiles;     // batch * tiles_per_instance
     uint32_t tiles_per_inst;  // ceil(groups / groups-per-wave-tile)
     uint32_t groups;          // N / n_cache
@@ -95,8 +96,10 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 }
 
 // Row fragment of FPL consecutive features, element offset `off` into a buffer of type `dtype`.
+// NCN_BF16X2: the value is the sum of the two planes, `plane` elements apart.
 template <int FPL>
-__device__ __forceinline__ void load_frag(const void* base, int dtype, int64_t off, bool valid, float (&v)[FPL]) {
+__device__ __forceinline__ void load_frag(const void* base, int dtype, int64_t off, bool valid, float (&v)[FPL],
+                                          int64_t plane = 0) {
     static_assert(FPL % 4 == 0, "fragment must be a multiple of 4 features");
     if (!valid) {
 #pragma unroll
@@ -118,11 +121,21 @@ __device__ __forceinline__ void load_frag(const void* base, int dtype, int64_t o
             v[4 * k + 0] = bf16_to_f32(t.x & 0xffffu); v[4 * k + 1] = bf16_to_f32(t.x >> 16);
             v[4 * k + 2] = bf16_to_f32(t.y & 0xffffu); v[4 * k + 3] = bf16_to_f32(t.y >> 16);
         }
+        if (dtype == NCN_BF16X2) {
+            const uint2* q = reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(base) + off + plane);
+#pragma unroll
+            for (int k = 0; k < FPL / 4; ++k) {
+                uint2 t = q[k];
+                v[4 * k + 0] += bf16_to_f32(t.x & 0xffffu); v[4 * k + 1] += bf16_to_f32(t.x >> 16);
+                v[4 * k + 2] += bf16_to_f32(t.y & 0xffffu); v[4 * k + 3] += bf16_to_f32(t.y >> 16);
+            }
+        }
     }
 }
 
 template <int FPL>
-__device__ __forceinline__ void store_frag(void* base, int dtype, int64_t off, bool valid, const float (&v)[FPL]) {
+__device__ __forceinline__ void store_frag(void* base, int dtype, int64_t off, bool valid, const float (&v)[FPL],
+                                           int64_t plane = 0) {
     if (!valid) return;
     if (dtype == NCN_F32) {
         float4* p = reinterpret_cast<float4*>(static_cast<float*>(base) + off);
@@ -136,18 +149,31 @@ __device__ __forceinline__ void store_frag(void* base, int dtype, int64_t off, b
             t.x = pack_bf16x2(v[4 * k + 0], v[4 * k + 1]);
             t.y = pack_bf16x2(v[4 * k + 2], v[4 * k + 3]);
             p[k] = t;
+            if (dtype == NCN_BF16X2) {   // second plane: what the rounding took away (the difference is exact in float32)
+                uint2 u;
+                u.x = pack_bf16x2(v[4 * k + 0] - bf16_to_f32(t.x & 0xffffu), v[4 * k + 1] - bf16_to_f32(t.x >> 16));
+                u.y = pack_bf16x2(v[4 * k + 2] - bf16_to_f32(t.y & 0xffffu), v[4 * k + 3] - bf16_to_f32(t.y >> 16));
+                reinterpret_cast<uint2*>(static_cast<uint16_t*>(base) + off + plane)[k] = u;
+            }
         }
     }
 }
 
-__device__ __forceinline__ float load_elem(const void* base, int dtype, int64_t off) {
+__device__ __forceinline__ float load_elem(const void* base, int dtype, int64_t off, int64_t plane = 0) {
     if (dtype == NCN_F32) return static_cast<const float*>(base)[off];
-    return bf16_to_f32(static_cast<const uint16_t*>(base)[off]);
+    const uint16_t* p = static_cast<const uint16_t*>(base);
+    return dtype == NCN_BF16X2 ? bf16_to_f32(p[off]) + bf16_to_f32(p[off + plane]) : bf16_to_f32(p[off]);
 }
 
-__device__ __forceinline__ void store_elem(void* base, int dtype, int64_t off, float v) {
-    if (dtype == NCN_F32) static_cast<float*>(base)[off] = v;
-    else static_cast<uint16_t*>(base)[off] = static_cast<uint16_t>(f32_to_bf16(v));
+__device__ __forceinline__ void store_elem(void* base, int dtype, int64_t off, float v, int64_t plane = 0) {
+    if (dtype == NCN_F32) {
+        static_cast<float*>(base)[off] = v;
+    } else {
+        uint16_t* p = static_cast<uint16_t*>(base);
+        const uint32_t hi = f32_to_bf16(v);
+        p[off] = static_cast<uint16_t>(hi);
+        if (dtype == NCN_BF16X2) p[off + plane] = static_cast<uint16_t>(f32_to_bf16(v - bf16_to_f32(hi)));
+    }
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -242,13 +242,13 @@ __global__ void __launch_bounds__(256) pass_through_kernel(const StageArgs A, co
         const int64_t pos = slot_position(A, (uint32_t)(k / A.n_cache), (uint32_t)(k % A.n_cache));
         const int64_t off = ((int64_t)b * A.N + pos) * A.E;
         for (int64_t e = lane; e < A.E; e += 64) {
-            const float v0 = load_elem(A.in0, A.in_dtype, off + e), v1 = load_elem(A.in1, A.in_dtype, off + e);
+            const float v0 = load_elem(A.in0, A.in_dtype, off + e, A.plane), v1 = load_elem(A.in1, A.in_dtype, off + e, A.plane);
             if (backward) {
                 store_elem(A.out0, A.out_dtype, off + e, load_elem(A.g0, A.g_dtype, off + e));
                 store_elem(A.out1, A.out_dtype, off + e, A.g1 ? load_elem(A.g1, A.g_dtype, off + e) : 0.f);
             } else {
-                store_elem(A.out0, A.out_dtype, off + e, v0);
-                store_elem(A.out1, A.out_dtype, off + e, v1);
+                store_elem(A.out0, A.out_dtype, off + e, v0, A.plane);
+                store_elem(A.out1, A.out_dtype, off + e, v1, A.plane);
             }
             if (A.aux0) {
                 A.aux0[off + e] = v0;

@@ -385,9 +385,17 @@ __device__ __forceinline__ void backward_steps(float (&Y)[R][F], float (&B)[R][F
     const int fl = lane % T::LF;                                                                \
     float wi[F], wj[F];                                                                         \
     load_w<F>(A.W, A.E, head, EC, fl, wi, wj);                                                  \
-    _Pragma("unroll") for (int f = 0; f < F; ++f) {                                             \
-        wi[f] *= A.tab.gamma;                                                                   \
-        wj[f] *= A.tab.gamma;                                                                   \
+    bool w_raw = true;
+
+// The weights are scaled by gamma once, after the loads of the wave's first tile have been issued: scaling them in the
+// prologue would wait for them before the tile's own loads are even on their way (one memory latency after the other).
+#define NCN_SCALE_W_ONCE                                                                        \
+    if (w_raw) {                                                                                \
+        w_raw = false;                                                                          \
+        _Pragma("unroll") for (int f = 0; f < F; ++f) {                                         \
+            wi[f] *= A.tab.gamma;                                                               \
+            wj[f] *= A.tab.gamma;                                                               \
+        }                                                                                       \
     }
 
 // Row rr of this lane is live when its slot is below the group's live rows (always, or never, without lengths).
@@ -406,14 +414,15 @@ __global__ void __launch_bounds__(kBlockThreads, (TANH_ONLY && !INDEXED && R == 
             load_frag<F>(A.in0, A.in_dtype, off[rr], valid, x[rr]);
             load_frag<F>(A.in1, A.in_dtype, off[rr], valid, a[rr]);
         }
+        NCN_SCALE_W_ONCE
         scale_tile<R, F>(x, a, A.tab.kappa, A.tab.a_scale);
         forward_core<NC, EC, R, F, TANH_ONLY, INDEXED>(x, a, wi, wj, A.tab, lane, slots, live);
         scale_tile<R, F>(x, a, A.tab.inv_kappa, A.tab.inv_a_scale);
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) {
             const bool valid = INDEXED ? NCN_ROW_LIVE(rr) : live != 0;
-            store_frag<F>(A.out0, A.out_dtype, off[rr], valid, x[rr]);
-            store_frag<F>(A.out1, A.out_dtype, off[rr], valid, a[rr]);
+            store_frag<F>(A.out0, A.out_dtype, off[rr], valid, x[rr], A.plane);
+            store_frag<F>(A.out1, A.out_dtype, off[rr], valid, a[rr], A.plane);
             if (A.aux0) {
                 store_frag<F>(A.aux0, NCN_F32, off[rr], valid, x[rr]);
                 store_frag<F>(A.aux1, NCN_F32, off[rr], valid, a[rr]);
@@ -432,9 +441,10 @@ __global__ void __launch_bounds__(kBlockThreads) stage_inverse_kernel(const Stag
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) {
             const bool valid = INDEXED ? NCN_ROW_LIVE(rr) : live != 0;
-            load_frag<F>(A.in0, A.in_dtype, off[rr], valid, y[rr]);
-            load_frag<F>(A.in1, A.in_dtype, off[rr], valid, b[rr]);
+            load_frag<F>(A.in0, A.in_dtype, off[rr], valid, y[rr], A.plane);
+            load_frag<F>(A.in1, A.in_dtype, off[rr], valid, b[rr], A.plane);
         }
+        NCN_SCALE_W_ONCE
         scale_tile<R, F>(y, b, A.tab.kappa, A.tab.b_scale);
         inverse_core<NC, EC, R, F, TANH_ONLY, INDEXED>(y, b, wi, wj, A.tab, lane, slots, live);
         scale_tile<R, F>(y, b, A.tab.inv_kappa, A.tab.inv_b_scale);
@@ -463,11 +473,12 @@ __global__ void __launch_bounds__(kBlockThreads, (TANH_ONLY && R * F <= 16 && F 
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) {
             const bool valid = INDEXED ? NCN_ROW_LIVE(rr) : live != 0;
-            load_frag<F>(A.in0, A.in_dtype, off[rr], valid, Y[rr]);
-            load_frag<F>(A.in1, A.in_dtype, off[rr], valid, B[rr]);
+            load_frag<F>(A.in0, A.in_dtype, off[rr], valid, Y[rr], A.plane);
+            load_frag<F>(A.in1, A.in_dtype, off[rr], valid, B[rr], A.plane);
             load_frag<F>(A.g0, A.g_dtype, off[rr], valid, G[rr]);
             load_frag<F>(A.g1, A.g_dtype, off[rr], valid && A.g1 != nullptr, H[rr]);
         }
+        NCN_SCALE_W_ONCE
         backward_steps<NC, EC, R, F, false, TANH_ONLY, INDEXED>(Y, B, G, H, wi, wj, dwi, dwj, 1.0f, A.tab, lane, slots,
                                                                live);
 #pragma unroll
@@ -503,6 +514,7 @@ __global__ void __launch_bounds__(kBlockThreads, (TANH_ONLY && R * F <= 16 && F 
     }
 }
 #undef NCN_ROW_LIVE
+#undef NCN_SCALE_W_ONCE
 #undef NCN_WAVE_PROLOGUE
 
 }  // namespace ncn

@@ -8,8 +8,9 @@ instead and changes nothing else.  Behavioural differences:
     are equal;
   * reset_parameters uses the stored embed_dim (the reference reads an attribute it never sets,
     ncn_pytorch_wrapper_v2.py:87-90);
-  * bfloat16 inputs are supported: the node then saves float32 copies of its outputs, because the
-    reversible backward divides by m at every step and would amplify bf16 rounding past 2e-2.
+  * bfloat16 inputs are supported: the node then saves, beside its bfloat16 outputs, what their rounding took away
+    (a second bfloat16 plane; float32 copies on the generic kernels), because the reversible backward divides by m at
+    every step and would amplify bare bf16 rounding past 2e-2.
 """
 import math
 from typing import Tuple
@@ -33,13 +34,8 @@ class NCNFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, xa, W, alpha, activation, n_cache, n_head, module_l):
-        if x.dtype == torch.float32:
-            yi, ya = ncn_cuda_module.forward_stages(x, xa, W, alpha, activation, n_cache, n_head, module_l, 1)
-            ctx.save_for_backward(yi, ya, W)
-        else:
-            yi, ya, y32, ya32 = ncn_cuda_module.forward_stages(x, xa, W, alpha, activation, n_cache, n_head,
-                                                               module_l, 1, save_fp32=True)
-            ctx.save_for_backward(y32, ya32, W)
+        yi, ya, sy, sya = ncn_cuda_module.forward_stages_saving(x, xa, W, alpha, activation, n_cache, n_head, module_l)
+        ctx.save_for_backward(sy, sya, W)
         ctx.alpha = alpha
         ctx.activation = activation
         ctx.n_cache = n_cache

@@ -146,10 +146,39 @@ def _grouping(group_index, ctx_len, batch, N, n_stages, dev, check_tables):
     return gi, cl
 
 
+def _is_two_plane(t):
+    """A value kept as two bfloat16 planes, [2, batch, N, E]: what forward_stages(save_residual=True) returns."""
+    return isinstance(t, torch.Tensor) and t.dim() == 4 and t.shape[0] == 2 and t.dtype == torch.bfloat16
+
+
+def residual_save_supported(x, n_cache, n_head, alpha=0.9, m=M_DEFAULT):
+    """True when forward_stages(save_residual=True) can run this call: the register kernels only."""
+    shape = _lib.NcnShape(x.shape[0], x.shape[1], x.shape[2], int(n_head), int(n_cache))
+    return _lib.load().ncn_kernel_path_scalars(ctypes.byref(shape), float(alpha), float(m)) == 2
+
+
+def _check_out(out, like, dtype):
+    """The caller's output tensors go to the library as they are: they must be what it will write."""
+    if not (isinstance(out, (tuple, list)) and len(out) == 2):
+        raise TypeError("out must be a pair of tensors (y, ya)")
+    for t in out:
+        if not isinstance(t, torch.Tensor):
+            raise TypeError("out must hold torch tensors")
+        if t.shape != like.shape or t.dtype != dtype or t.device != like.device:
+            raise ValueError(f"out tensors must be {tuple(like.shape)} {dtype} on {like.device}, got "
+                             f"{tuple(t.shape)} {t.dtype} on {t.device}")
+        if not t.is_contiguous() or t.data_ptr() % 16 != 0:
+            raise ValueError("out tensors must be contiguous and 16-byte aligned")
+
+
 def forward_stages(x, xa, W, alpha, activation, cache_dim, nhead, first_stage, n_stages, *, m=M_DEFAULT,
-                   out_dtype=None, save_fp32=False, out=None, group_index=None, ctx_len=None, check_tables=True):
+                   out_dtype=None, save_fp32=False, save_residual=False, out=None, group_index=None, ctx_len=None,
+                   check_tables=True):
     """Stages first_stage .. first_stage+n_stages-1 in one call.  W: [n_stages, 2E] (any shape with that many
-    values).  Returns (y, ya) or, with save_fp32, (y, ya, y32, ya32) where y32/ya32 are float32 copies.
+    values).  Returns (y, ya) or, with save_fp32, (y, ya, y32, ya32) where y32/ya32 are float32 copies, or, with
+    save_residual (bfloat16 outputs, one stage, register-kernel shapes), (y, ya, ys, yas) where ys, yas are
+    [2, batch, N, E] bfloat16: plane 0 is y (the same memory), plane 1 what its rounding took away -- what
+    backward_stages takes in place of float32 copies at two thirds of the bytes written.
     group_index [n_stages, N] replaces the stride permutation by a table of positions in (group, slot) order and
     ctx_len [batch] gives every batch entry its own number of live slots (the group_tensor / ctxlen_tensor of
     ncn_triton/ncn_triton_old.py:362-387); rows past the length pass through."""
@@ -159,7 +188,19 @@ def forward_stages(x, xa, W, alpha, activation, cache_dim, nhead, first_stage, n
     gi, cl = _grouping(group_index, ctx_len, x.shape[0], x.shape[1], n_stages, dev, check_tables)
     x, xa, w = _prep(x.detach()), _prep(xa.detach()), _w32(W)
     out_dtype = x.dtype if out_dtype is None else out_dtype
-    if out is not None:
+    if out is not None and out_dtype not in _DTYPES:
+        raise TypeError(f"out_dtype must be float32 or bfloat16, got {out_dtype}")
+    out_code = _DTYPES[out_dtype]
+    ys = yas = None
+    if save_residual:
+        if out_dtype != torch.bfloat16 or n_stages != 1 or save_fp32 or out is not None:
+            raise ValueError("save_residual needs bfloat16 outputs, one stage, and neither save_fp32 nor out")
+        ys = torch.empty((2,) + tuple(x.shape), dtype=torch.bfloat16, device=dev)
+        yas = torch.empty((2,) + tuple(x.shape), dtype=torch.bfloat16, device=dev)
+        y, ya = ys[0], yas[0]
+        out_code = _lib.NCN_BF16X2
+    elif out is not None:
+        _check_out(out, x, out_dtype)
         y, ya = out
     else:
         y = torch.empty(x.shape, dtype=out_dtype, device=dev)
@@ -176,29 +217,51 @@ def forward_stages(x, xa, W, alpha, activation, cache_dim, nhead, first_stage, n
     ws, ws_bytes = None, 0
     if indexed:
         with torch.cuda.device(dev):
-            rc = lib.ncn_forward_indexed(_ptr(x), _ptr(xa), _DTYPES[x.dtype], _ptr(y), _ptr(ya), _DTYPES[out_dtype],
+            rc = lib.ncn_forward_indexed(_ptr(x), _ptr(xa), _DTYPES[x.dtype], _ptr(y), _ptr(ya), out_code,
                                          _ptr(aux[0]), _ptr(aux[1]), _ptr(w), _ptr(gi), _ptr(cl), ctypes.byref(shape),
                                          int(first_stage), int(n_stages), float(alpha), float(m), int(activation),
                                          _stream(dev))
         _lib.check(rc, "ncn_forward_indexed")
-        return (y, ya, y32, ya32) if save_fp32 else (y, ya)
+        return (y, ya, ys, yas) if save_residual else (y, ya, y32, ya32) if save_fp32 else (y, ya)
     if n_stages > 1:
         ws_bytes = lib.ncn_workspace_bytes_stages(ctypes.byref(shape), int(first_stage), int(n_stages), int(activation), 0)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
     with torch.cuda.device(dev):
-        rc = lib.ncn_forward(_ptr(x), _ptr(xa), _DTYPES[x.dtype], _ptr(y), _ptr(ya), _DTYPES[out_dtype],
+        rc = lib.ncn_forward(_ptr(x), _ptr(xa), _DTYPES[x.dtype], _ptr(y), _ptr(ya), out_code,
                              _ptr(aux[0]), _ptr(aux[1]), _ptr(w), _ptr(ws), ctypes.c_size_t(ws_bytes),
                              ctypes.byref(shape), int(first_stage), int(n_stages), float(alpha), float(m),
                              int(activation), _stream(dev))
     _lib.check(rc, "ncn_forward")
-    return (y, ya, y32, ya32) if save_fp32 else (y, ya)
+    return (y, ya, ys, yas) if save_residual else (y, ya, y32, ya32) if save_fp32 else (y, ya)
+
+
+def forward_stages_saving(x, xa, W, alpha, activation, cache_dim, nhead, stage, *, m=M_DEFAULT, group_index=None,
+                          ctx_len=None, check_tables=True):
+    """One stage forward, and what an autograd node should keep for backward_stages: returns (y, ya, saved_y, saved_ya).
+    float32: the outputs themselves.  bfloat16: the outputs plus what their rounding took away, as two bfloat16 planes
+    on the register kernels and as float32 copies on the generic ones (a reversible backward would amplify bare
+    bfloat16 rounding by (1/m)^n_cache, 5.4x at 16 rows)."""
+    kw = dict(m=m, group_index=group_index, ctx_len=ctx_len, check_tables=check_tables)
+    if x.dtype == torch.float32:
+        y, ya = forward_stages(x, xa, W, alpha, activation, cache_dim, nhead, stage, 1, **kw)
+        return y, ya, y, ya
+    if x.dim() == 3 and residual_save_supported(x, cache_dim, nhead, alpha, m):
+        return forward_stages(x, xa, W, alpha, activation, cache_dim, nhead, stage, 1, save_residual=True, **kw)
+    return forward_stages(x, xa, W, alpha, activation, cache_dim, nhead, stage, 1, save_fp32=True, **kw)
 
 
 def backward_stages(y, ya, dy, dya, W, alpha, activation, cache_dim, nhead, first_stage, n_stages, *, m=M_DEFAULT,
                     grad_dtype=None, want_inputs=True, group_index=None, ctx_len=None, check_tables=True):
     """Reversible backward of stages first_stage+n_stages-1 .. first_stage from the outputs y, ya of the last one.
-    dya may be None (zeros).  Returns (x_rec, xa_rec, dx, dxa, dW[n_stages, 2E]); x_rec/xa_rec are None when
+    dya may be None (zeros).  y, ya may be the two-plane tensors [2, batch, N, E] of forward_stages(save_residual=True)
+    (one stage).  Returns (x_rec, xa_rec, dx, dxa, dW[n_stages, 2E]); x_rec/xa_rec are None when
     want_inputs is False and n_stages == 1."""
+    two_plane = _is_two_plane(y) and _is_two_plane(ya)
+    if two_plane and n_stages != 1:
+        raise ValueError("two-plane saved outputs hold one stage: n_stages must be 1")
+    ys_full, yas_full = y, ya
+    if two_plane:
+        y, ya = ys_full[0], yas_full[0]
     shape = validate(y, ya, W, cache_dim, nhead, activation, first_stage, n_stages, what="y")
     if dy.shape != y.shape or (dya is not None and dya.shape != y.shape):
         raise ValueError("dy/dya must have the shape of y")
@@ -207,24 +270,30 @@ def backward_stages(y, ya, dy, dya, W, alpha, activation, cache_dim, nhead, firs
     dev = _require_gpu(y, ya, dy, dya, W)
     indexed = group_index is not None or ctx_len is not None
     gi, cl = _grouping(group_index, ctx_len, y.shape[0], y.shape[1], n_stages, dev, check_tables)
-    y, ya, dy, w = _prep(y.detach()), _prep(ya.detach()), _prep(dy.detach()), _w32(W)
+    if two_plane:
+        y, ya = _prep(ys_full.detach()), _prep(yas_full.detach())
+        y_code = _lib.NCN_BF16X2
+    else:
+        y, ya = _prep(y.detach()), _prep(ya.detach())
+        y_code = _DTYPES[y.dtype]
+    dy, w = _prep(dy.detach()), _w32(W)
     dya = _prep(dya.detach()) if dya is not None else None
     grad_dtype = dy.dtype if grad_dtype is None else grad_dtype
     need_state = want_inputs or n_stages > 1
     if n_stages > 1 and grad_dtype != torch.float32:
         raise ValueError("multi-stage backward carries its state in float32: use grad_dtype=torch.float32")
-    dx = torch.empty(y.shape, dtype=grad_dtype, device=dev)
-    dxa = torch.empty(y.shape, dtype=grad_dtype, device=dev)
-    x_rec = torch.empty(y.shape, dtype=torch.float32, device=dev) if need_state else None
-    xa_rec = torch.empty(y.shape, dtype=torch.float32, device=dev) if need_state else None
-    E = y.shape[2]
+    dx = torch.empty(dy.shape, dtype=grad_dtype, device=dev)
+    dxa = torch.empty(dy.shape, dtype=grad_dtype, device=dev)
+    x_rec = torch.empty(dy.shape, dtype=torch.float32, device=dev) if need_state else None
+    xa_rec = torch.empty(dy.shape, dtype=torch.float32, device=dev) if need_state else None
+    E = dy.shape[2]
     dW = torch.empty(n_stages, 2 * E, dtype=torch.float32, device=dev)
     lib = _lib.load()
     if indexed:
         ws_bytes = lib.ncn_workspace_bytes(ctypes.byref(shape))
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
         with torch.cuda.device(dev):
-            rc = lib.ncn_backward_indexed(_ptr(y), _ptr(ya), _DTYPES[y.dtype], _ptr(dy), _ptr(dya), _DTYPES[dy.dtype],
+            rc = lib.ncn_backward_indexed(_ptr(y), _ptr(ya), y_code, _ptr(dy), _ptr(dya), _DTYPES[dy.dtype],
                                           _ptr(dx), _ptr(dxa), _DTYPES[grad_dtype], _ptr(x_rec), _ptr(xa_rec), _ptr(w),
                                           _ptr(dW), _ptr(ws), ctypes.c_size_t(ws_bytes), _ptr(gi), _ptr(cl),
                                           ctypes.byref(shape), int(first_stage), int(n_stages), float(alpha), float(m),
@@ -234,7 +303,7 @@ def backward_stages(y, ya, dy, dya, W, alpha, activation, cache_dim, nhead, firs
     ws_bytes = lib.ncn_workspace_bytes_stages(ctypes.byref(shape), int(first_stage), int(n_stages), int(activation), 1)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
-        rc = lib.ncn_backward(_ptr(y), _ptr(ya), _DTYPES[y.dtype], _ptr(dy), _ptr(dya), _DTYPES[dy.dtype],
+        rc = lib.ncn_backward(_ptr(y), _ptr(ya), y_code, _ptr(dy), _ptr(dya), _DTYPES[dy.dtype],
                               _ptr(dx), _ptr(dxa), _DTYPES[grad_dtype], _ptr(x_rec), _ptr(xa_rec), _ptr(w), _ptr(dW),
                               _ptr(ws), ctypes.c_size_t(ws_bytes), ctypes.byref(shape), int(first_stage),
                               int(n_stages), float(alpha), float(m), int(activation), _stream(dev))

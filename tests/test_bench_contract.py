@@ -35,8 +35,11 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     assert d["unit"] == "tokens/s" and d["vs_baseline"] is None and d["data"] == "synthetic" and d["dtype"] == "f32"
     assert "workload" in d["config"] and "model" not in d["config"]
     r = d["roofline"]
-    assert r["bound"] in ("hbm", "mfma") and r["unit"] == "GB/s" and r["peak"] == 8000.0
+    assert r["bound"] == "hbm" and r["unit"] == "GB/s" and r["peak"] == 8000.0      # groups of 4 rows: bandwidth-bound
     assert abs(r["frac"] - r["achieved"] / r["peak"]) < 1e-12 and "traffic" in r
+    assert r["valu_achieved_TFLOPs"] > 0 and r["hbm_achieved_GBps"] == r["achieved"]
+    assert d["stack"]["min_ms_per_step"] <= d["stack"]["median_ms_per_step"] <= d["stack"]["max_ms_per_step"]
+    assert "B=4096 D=1024 g=4" in d["metric"]
     c = d["cpu_baseline"]
     assert c["kind"] in ("reference", "port") and c["cores"] >= 1 and c["value"] > 0 and c["sample"]
     assert abs(d["value"] - 32 * 128 / (d["ms_per_step"] * 1e-3)) < 1e-6 * d["value"]

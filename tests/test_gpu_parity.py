@@ -193,9 +193,12 @@ def test_other_activations_vs_oracle(M, act, shape):
         assert O.rel_err(dWs[l], ref_dWs[l]) < TOL_F32
 
 
-def test_bf16_storage_fp32_arithmetic(M):
+@pytest.mark.parametrize("save", ["two_bf16_planes", "float32_copies"])
+def test_bf16_storage_fp32_arithmetic(M, save):
     """bf16 activations and weights, float32 arithmetic: compared with the oracle run in float32 on the
-    same bf16-rounded inputs.  Tolerance 2e-2 relative."""
+    same bf16-rounded inputs.  Tolerance 2e-2 relative.  The saved outputs are the bf16 outputs plus what their
+    rounding took away (a second bf16 plane), or float32 copies; the two reconstructions must agree to the 16 bits the
+    planes hold."""
     batch, N, E, C, n, L = 4, 256, 128, 4, 16, 3
     alpha = 0.9
     x, xa, Ws, dyi, dya = O.make_inputs(batch, N, E, L, n, seed=0, xa_zero=True, dtype=torch.bfloat16)
@@ -207,15 +210,27 @@ def test_bf16_storage_fp32_arithmetic(M):
     saved = []
     cx, cxa = gx, gxa
     for l in range(L):
-        cx, cxa, y32, ya32 = M.forward_stages(cx, cxa, gWs[l], alpha, 0, n, C, l, 1, save_fp32=True)
-        assert cx.dtype == torch.bfloat16 and y32.dtype == torch.float32
-        saved.append((y32, ya32))
+        px, pxa = cx, cxa
+        if save == "float32_copies":
+            cx, cxa, y32, ya32 = M.forward_stages(px, pxa, gWs[l], alpha, 0, n, C, l, 1, save_fp32=True)
+            assert cx.dtype == torch.bfloat16 and y32.dtype == torch.float32
+        else:
+            cx, cxa, y32, ya32 = M.forward_stages(px, pxa, gWs[l], alpha, 0, n, C, l, 1, save_residual=True)
+            assert cx.dtype == torch.bfloat16 and y32.dtype == torch.bfloat16 and tuple(y32.shape) == (2, batch, N, E)
+            assert y32[0].data_ptr() == cx.data_ptr()       # plane 0 is the output itself
+            bx, _, f32y, f32ya = M.forward_stages(px, pxa, gWs[l], alpha, 0, n, C, l, 1, save_fp32=True)
+            assert torch.equal(bx, cx)
+            assert O.rel_err(y32[0].float() + y32[1].float(), f32y) < 2e-5    # 16 significant bits of the float32 value
+            assert O.rel_err(ya32[0].float() + ya32[1].float(), f32ya) < 2e-5
+        saved.append((y32, ya32, cx, cxa))
     assert O.rel_err(cx, ref_yi) < TOL_BF16
     assert O.rel_err(cxa, ref_ya) < TOL_BF16
     dy, dya_ = gdyi, gdya
     for l in range(L - 1, -1, -1):
-        _, _, dy, dya_, dW = M.backward_stages(saved[l][0], saved[l][1], dy, dya_, gWs[l], alpha, 0, n, C, l, 1,
-                                               grad_dtype=torch.bfloat16, want_inputs=False)
+        xr, _, dy, dya_, dW = M.backward_stages(saved[l][0], saved[l][1], dy, dya_, gWs[l], alpha, 0, n, C, l, 1,
+                                                grad_dtype=torch.bfloat16, want_inputs=True)
+        prev = saved[l - 1][2] if l else gx
+        assert O.rel_err(xr, prev.float()) < 1e-4     # the inversion of 16 steps amplifies the 2^-17 of the planes 5.4 times
         assert O.rel_err(dW[0], ref_dWs[l]) < TOL_BF16, f"dW{l}"
     assert dy.dtype == torch.bfloat16
     assert O.rel_err(dy, ref_dx) < TOL_BF16
