@@ -1,6 +1,7 @@
 """ctypes binding of libncn_hip.so (C ABI declared in include/ncn_hip.h).
 
-There is no fallback: if the library is missing or a symbol is absent, loading raises.
+There is no CPU or PyTorch fallback.  A library that is missing, or older than one of its sources, is built on the
+spot with hipcc (ncn_cuda_amd/_build.py, about a minute); if that cannot be done, loading raises.
 """
 import ctypes
 import os
@@ -25,15 +26,37 @@ class NcnShape(ctypes.Structure):
 _lib = None
 
 
+def _stale_reason():
+    """Why the shared library has to be built before it can be loaded, or None."""
+    if not os.path.exists(LIB_PATH):
+        return "libncn_hip.so is missing"
+    built = os.path.getmtime(LIB_PATH)
+    roots = [os.path.join(PKG_DIR, "csrc"), os.path.join(os.path.dirname(PKG_DIR), "include")]
+    for root in roots:
+        if not os.path.isdir(root):
+            continue                      # an installed copy without sources: take the library as it is
+        for name in os.listdir(root):
+            if name.endswith((".hip", ".h")) and os.path.getmtime(os.path.join(root, name)) > built:
+                return f"libncn_hip.so is older than {name}"
+    return None
+
+
 def load():
     """Load the shared library once and declare the prototypes."""
     global _lib
     if _lib is not None:
         return _lib
-    if not os.path.exists(LIB_PATH):
-        raise RuntimeError(
-            f"{LIB_PATH} is missing: build it with `python -m ncn_cuda_amd._build` "
-            "(or __graft_entry__.build()); there is no CPU or PyTorch fallback for the NCN kernels")
+    reason = _stale_reason()
+    if reason:
+        import sys
+        from . import _build
+        print(f"ncn_cuda_amd: {reason}: building it with hipcc (about a minute)", file=sys.stderr)
+        try:
+            _build.build()
+        except Exception as exc:
+            raise RuntimeError(
+                f"{LIB_PATH}: {reason}, and building it failed ({exc}); build it with `python -m ncn_cuda_amd._build` "
+                "(or __graft_entry__.build()): there is no CPU or PyTorch fallback for the NCN kernels") from exc
     lib = ctypes.CDLL(LIB_PATH)
     vp, f32p, shp = ctypes.c_void_p, ctypes.c_void_p, ctypes.POINTER(NcnShape)
     i, fl = ctypes.c_int, ctypes.c_float

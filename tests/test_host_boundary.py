@@ -318,10 +318,16 @@ def test_multi_stage_plan_declines_ineligible_shapes(lib):
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
-    """No fallback: if libncn_hip.so is absent the binding raises instead of computing something else."""
-    from ncn_cuda_amd import _lib
+    """No fallback: if libncn_hip.so is absent and cannot be built, the binding raises instead of computing something
+    else."""
+    from ncn_cuda_amd import _build, _lib
+
+    def no_compiler():
+        raise RuntimeError("hipcc not found")
+
     monkeypatch.setattr(_lib, "_lib", None)
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libncn_hip.so"))
+    monkeypatch.setattr(_build, "build", no_compiler)
     with pytest.raises(RuntimeError, match="no CPU or PyTorch fallback"):
         _lib.load()
 
@@ -341,3 +347,14 @@ def test_header_is_valid_c(tmp_path):
                    "int size_ok[sizeof(ncn_shape) == 32 ? 1 : -1];\n")
     subprocess.run([gcc, "-std=c99", "-Wall", "-Werror", "-Wno-pedantic", "-I", os.path.join(ROOT, "include"), "-c",
                     str(src), "-o", str(tmp_path / "use_header.o")], check=True)
+
+
+def test_library_staleness_check(lib, monkeypatch, tmp_path):
+    """load() builds a library that is missing or older than a source instead of failing: the check behind it."""
+    assert lib._stale_reason() is None                      # what build() left is newer than every source
+    monkeypatch.setattr(lib, "LIB_PATH", str(tmp_path / "libncn_hip.so"))
+    assert "missing" in lib._stale_reason()
+    (tmp_path / "libncn_hip.so").write_bytes(b"")
+    import os
+    os.utime(tmp_path / "libncn_hip.so", (1, 1))            # older than any source file
+    assert "older than" in lib._stale_reason()
