@@ -159,6 +159,65 @@ __device__ __forceinline__ void store_frag(void* base, int dtype, int64_t off, b
     }
 }
 
+// A register tile on its way from global memory: R row fragments of FPL features, still as loaded.  issue() only
+// requests the data (one branch on the element type around all the loads of the tile), finish() turns it into floats:
+// a kernel issues the loads of all its input tiles before it finishes the first, so that their latencies overlap
+// instead of following one another (converting each fragment as it is loaded waits for every load in turn).
+// The offsets must be valid addresses for every lane (lanes without work read some row of their own batch entry and
+// are zeroed afterwards where that matters).
+template <int R, int FPL>
+__device__ __forceinline__ void issue_tile(const void* base, int dtype, const int64_t (&off)[R], float (&v)[R][FPL],
+                                           int64_t plane = 0) {
+    static_assert(FPL % 4 == 0, "fragment must be a multiple of 4 features");
+    // the registers of the fragment hold the raw words until finish_tile: float32 all four of a chunk, bfloat16 the
+    // first two, two planes the value plane in the first two and the residual plane in the last two
+    if (dtype == NCN_F32) {
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr)
+#pragma unroll
+            for (int k = 0; k < FPL / 4; ++k) {
+                const float4 t = reinterpret_cast<const float4*>(static_cast<const float*>(base) + off[rr])[k];
+                v[rr][4 * k] = t.x; v[rr][4 * k + 1] = t.y; v[rr][4 * k + 2] = t.z; v[rr][4 * k + 3] = t.w;
+            }
+    } else if (dtype == NCN_BF16) {
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr)
+#pragma unroll
+            for (int k = 0; k < FPL / 4; ++k) {
+                const float2 t = reinterpret_cast<const float2*>(static_cast<const uint16_t*>(base) + off[rr])[k];
+                v[rr][4 * k] = t.x; v[rr][4 * k + 1] = t.y;
+            }
+    } else {
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr)
+#pragma unroll
+            for (int k = 0; k < FPL / 4; ++k) {
+                const float2 t = reinterpret_cast<const float2*>(static_cast<const uint16_t*>(base) + off[rr])[k];
+                const float2 u = reinterpret_cast<const float2*>(static_cast<const uint16_t*>(base) + off[rr] + plane)[k];
+                v[rr][4 * k] = t.x; v[rr][4 * k + 1] = t.y; v[rr][4 * k + 2] = u.x; v[rr][4 * k + 3] = u.y;
+            }
+    }
+}
+
+template <int R, int FPL>
+__device__ __forceinline__ void finish_tile(int dtype, float (&v)[R][FPL]) {
+    if (dtype == NCN_F32) return;
+#pragma unroll
+    for (int rr = 0; rr < R; ++rr)
+#pragma unroll
+        for (int k = 0; k < FPL / 4; ++k) {
+            float* o = &v[rr][4 * k];
+            const uint32_t w0 = __float_as_uint(o[0]), w1 = __float_as_uint(o[1]);
+            const uint32_t r0 = __float_as_uint(o[2]), r1 = __float_as_uint(o[3]);
+            o[0] = __uint_as_float(w0 << 16); o[1] = __uint_as_float(w0 & 0xffff0000u);
+            o[2] = __uint_as_float(w1 << 16); o[3] = __uint_as_float(w1 & 0xffff0000u);
+            if (dtype == NCN_BF16X2) {
+                o[0] += __uint_as_float(r0 << 16); o[1] += __uint_as_float(r0 & 0xffff0000u);
+                o[2] += __uint_as_float(r1 << 16); o[3] += __uint_as_float(r1 & 0xffff0000u);
+            }
+        }
+}
+
 __device__ __forceinline__ float load_elem(const void* base, int dtype, int64_t off, int64_t plane = 0) {
     if (dtype == NCN_F32) return static_cast<const float*>(base)[off];
     const uint16_t* p = static_cast<const uint16_t*>(base);

@@ -401,6 +401,18 @@ __device__ __forceinline__ void backward_steps(float (&Y)[R][F], float (&B)[R][F
 // Row rr of this lane is live when its slot is below the group's live rows (always, or never, without lengths).
 #define NCN_ROW_LIVE(rr) ((int)(((lane / T::LF) % T::LR) * R + (rr)) < live)
 
+// Tiles are loaded without predicates (the offsets of lanes and rows without work point at rows that exist): rows past
+// a context length, and the lanes of a wave tile past the last group, are zeroed here, so that they add nothing to the
+// sums of their group or to dW.
+#define NCN_ZERO_DEAD_ROWS(p, q)                                                                \
+    _Pragma("unroll") for (int rr = 0; rr < R; ++rr) {                                          \
+        const bool dead = !(INDEXED ? NCN_ROW_LIVE(rr) : live != 0);                            \
+        _Pragma("unroll") for (int f = 0; f < F; ++f) {                                         \
+            p[rr][f] = dead ? 0.f : p[rr][f];                                                   \
+            q[rr][f] = dead ? 0.f : q[rr][f];                                                   \
+        }                                                                                       \
+    }
+
 template <int NC, int EC, int R, int F, bool TANH_ONLY = true, bool INDEXED = false>
 __global__ void __launch_bounds__(kBlockThreads, (TANH_ONLY && !INDEXED && R == 4 && F == 4) ? 6 : 1) stage_forward_kernel(const StageArgs A) {
     NCN_WAVE_PROLOGUE
@@ -408,13 +420,12 @@ __global__ void __launch_bounds__(kBlockThreads, (TANH_ONLY && !INDEXED && R == 
         int64_t off[R];
         const int live = tile_offsets<NC, EC, R, F, INDEXED>(A, t, lane, head, off);
         float x[R][F], a[R][F];
-#pragma unroll
-        for (int rr = 0; rr < R; ++rr) {
-            const bool valid = INDEXED ? NCN_ROW_LIVE(rr) : live != 0;
-            load_frag<F>(A.in0, A.in_dtype, off[rr], valid, x[rr]);
-            load_frag<F>(A.in1, A.in_dtype, off[rr], valid, a[rr]);
-        }
+        issue_tile<R, F>(A.in0, A.in_dtype, off, x);
+        issue_tile<R, F>(A.in1, A.in_dtype, off, a);
         NCN_SCALE_W_ONCE
+        finish_tile<R, F>(A.in_dtype, x);
+        finish_tile<R, F>(A.in_dtype, a);
+        NCN_ZERO_DEAD_ROWS(x, a)
         scale_tile<R, F>(x, a, A.tab.kappa, A.tab.a_scale);
         forward_core<NC, EC, R, F, TANH_ONLY, INDEXED>(x, a, wi, wj, A.tab, lane, slots, live);
         scale_tile<R, F>(x, a, A.tab.inv_kappa, A.tab.inv_a_scale);
@@ -438,13 +449,12 @@ __global__ void __launch_bounds__(kBlockThreads) stage_inverse_kernel(const Stag
         int64_t off[R];
         const int live = tile_offsets<NC, EC, R, F, INDEXED>(A, t, lane, head, off);
         float y[R][F], b[R][F];
-#pragma unroll
-        for (int rr = 0; rr < R; ++rr) {
-            const bool valid = INDEXED ? NCN_ROW_LIVE(rr) : live != 0;
-            load_frag<F>(A.in0, A.in_dtype, off[rr], valid, y[rr], A.plane);
-            load_frag<F>(A.in1, A.in_dtype, off[rr], valid, b[rr], A.plane);
-        }
+        issue_tile<R, F>(A.in0, A.in_dtype, off, y, A.plane);
+        issue_tile<R, F>(A.in1, A.in_dtype, off, b, A.plane);
         NCN_SCALE_W_ONCE
+        finish_tile<R, F>(A.in_dtype, y);
+        finish_tile<R, F>(A.in_dtype, b);
+        NCN_ZERO_DEAD_ROWS(y, b)
         scale_tile<R, F>(y, b, A.tab.kappa, A.tab.b_scale);
         inverse_core<NC, EC, R, F, TANH_ONLY, INDEXED>(y, b, wi, wj, A.tab, lane, slots, live);
         scale_tile<R, F>(y, b, A.tab.inv_kappa, A.tab.inv_b_scale);
@@ -470,15 +480,24 @@ __global__ void __launch_bounds__(kBlockThreads, (TANH_ONLY && R * F <= 16 && F 
         int64_t off[R];
         const int live = tile_offsets<NC, EC, R, F, INDEXED>(A, t, lane, head, off);
         float Y[R][F], B[R][F], G[R][F], H[R][F];
+        issue_tile<R, F>(A.in0, A.in_dtype, off, Y, A.plane);
+        issue_tile<R, F>(A.in1, A.in_dtype, off, B, A.plane);
+        issue_tile<R, F>(A.g0, A.g_dtype, off, G);
+        if (A.g1) {
+            issue_tile<R, F>(A.g1, A.g_dtype, off, H);
+        } else {
 #pragma unroll
-        for (int rr = 0; rr < R; ++rr) {
-            const bool valid = INDEXED ? NCN_ROW_LIVE(rr) : live != 0;
-            load_frag<F>(A.in0, A.in_dtype, off[rr], valid, Y[rr], A.plane);
-            load_frag<F>(A.in1, A.in_dtype, off[rr], valid, B[rr], A.plane);
-            load_frag<F>(A.g0, A.g_dtype, off[rr], valid, G[rr]);
-            load_frag<F>(A.g1, A.g_dtype, off[rr], valid && A.g1 != nullptr, H[rr]);
+            for (int rr = 0; rr < R; ++rr)
+#pragma unroll
+                for (int f = 0; f < F; ++f) H[rr][f] = 0.f;
         }
         NCN_SCALE_W_ONCE
+        finish_tile<R, F>(A.in_dtype, Y);
+        finish_tile<R, F>(A.in_dtype, B);
+        finish_tile<R, F>(A.g_dtype, G);
+        if (A.g1) finish_tile<R, F>(A.g_dtype, H);
+        NCN_ZERO_DEAD_ROWS(Y, B)
+        NCN_ZERO_DEAD_ROWS(G, H)
         backward_steps<NC, EC, R, F, false, TANH_ONLY, INDEXED>(Y, B, G, H, wi, wj, dwi, dwj, 1.0f, A.tab, lane, slots,
                                                                live);
 #pragma unroll
@@ -514,6 +533,7 @@ __global__ void __launch_bounds__(kBlockThreads, (TANH_ONLY && R * F <= 16 && F 
     }
 }
 #undef NCN_ROW_LIVE
+#undef NCN_ZERO_DEAD_ROWS
 #undef NCN_SCALE_W_ONCE
 #undef NCN_WAVE_PROLOGUE
 
