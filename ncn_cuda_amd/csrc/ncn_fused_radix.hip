@@ -43,19 +43,19 @@ hipError_t launch_t(Pass pass, const FusedArgs& a, int grid, size_t lds, hipStre
     if (backward) {
         auto k = tanh_only ? fused_backward_kernel<NC, EC, t.r, t.f, true, true>
                            : fused_backward_kernel<NC, EC, t.r, t.f, false, true>;
-        err = hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        err = ensure_dynamic_lds(reinterpret_cast<const void*>(k), lds);
         if (err != hipSuccess) return err;
         hipLaunchKernelGGL(k, dim3(grid), dim3(64 * kFusedWavesBwd), lds, s, a);
     } else if (pass == kInverse) {
         auto k = tanh_only ? fused_forward_kernel<NC, EC, t.r, t.f, true, true, true>
                            : fused_forward_kernel<NC, EC, t.r, t.f, false, true, true>;
-        err = hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        err = ensure_dynamic_lds(reinterpret_cast<const void*>(k), lds);
         if (err != hipSuccess) return err;
         hipLaunchKernelGGL(k, dim3(grid), dim3(64 * kFusedWavesFwd), lds, s, a);
     } else {
         auto k = tanh_only ? fused_forward_kernel<NC, EC, t.r, t.f, true, true>
                            : fused_forward_kernel<NC, EC, t.r, t.f, false, true>;
-        err = hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        err = ensure_dynamic_lds(reinterpret_cast<const void*>(k), lds);
         if (err != hipSuccess) return err;
         hipLaunchKernelGGL(k, dim3(grid), dim3(64 * kFusedWavesFwd), lds, s, a);
     }

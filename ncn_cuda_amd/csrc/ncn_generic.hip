@@ -4,6 +4,10 @@
 // and the sum over a group's rows are plain LDS reads.  This is the slow, shape-agnostic path; the
 // register kernels in ncn_stage_kernels.h cover the shapes that matter for speed.
 // Same arithmetic as there; see that file for the formulas and their reference citations.
+#include <map>
+#include <mutex>
+#include <utility>
+
 #include "ncn_launch.h"
 
 namespace ncn {
@@ -260,6 +264,20 @@ __global__ void __launch_bounds__(256) pass_through_kernel(const StageArgs A, co
 
 }  // namespace
 
+hipError_t ensure_dynamic_lds(const void* kernel, size_t bytes) {
+    static std::mutex mu;
+    static std::map<std::pair<int, const void*>, size_t> raised;
+    int dev = 0;
+    hipError_t err = hipGetDevice(&dev);
+    if (err != hipSuccess) return err;
+    std::lock_guard<std::mutex> lock(mu);
+    size_t& have = raised[std::make_pair(dev, kernel)];
+    if (bytes <= have) return hipSuccess;
+    err = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (err == hipSuccess) have = bytes;
+    return err;
+}
+
 hipError_t launch_pass_through(Pass pass, const StageArgs& a, int64_t batch, hipStream_t s) {
     const int64_t per_entry = (a.N + 3) / 4;
     const unsigned gx = (unsigned)(per_entry < 64 ? per_entry : 64);
@@ -274,13 +292,11 @@ hipError_t launch_generic(Pass pass, const StageArgs& a, int n_head, int grid_x,
     const dim3 grid(grid_x, n_head), block(64);
     hipError_t err;
     if (pass == kBackward) {
-        err = hipFuncSetAttribute(reinterpret_cast<const void*>(generic_backward_kernel),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        err = ensure_dynamic_lds(reinterpret_cast<const void*>(generic_backward_kernel), lds_bytes);
         if (err != hipSuccess) return err;
         hipLaunchKernelGGL(generic_backward_kernel, grid, block, lds_bytes, s, a);
     } else {
-        err = hipFuncSetAttribute(reinterpret_cast<const void*>(generic_forward_kernel),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        err = ensure_dynamic_lds(reinterpret_cast<const void*>(generic_forward_kernel), lds_bytes);
         if (err != hipSuccess) return err;
         hipLaunchKernelGGL(generic_forward_kernel, grid, block, lds_bytes, s, a, pass == kInverse ? 1 : 0);
     }

@@ -62,6 +62,10 @@ struct ReduceJob {
 // out[col] of every segment = sum of its rows, in a fixed order; level1 is scratch of kReduceLevel1Rows * 2E floats.
 hipError_t launch_reduce_job(const ReduceJob& job, float* level1, hipStream_t s);
 
+// Raises a kernel's dynamic LDS limit to `bytes` on the current device unless an earlier call already raised it that
+// far (the limit is kept per device and kernel for the life of the process: one driver call instead of one per launch).
+hipError_t ensure_dynamic_lds(const void* kernel, size_t bytes);
+
 hipError_t launch_fast_forward(Pass pass, const StageArgs& a, int n_head, int grid_x, hipStream_t s);
 hipError_t launch_fast_backward(const StageArgs& a, int n_head, int grid_x, hipStream_t s);
 // the same kernels built to honour a.table and a.ctx_len (the plain builds ignore both)
