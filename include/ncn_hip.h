@@ -173,6 +173,21 @@ int ncn_inverse(const void* y, const void* ya, int in_dtype,
                 float alpha, float m, int activation, void* stream);
 
 /*
+ * ncn_inverse with scratch: with ncn_workspace_bytes_stages(shape, first_stage, n_stages, activation, 0) bytes (the
+ * forward's figure) and float32 outputs every multi-stage pass runs as one launch, halo passes included: the passes
+ * read one pair of buffers and write another, scratch and x, xa in turns.  With less scratch, or where the turns would
+ * make the first pass write into its own input (x == y with an odd number of passes), it does what ncn_inverse does.
+ * Replaces the same reference code as ncn_inverse; the reference has no multi-stage inverse
+ * (torch_ref/ncn_pytorch_invertible.py:87-113 undoes one stage per call).
+ */
+int ncn_inverse_ws(const void* y, const void* ya, int in_dtype,
+                   void* x, void* xa, int out_dtype,
+                   const float* W,
+                   void* workspace, size_t workspace_bytes,
+                   const ncn_shape* shape, int first_stage, int n_stages,
+                   float alpha, float m, int activation, void* stream);
+
+/*
  * The same three operations with the grouping given as a table and, optionally, one context length per batch entry.
  * Replaces: the group_tensor / ctxlen_tensor arguments of fused_chunk_linear_ncn and its kernels
  *           (ncn_triton/ncn_triton_old.py:53-57, 66-71, 93-96, 362-387), whose tables come from helpers such as the

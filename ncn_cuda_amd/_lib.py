@@ -13,7 +13,7 @@ NCN_F32, NCN_BF16, NCN_BF16X2 = 0, 1, 2
 ACT_TANH, ACT_RELU, ACT_SIGMOID, ACT_LEAKY_RELU, ACT_LINEAR = 0, 1, 2, 3, -1
 
 EXPORTS = ("ncn_forward", "ncn_backward", "ncn_inverse", "ncn_forward_indexed", "ncn_backward_indexed",
-           "ncn_inverse_indexed", "ncn_forward_radix", "ncn_backward_radix", "ncn_inverse_radix", "ncn_plan_radix", "ncn_workspace_bytes", "ncn_workspace_bytes_stages",
+           "ncn_inverse_indexed", "ncn_inverse_ws", "ncn_forward_radix", "ncn_backward_radix", "ncn_inverse_radix", "ncn_plan_radix", "ncn_workspace_bytes", "ncn_workspace_bytes_stages",
            "ncn_plan_passes", "ncn_kernel_path",
            "ncn_check_shape", "ncn_error_string", "ncn_version", "ncn_backward_static", "ncn_static_scratch_bytes", "ncn_kernel_path_scalars")
 
@@ -76,6 +76,8 @@ def load():
     lib.ncn_backward_indexed.restype = i
     lib.ncn_backward_indexed.argtypes = [vp, vp, i, vp, vp, i, vp, vp, i, f32p, f32p, f32p, f32p, vp, ctypes.c_size_t,
                                          vp, vp, shp, i, i, fl, fl, i, vp]
+    lib.ncn_inverse_ws.restype = i
+    lib.ncn_inverse_ws.argtypes = [vp, vp, i, vp, vp, i, f32p, vp, ctypes.c_size_t, shp, i, i, fl, fl, i, vp]
     lib.ncn_inverse_indexed.restype = i
     lib.ncn_inverse_indexed.argtypes = [vp, vp, i, vp, vp, i, f32p, vp, vp, shp, i, i, fl, fl, i, vp]
     lib.ncn_forward_radix.restype = i

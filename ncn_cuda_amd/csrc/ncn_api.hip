@@ -495,7 +495,7 @@ static int forward_impl(const void* x, const void* xa, int in_dtype, void* y, vo
 }
 
 static int inverse_impl(const void* y, const void* ya, int in_dtype, void* x, void* xa, int out_dtype, const float* W,
-                        const Grouping& grouping, const ncn_shape* shape, int first_stage, int n_stages, float alpha,
+                        void* workspace, size_t workspace_bytes, const Grouping& grouping, const ncn_shape* shape, int first_stage, int n_stages, float alpha,
                         float m, int activation, void* stream) {
     int rc = check_shape(shape, first_stage, n_stages, activation);
     if (rc != NCN_OK) return rc;
@@ -505,16 +505,57 @@ static int inverse_impl(const void* y, const void* ya, int in_dtype, void* x, vo
     const int path = kernel_path_for(shape, activation, alpha, m);
     if (path == 0) return NCN_ERR_UNSUPPORTED;
     if (!known_dtype_or_x2(in_dtype, n_stages, path) || !known_dtype(out_dtype)) return NCN_ERR_DTYPE;
-    if (!aligned16(x) || !aligned16(xa) || !aligned16(y) || !aligned16(ya) || !aligned16(W)) return NCN_ERR_ALIGN;
+    if (!aligned16(x) || !aligned16(xa) || !aligned16(y) || !aligned16(ya) || !aligned16(W) || !aligned16(workspace))
+        return NCN_ERR_ALIGN;
     const Plan p = make_plan(shape, path);
     hipStream_t s = static_cast<hipStream_t>(stream);
 
-    // several stages: LDS-resident passes, last pass of the range first.  There is no scratch to ping-pong with: the
+    // several stages: LDS-resident passes, last pass of the range first.  Without scratch to ping-pong with, the
     // first pass to run goes from y, ya to x, xa and the others work in place on x, xa, which a halo pass must not,
     // so the stages of such a pass are undone by one-stage launches (closed passes and one-stage launches may).
     std::vector<FusedPass> passes;
     if (grouping.plain() && (out_dtype == NCN_F32 || n_stages == 1))
         passes = multi_stage_plan(shape, first_stage, n_stages, activation, false, path);
+    // With scratch every pass reads one pair of buffers and writes another (scratch and x, xa in turns, so that the
+    // last pass to run lands in x, xa), as the forward does, and every multi-stage pass runs as one.
+    const bool ping_pong = passes.size() >= 2 && out_dtype == NCN_F32 && workspace &&
+                           workspace_bytes >= temp_bytes(shape, false) &&
+                           !((x == y || xa == ya) && ((passes.size() - 1) % 2) == 0);   // never straight from y into y
+    if (ping_pong) {
+        const int64_t wstride = 2 * shape->E;
+        const size_t np = passes.size();
+        const size_t one = temp_bytes(shape, false) / 2;
+        void* t0 = workspace;
+        void* t1 = static_cast<char*>(workspace) + one;
+        const void* cur0 = y;
+        const void* cur1 = ya;
+        int cur_dtype = in_dtype;
+        for (size_t e = 0; e < np; ++e) {
+            const FusedPass& ps = passes[np - 1 - e];
+            const bool to_out = ((np - 1 - e) % 2) == 0;
+            void* d0 = to_out ? x : t0;
+            void* d1 = to_out ? xa : t1;
+            hipError_t err;
+            if (ps.single) {
+                StageArgs a{};
+                fill_common(a, shape, p, first_stage + ps.first, alpha, m, activation);
+                a.in0 = cur0; a.in1 = cur1; a.in_dtype = cur_dtype;
+                a.out0 = d0; a.out1 = d1; a.out_dtype = NCN_F32;
+                a.W = W + ps.first * wstride;
+                err = launch_fast_forward(kInverse, a, shape->n_head, p.grid_fwd, s);
+            } else {
+                FusedArgs a{};
+                a.in0 = cur0; a.in1 = cur1; a.in_dtype = cur_dtype;
+                a.out0 = d0; a.out1 = d1; a.out_dtype = NCN_F32;
+                a.W = W + ps.first * wstride;
+                fill_step_table(a.tab, shape->n_cache, alpha, m, activation);
+                err = launch_fused(kInverse, a, shape, ps, s);
+            }
+            if (err != hipSuccess) return (int)err;
+            cur0 = d0; cur1 = d1; cur_dtype = NCN_F32;
+        }
+        return NCN_OK;
+    }
     if (!passes.empty()) {
         const int64_t wstride = 2 * shape->E;
         const size_t np = passes.size();
@@ -703,15 +744,22 @@ int ncn_forward_indexed(const void* x, const void* xa, int in_dtype, void* y, vo
 int ncn_inverse(const void* y, const void* ya, int in_dtype, void* x, void* xa, int out_dtype, const float* W,
                 const ncn_shape* shape, int first_stage, int n_stages, float alpha, float m, int activation,
                 void* stream) {
-    return inverse_impl(y, ya, in_dtype, x, xa, out_dtype, W, Grouping{nullptr, nullptr}, shape, first_stage, n_stages,
-                        alpha, m, activation, stream);
+    return inverse_impl(y, ya, in_dtype, x, xa, out_dtype, W, nullptr, 0, Grouping{nullptr, nullptr}, shape,
+                        first_stage, n_stages, alpha, m, activation, stream);
+}
+
+int ncn_inverse_ws(const void* y, const void* ya, int in_dtype, void* x, void* xa, int out_dtype, const float* W,
+                   void* workspace, size_t workspace_bytes, const ncn_shape* shape, int first_stage, int n_stages,
+                   float alpha, float m, int activation, void* stream) {
+    return inverse_impl(y, ya, in_dtype, x, xa, out_dtype, W, workspace, workspace_bytes, Grouping{nullptr, nullptr},
+                        shape, first_stage, n_stages, alpha, m, activation, stream);
 }
 
 int ncn_inverse_indexed(const void* y, const void* ya, int in_dtype, void* x, void* xa, int out_dtype, const float* W,
                         const int32_t* group_index, const int32_t* ctx_len, const ncn_shape* shape, int first_stage,
                         int n_stages, float alpha, float m, int activation, void* stream) {
-    return inverse_impl(y, ya, in_dtype, x, xa, out_dtype, W, Grouping{group_index, ctx_len}, shape, first_stage,
-                        n_stages, alpha, m, activation, stream);
+    return inverse_impl(y, ya, in_dtype, x, xa, out_dtype, W, nullptr, 0, Grouping{group_index, ctx_len}, shape,
+                        first_stage, n_stages, alpha, m, activation, stream);
 }
 
 int ncn_backward(const void* y, const void* ya, int y_dtype, const void* dy, const void* dya, int dy_dtype, void* dx,

@@ -312,8 +312,9 @@ def backward_stages(y, ya, dy, dya, W, alpha, activation, cache_dim, nhead, firs
 
 
 def inverse_stages(y, ya, W, alpha, activation, cache_dim, nhead, first_stage, n_stages, *, m=M_DEFAULT,
-                   out_dtype=None, group_index=None, ctx_len=None, check_tables=True):
-    """x, xa with forward_stages(x, xa, ...) == (y, ya)."""
+                   out_dtype=None, group_index=None, ctx_len=None, check_tables=True, scratch=True):
+    """x, xa with forward_stages(x, xa, ...) == (y, ya).  scratch: with several stages, allocate the scratch that lets
+    every multi-stage pass run as one (ncn_inverse_ws); without it the stages of a halo pass run one launch each."""
     shape = validate(y, ya, W, cache_dim, nhead, activation, first_stage, n_stages, what="y")
     dev = _require_gpu(y, ya, W)
     indexed = group_index is not None or ctx_len is not None
@@ -330,10 +331,23 @@ def inverse_stages(y, ya, W, alpha, activation, cache_dim, nhead, first_stage, n
                                                  int(activation), _stream(dev))
         _lib.check(rc, "ncn_inverse_indexed")
         return x, xa
+    lib = _lib.load()
+    ws_bytes = 0
+    if scratch and n_stages > 1 and out_dtype == torch.float32:
+        ws_bytes = lib.ncn_workspace_bytes_stages(ctypes.byref(shape), int(first_stage), int(n_stages), int(activation), 0)
+    if ws_bytes:
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        with torch.cuda.device(dev):
+            rc = lib.ncn_inverse_ws(_ptr(y), _ptr(ya), _DTYPES[y.dtype], _ptr(x), _ptr(xa), _DTYPES[out_dtype],
+                                    _ptr(w), _ptr(ws), ctypes.c_size_t(ws_bytes), ctypes.byref(shape),
+                                    int(first_stage), int(n_stages), float(alpha), float(m), int(activation),
+                                    _stream(dev))
+        _lib.check(rc, "ncn_inverse_ws")
+        return x, xa
     with torch.cuda.device(dev):
-        rc = _lib.load().ncn_inverse(_ptr(y), _ptr(ya), _DTYPES[y.dtype], _ptr(x), _ptr(xa), _DTYPES[out_dtype],
-                                     _ptr(w), ctypes.byref(shape), int(first_stage), int(n_stages), float(alpha),
-                                     float(m), int(activation), _stream(dev))
+        rc = lib.ncn_inverse(_ptr(y), _ptr(ya), _DTYPES[y.dtype], _ptr(x), _ptr(xa), _DTYPES[out_dtype],
+                             _ptr(w), ctypes.byref(shape), int(first_stage), int(n_stages), float(alpha),
+                             float(m), int(activation), _stream(dev))
     _lib.check(rc, "ncn_inverse")
     return x, xa
 

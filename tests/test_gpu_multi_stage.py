@@ -153,6 +153,21 @@ def test_multi_stage_inverse(M, case):
     assert rc == 0
     torch.cuda.synchronize()
     assert O.rel_err(py, xi) < tol and O.rel_err(pya, xai) < tol
+    # without scratch (ncn_inverse) and with it (ncn_inverse_ws, what inverse_stages calls): same stages, other launches
+    xn, xan = M.inverse_stages(y, ya, Wst, alpha, 0, n, C, first, L, scratch=False)
+    assert O.rel_err(xn, xi) < tol and O.rel_err(xan, xai) < tol
+    # ncn_inverse_ws in place, with the forward's scratch size
+    ws_bytes = _lib.load().ncn_workspace_bytes_stages(ctypes.byref(shape), first, L, 0, 0)
+    ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device="cuda")
+    qy, qya = y.clone(), ya.clone()
+    rc = _lib.load().ncn_inverse_ws(ctypes.c_void_p(qy.data_ptr()), ctypes.c_void_p(qya.data_ptr()), 0,
+                                    ctypes.c_void_p(qy.data_ptr()), ctypes.c_void_p(qya.data_ptr()), 0,
+                                    ctypes.c_void_p(Wst.data_ptr()), ctypes.c_void_p(ws.data_ptr()),
+                                    ctypes.c_size_t(ws_bytes), ctypes.byref(shape), first, L, alpha, 0.9, 0,
+                                    ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert O.rel_err(qy, xi) < tol and O.rel_err(qya, xai) < tol
 
 
 def _stage_by_stage_dW(M, outs, gdy, gdya, gWs, alpha, act, n, C, first):
