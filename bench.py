@@ -71,11 +71,12 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", default="cfg3", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--grouping", default="closed", choices=["closed", "stride-table", "radix-table", "ragged", "radix"],
+    ap.add_argument("--grouping", default="closed", choices=["closed", "stride-table", "radix-table", "ragged", "lengths", "radix"],
                     help="closed: the stride permutation in closed form (the headline path).  The others go through "
                          "the *_indexed entry points, one call per stage: the same permutation as a table, the "
                          "radix-n digit grouping as a table, or the stride table with one context length per batch "
-                         "entry (N - 1 - b mod n_cache live rows).  radix: levels 0 .. L-1 of the radix-n digit grouping "
+                         "entry (N - 1 - b mod n_cache live rows).  lengths: the closed-form permutation with the same "
+                         "lengths and no table, whole segments per call (multi-stage LDS passes for small groups).  radix: levels 0 .. L-1 of the radix-n digit grouping "
                          "through ncn_forward_radix / ncn_backward_radix (needs n_cache^L to divide N; several levels "
                          "per LDS pass for n_cache 2 and 4; float32 between calls)")
     ap.add_argument("--copy-probe", action="store_true",
@@ -117,9 +118,11 @@ def main():
     # Stages per saved checkpoint: 1 for the headline shape (every stage saves its outputs, like the reference's
     # autograd node); small groups run whole segments per call (multi-stage LDS passes) and reverse them from the
     # segment's outputs: rounding grows like (1/m)^(n_cache * stages), kept below 16x.
-    save_every = max(1, 26 // n) if args.grouping in ("closed", "radix") else 1   # tables run stage by stage
+    save_every = max(1, 26 // n) if args.grouping in ("closed", "radix", "lengths") else 1   # tables run stage by stage
     tables = lens = None
-    if args.grouping not in ("closed", "radix"):
+    if args.grouping == "lengths":   # the closed-form permutation with one context length per batch entry
+        lens = (N - 1 - torch.arange(batch, device=dev) % n).to(torch.int32)
+    elif args.grouping not in ("closed", "radix"):
         from ncn_cuda_amd import chunk_linear as CL
         if args.grouping == "radix-table":
             levels = 1
@@ -146,10 +149,12 @@ def main():
                 saved.append((y32, ya32))
             elif bf16 and cnt == 1:
                 # bf16 outputs plus what their rounding took away (a second bf16 plane): what the backward inverts
-                cx, cxa, ys, yas = M.forward_stages(cx, cxa, Wst[a], alpha, 0, n, C, a, 1, save_residual=True)
+                cx, cxa, ys, yas = M.forward_stages(cx, cxa, Wst[a], alpha, 0, n, C, a, 1, save_residual=True,
+                                                    ctx_len=lens)
                 saved.append((ys, yas))
             else:
-                cx, cxa = M.forward_stages(cx, cxa, Wst[a:a + cnt], alpha, 0, n, C, a, cnt, out_dtype=torch.float32)
+                cx, cxa = M.forward_stages(cx, cxa, Wst[a:a + cnt], alpha, 0, n, C, a, cnt, out_dtype=torch.float32,
+                                           ctx_len=lens)
                 saved.append((cx, cxa))
         dy, dya_ = gdyi, None  # the reference script back-propagates through yi only (grad_test_bench.py:121)
         dWs = [None] * len(segs)
@@ -158,7 +163,8 @@ def main():
             if events is not None:
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 e0.record()
-            extra = {} if tables is None else dict(group_index=tables[a], ctx_len=lens, check_tables=False)
+            extra = (dict(group_index=tables[a], ctx_len=lens, check_tables=False) if tables is not None else
+                     dict(ctx_len=lens))
             if args.grouping == "radix":
                 _, _, dy, dya_, dWs[k] = M.backward_radix(saved[k][0], saved[k][1], dy, dya_, Wst[a:a + cnt], alpha, 0,
                                                           n, C, a, cnt)

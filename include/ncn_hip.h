@@ -201,8 +201,14 @@ int ncn_inverse_ws(const void* y, const void* ya, int in_dtype,
  *                 on its live rows only, with as many steps as it has live rows; rows past the length pass through
  *                 (forward, inverse: out = in; backward: dx = dy, dxa = dya, x_rec = y, no share in dW).  Values are
  *                 clamped to [0, N].
- * Everything else as in ncn_forward / ncn_backward / ncn_inverse, except that these always run stage by stage (no
- * multi-stage passes, so forward takes no workspace) and ncn_backward_indexed needs ncn_workspace_bytes(shape).
+ * Everything else as in ncn_forward / ncn_backward / ncn_inverse.  With a table these run stage by stage and
+ * ncn_backward_indexed needs ncn_workspace_bytes(shape).  With lengths only (group_index NULL) the grouping is the
+ * stride permutation and several stages use the multi-stage LDS passes where ncn_forward / ncn_inverse / ncn_backward
+ * would (float32 between passes): forward and inverse take no workspace, so their first pass goes from the inputs to
+ * the outputs and the others work in place on the outputs, where the stages of a halo pass run one launch each;
+ * ncn_backward_indexed uses the passes when given ncn_workspace_bytes_stages(.., backward = 1) bytes.  Inside a pass
+ * the rows past a length stay in LDS in the kernels' scaled form, so they come out equal to their inputs to rounding
+ * (one launch per stage copies them bit for bit).
  */
 int ncn_forward_indexed(const void* x, const void* xa, int in_dtype,
                         void* y, void* ya, int out_dtype,

@@ -14,7 +14,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libncn_hip.so")
 SOURCES = ["ncn_api.hip", "ncn_fwd.hip", "ncn_bwd.hip", "ncn_fwd_indexed.hip", "ncn_bwd_indexed.hip", "ncn_generic.hip",
-           "ncn_fused.hip", "ncn_fused_radix.hip"]
+           "ncn_fused.hip", "ncn_fused_radix.hip", "ncn_fused_lengths.hip"]
 # packed-fp32 VALU instructions are switched off for device code on purpose (flag is device-only;
 # the host pass prints a harmless "not a recognized feature" note).
 HIPCC_FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17",

@@ -162,6 +162,7 @@ struct Grouping {
     const int32_t* ctx_len;  // [batch] or null
     int radix_first = -1;    // >= 0: stage k is radix level radix_first + k (no table then)
     bool plain() const { return !table && !ctx_len && radix_first < 0; }
+    bool permutation() const { return !table && radix_first < 0; }   // the stride permutation, with or without lengths
 };
 
 uint32_t upow(uint32_t b, int e) {
@@ -427,14 +428,56 @@ static int forward_impl(const void* x, const void* xa, int in_dtype, void* y, vo
 
     // several stages: LDS-resident passes when the shape allows and the buffers permit the ping-pong
     std::vector<FusedPass> passes;
-    if (grouping.plain()) passes = multi_stage_plan(shape, first_stage, n_stages, activation, false, path);
+    if (grouping.permutation()) passes = multi_stage_plan(shape, first_stage, n_stages, activation, false, path);
     const size_t np = passes.size();
-    bool fused_ok = np > 0;
-    if (np >= 2 && (out_dtype != NCN_F32 || !workspace || workspace_bytes < temp_bytes(shape, false))) fused_ok = false;
-    // a halo pass (or a one-stage launch feeding one) must not write where another workgroup still reads its halo:
-    // refuse the in-place case when the first pass would write straight into x, xa
-    if (np >= 1 && (x == y || xa == ya) && ((np - 1) % 2) == 0 && !passes[0].closed && !passes[0].single) fused_ok = false;
-    if (fused_ok) {
+    // one stage of the range with the one-stage kernel (and, with lengths, the launch for the rows past them)
+    auto run_stage = [&](int k, const void* i0, const void* i1, int i_dtype, void* o0, void* o1, int o_dtype,
+                         bool with_copies) -> hipError_t {
+        StageArgs a{};
+        fill_common(a, shape, p, first_stage + k, alpha, m, activation, grouping, k);
+        a.in0 = i0; a.in1 = i1; a.in_dtype = i_dtype;
+        a.out0 = o0; a.out1 = o1; a.out_dtype = o_dtype;
+        a.aux0 = with_copies ? y32 : nullptr; a.aux1 = with_copies ? ya32 : nullptr;
+        a.W = W + k * wstride;
+        hipError_t err = grouping.plain() ? launch_fast_forward(kForward, a, shape->n_head, p.grid_fwd, s)
+                                          : launch_fast_forward_indexed(kForward, a, shape->n_head, p.grid_fwd, s);
+        if (err == hipSuccess && grouping.ctx_len) err = launch_ragged_rest(kForward, a, shape, p.path, 0, s);
+        return err;
+    };
+    bool fused_ok = np > 0 && (np < 2 || out_dtype == NCN_F32);
+    // Buffers in turns (scratch and y, ya) when the scratch is there; a halo pass (or a one-stage launch feeding one)
+    // must not write where another workgroup still reads its halo, so not when the first pass would write straight
+    // into x, xa.  Otherwise the first pass goes from x, xa to y, ya and the others work in place on y, ya, where the
+    // stages of a halo pass run one launch each (closed passes and one-stage launches may work in place).
+    const bool turns = fused_ok && (np < 2 || (workspace && workspace_bytes >= temp_bytes(shape, false))) &&
+                       !((x == y || xa == ya) && ((np - 1) % 2) == 0 && !passes[0].closed && !passes[0].single);
+    if (fused_ok && !turns) {
+        for (size_t k = 0; k < np; ++k) {
+            const FusedPass& ps = passes[k];
+            const bool last = (k + 1 == np);
+            const bool in_place = k > 0 || x == y || xa == ya;
+            hipError_t err = hipSuccess;
+            if (ps.single || (!ps.closed && in_place)) {
+                for (int j = ps.first; j < ps.first + ps.count && err == hipSuccess; ++j) {
+                    const bool from_x = (k == 0 && j == ps.first);
+                    err = run_stage(j, from_x ? x : y, from_x ? xa : ya, from_x ? in_dtype : out_dtype, y, ya, out_dtype,
+                                    last && j == ps.first + ps.count - 1);
+                }
+            } else {
+                FusedArgs a{};
+                a.in0 = k == 0 ? x : y; a.in1 = k == 0 ? xa : ya; a.in_dtype = k == 0 ? in_dtype : out_dtype;
+                a.out0 = y; a.out1 = ya; a.out_dtype = out_dtype;
+                a.aux0 = last ? y32 : nullptr; a.aux1 = last ? ya32 : nullptr;
+                a.W = W + ps.first * wstride;
+                a.ctx_len = grouping.ctx_len;
+                fill_step_table(a.tab, shape->n_cache, alpha, m, activation);
+                err = launch_fused(kForward, a, shape, ps, s);
+            }
+            if (err != hipSuccess) return (int)err;
+        }
+        return NCN_OK;
+    }
+    if (turns) {
         const size_t one = temp_bytes(shape, false) / 2;
         void* t0 = workspace;
         void* t1 = workspace ? static_cast<char*>(workspace) + one : nullptr;
@@ -450,19 +493,14 @@ static int forward_impl(const void* x, const void* xa, int in_dtype, void* y, vo
             const int d_dtype = to_out ? out_dtype : NCN_F32;
             hipError_t err;
             if (ps.single) {
-                StageArgs a{};
-                fill_common(a, shape, p, first_stage + ps.first, alpha, m, activation);
-                a.in0 = cur0; a.in1 = cur1; a.in_dtype = cur_dtype;
-                a.out0 = d0; a.out1 = d1; a.out_dtype = d_dtype;
-                a.aux0 = last ? y32 : nullptr; a.aux1 = last ? ya32 : nullptr;
-                a.W = W + ps.first * wstride;
-                err = launch_fast_forward(kForward, a, shape->n_head, p.grid_fwd, s);
+                err = run_stage(ps.first, cur0, cur1, cur_dtype, d0, d1, d_dtype, last);
             } else {
                 FusedArgs a{};
                 a.in0 = cur0; a.in1 = cur1; a.in_dtype = cur_dtype;
                 a.out0 = d0; a.out1 = d1; a.out_dtype = d_dtype;
                 a.aux0 = last ? y32 : nullptr; a.aux1 = last ? ya32 : nullptr;
                 a.W = W + ps.first * wstride;
+                a.ctx_len = grouping.ctx_len;
                 fill_step_table(a.tab, shape->n_cache, alpha, m, activation);
                 err = launch_fused(kForward, a, shape, ps, s);
             }
@@ -514,8 +552,19 @@ static int inverse_impl(const void* y, const void* ya, int in_dtype, void* x, vo
     // first pass to run goes from y, ya to x, xa and the others work in place on x, xa, which a halo pass must not,
     // so the stages of such a pass are undone by one-stage launches (closed passes and one-stage launches may).
     std::vector<FusedPass> passes;
-    if (grouping.plain() && (out_dtype == NCN_F32 || n_stages == 1))
+    if (grouping.permutation() && (out_dtype == NCN_F32 || n_stages == 1))
         passes = multi_stage_plan(shape, first_stage, n_stages, activation, false, path);
+    auto run_stage = [&](int k, const void* i0, const void* i1, int i_dtype, void* o0, void* o1, int o_dtype) -> hipError_t {
+        StageArgs a{};
+        fill_common(a, shape, p, first_stage + k, alpha, m, activation, grouping, k);
+        a.in0 = i0; a.in1 = i1; a.in_dtype = i_dtype;
+        a.out0 = o0; a.out1 = o1; a.out_dtype = o_dtype;
+        a.W = W + (int64_t)k * 2 * shape->E;
+        hipError_t err = grouping.plain() ? launch_fast_forward(kInverse, a, shape->n_head, p.grid_fwd, s)
+                                          : launch_fast_forward_indexed(kInverse, a, shape->n_head, p.grid_fwd, s);
+        if (err == hipSuccess && grouping.ctx_len) err = launch_ragged_rest(kInverse, a, shape, p.path, 0, s);
+        return err;
+    };
     // With scratch every pass reads one pair of buffers and writes another (scratch and x, xa in turns, so that the
     // last pass to run lands in x, xa), as the forward does, and every multi-stage pass runs as one.
     const bool ping_pong = passes.size() >= 2 && out_dtype == NCN_F32 && workspace &&
@@ -537,17 +586,13 @@ static int inverse_impl(const void* y, const void* ya, int in_dtype, void* x, vo
             void* d1 = to_out ? xa : t1;
             hipError_t err;
             if (ps.single) {
-                StageArgs a{};
-                fill_common(a, shape, p, first_stage + ps.first, alpha, m, activation);
-                a.in0 = cur0; a.in1 = cur1; a.in_dtype = cur_dtype;
-                a.out0 = d0; a.out1 = d1; a.out_dtype = NCN_F32;
-                a.W = W + ps.first * wstride;
-                err = launch_fast_forward(kInverse, a, shape->n_head, p.grid_fwd, s);
+                err = run_stage(ps.first, cur0, cur1, cur_dtype, d0, d1, NCN_F32);
             } else {
                 FusedArgs a{};
                 a.in0 = cur0; a.in1 = cur1; a.in_dtype = cur_dtype;
                 a.out0 = d0; a.out1 = d1; a.out_dtype = NCN_F32;
                 a.W = W + ps.first * wstride;
+                a.ctx_len = grouping.ctx_len;
                 fill_step_table(a.tab, shape->n_cache, alpha, m, activation);
                 err = launch_fused(kInverse, a, shape, ps, s);
             }
@@ -565,13 +610,9 @@ static int inverse_impl(const void* y, const void* ya, int in_dtype, void* x, vo
             const bool in_place = !top || x == y || xa == ya;
             if (ps.single || (!ps.closed && in_place)) {
                 for (int k = ps.first + ps.count - 1; k >= ps.first; --k) {
-                    StageArgs a{};
-                    fill_common(a, shape, p, first_stage + k, alpha, m, activation);
                     const bool from_y = top && k == ps.first + ps.count - 1;
-                    a.in0 = from_y ? y : x; a.in1 = from_y ? ya : xa; a.in_dtype = from_y ? in_dtype : out_dtype;
-                    a.out0 = x; a.out1 = xa; a.out_dtype = out_dtype;
-                    a.W = W + k * wstride;
-                    hipError_t err = launch_fast_forward(kInverse, a, shape->n_head, p.grid_fwd, s);
+                    hipError_t err = run_stage(k, from_y ? y : x, from_y ? ya : xa, from_y ? in_dtype : out_dtype, x, xa,
+                                               out_dtype);
                     if (err != hipSuccess) return (int)err;
                 }
             } else {
@@ -579,6 +620,7 @@ static int inverse_impl(const void* y, const void* ya, int in_dtype, void* x, vo
                 a.in0 = top ? y : x; a.in1 = top ? ya : xa; a.in_dtype = top ? in_dtype : out_dtype;
                 a.out0 = x; a.out1 = xa; a.out_dtype = out_dtype;
                 a.W = W + ps.first * wstride;
+                a.ctx_len = grouping.ctx_len;
                 fill_step_table(a.tab, shape->n_cache, alpha, m, activation);
                 hipError_t err = launch_fused(kInverse, a, shape, ps, s);
                 if (err != hipSuccess) return (int)err;
@@ -637,7 +679,7 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
     // several stages: LDS-resident passes, last pass of the range first; the state ping-pongs between the
     // output arrays and four float32 arrays behind the dW scratch (their grids count on kMaxGridX partial rows)
     std::vector<FusedPass> passes;
-    if (grouping.plain() && row_cap == kMaxGridX)
+    if (grouping.permutation() && row_cap == kMaxGridX)
         passes = multi_stage_plan(shape, first_stage, n_stages, activation, true, path);
     const size_t np = passes.size();
     bool fused_ok = np > 0;
@@ -668,14 +710,17 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
             if (err != hipSuccess) return (int)err;
             if (ps.single) {
                 StageArgs a{};
-                fill_common(a, shape, p, first_stage + ps.first, alpha, m, activation);
+                fill_common(a, shape, p, first_stage + ps.first, alpha, m, activation, grouping, ps.first);
                 a.in0 = cy; a.in1 = cya; a.in_dtype = cy_dtype;
                 a.g0 = cg; a.g1 = cga; a.g_dtype = cg_dtype;
                 a.out0 = ddx; a.out1 = ddxa; a.out_dtype = d_dtype;
                 a.aux0 = dxr; a.aux1 = dxar;
                 a.W = W + ps.first * wstride;
                 a.dw_partials = region;
-                err = launch_fast_backward(a, shape->n_head, p.grid_x, s);
+                err = grouping.plain() ? launch_fast_backward(a, shape->n_head, p.grid_x, s)
+                                       : launch_fast_backward_indexed(a, shape->n_head, p.grid_x, s);
+                if (err == hipSuccess && grouping.ctx_len)
+                    err = launch_ragged_rest(kBackward, a, shape, p.path, p.partial_rows, s);
             } else {
                 FusedArgs a{};
                 a.in0 = cy; a.in1 = cya; a.in_dtype = cy_dtype;
@@ -684,6 +729,7 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
                 a.aux0 = dxr; a.aux1 = dxar;
                 a.W = W + ps.first * wstride;
                 a.dw_partials = region;
+                a.ctx_len = grouping.ctx_len;
                 fill_step_table(a.tab, shape->n_cache, alpha, m, activation);
                 err = launch_fused(kBackward, a, shape, ps, s);
             }

@@ -200,6 +200,7 @@ hipError_t launch_fused(Pass pass, FusedArgs& a, const ncn_shape* sh, const Fuse
     a.scale_up = (float)std::pow((double)a.tab.m, -(double)(nc * p.count));
     const int grid = fused_grid(sh, p, backward);
     const size_t lds = fused_lds_bytes(nc, ec, backward, p.window, p.count);
+    if (a.ctx_len) return launch_fused_lengths(pass, a, nc, ec, grid, lds, s);
 #define NCN_CASE(NC, EC) \
     if (nc == NC && ec == EC) return launch_fused_t<NC, EC>(pass, a, grid, lds, s);
     NCN_FOR_EACH_FUSED_CONFIG(NCN_CASE)

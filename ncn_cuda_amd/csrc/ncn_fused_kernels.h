@@ -55,6 +55,7 @@ struct FusedArgs {
     float* aux1;       //          optional float32 copy of ya              xa_rec
     const float* W;    // [n_stages][2E], first stage of the pass first
     float* dw_partials;  // backward: [gridDim.x / n_head][n_stages][2E]
+    const int32_t* ctx_len;  // LENGTHS builds: [batch] live slots per batch entry (in the group order of each stage)
     int64_t N, E;
     int32_t n_head, n_stages;
     int32_t in_dtype, g_dtype, out_dtype, reserved;
@@ -76,7 +77,7 @@ struct FusedArgs {
 
 struct FusedItem {
     int head;
-    uint32_t cls, sub0, own_lo, own_cnt;
+    uint32_t cls, sub0, own_lo, own_cnt, batch;
     int64_t base;  // element offset of (batch, row 0, head slice)
 };
 
@@ -108,6 +109,7 @@ __device__ __forceinline__ FusedItem fused_item(const FusedArgs& A, uint32_t ite
         const uint32_t left = A.ring - k * A.own;
         it.own_cnt = left < A.own ? left : A.own;
     }
+    it.batch = b;
     it.base = (int64_t)b * A.N * A.E + (int64_t)it.head * EC;
     return it;
 }
@@ -144,6 +146,17 @@ __device__ __forceinline__ uint32_t fused_lds_row(const FusedArgs& A, uint32_t q
     uint32_t qi = qg + i * sstride;
     if (A.closed) qi = (qg & ~(A.ring - 1u)) | (qi & (A.ring - 1u));  // wrap inside the group's own ring
     return qi * NC + i;
+}
+
+// Live rows of the group whose slot-0 sub-block is window position qg, for a batch entry with `len` live slots: the
+// group's number is the block of its slot 0 (the stride permutation leaves slot 0 in place), its slots are
+// number * NC + 0 .. NC-1 (ncn_triton/ncn_triton_old.py:66, 93-96).
+template <int NC>
+__device__ __forceinline__ int fused_live_rows(const FusedArgs& A, const FusedItem& it, uint32_t qg, int32_t len) {
+    const uint32_t sub = (it.sub0 + qg) & (A.ring - 1u);
+    const uint32_t cls = A.closed ? it.cls + qg / A.ring : it.cls;
+    const int64_t r = (int64_t)len - (int64_t)(sub * A.class_stride + cls) * NC;
+    return (int)max((int64_t)0, min(r, (int64_t)NC));
 }
 
 template <int F>
@@ -249,8 +262,11 @@ __device__ __forceinline__ void fused_load_weights(const FusedArgs& A, int head,
 
 // TANH_ONLY as in the one-stage kernels: the tanh build has no branch on the activation code.
 // INVERSE: the same kernel undoes the stages instead, last one first (in0, in1 = y, ya; out0, out1 = x, xa).
-template <int NC, int EC, int R, int F, bool TANH_ONLY, bool RADIX = false, bool INVERSE = false>
+// LENGTHS: one context length per batch entry; the group a length cuts runs its live steps on its live rows, rows
+// past the length stay in LDS as they came (a row may be live in one stage of the pass and past the length in another).
+template <int NC, int EC, int R, int F, bool TANH_ONLY, bool RADIX = false, bool INVERSE = false, bool LENGTHS = false>
 __global__ void __launch_bounds__(64 * kFusedWavesFwd) fused_forward_kernel(const FusedArgs A) {
+    static_assert(!(RADIX && LENGTHS), "context lengths go with the stride permutation");
     constexpr int NW = kFusedWavesFwd;
     using T = Tile<NC, EC, R, F>;
     extern __shared__ float4 fused_lds4[];
@@ -275,6 +291,7 @@ __global__ void __launch_bounds__(64 * kFusedWavesFwd) fused_forward_kernel(cons
     }
     for (uint32_t item = blockIdx.x; item < A.total_items; item += gridDim.x) {
         const FusedItem it = fused_item<NC, EC, RADIX>(A, item);
+        const int32_t len = LENGTHS ? max(0, min(A.ctx_len[it.batch], (int32_t)A.N)) : 0;
         fused_commit_rows<EC, NW, K>(rx, A.in_dtype, xs, rows, A.tab.kappa);
         fused_commit_rows<EC, NW, K>(ra, A.in_dtype, as, rows, INVERSE ? A.tab.b_scale : A.tab.a_scale);
         __syncthreads();
@@ -302,11 +319,13 @@ __global__ void __launch_bounds__(64 * kFusedWavesFwd) fused_forward_kernel(cons
                     lds_load_frag<F>(xs + row[rr], x[rr]);
                     lds_load_frag<F>(as + row[rr], a[rr]);
                 }
-                if (INVERSE) inverse_core<NC, EC, R, F, TANH_ONLY, false, true>(x, a, wi, wj, A.tab, lane, slots);
-                else forward_core<NC, EC, R, F, TANH_ONLY, false, true>(x, a, wi, wj, A.tab, lane, slots);
+                const int live = !LENGTHS ? NC : valid ? fused_live_rows<NC>(A, it, qg, len) : 0;
+                if (INVERSE) inverse_core<NC, EC, R, F, TANH_ONLY, LENGTHS, true>(x, a, wi, wj, A.tab, lane, slots, live);
+                else forward_core<NC, EC, R, F, TANH_ONLY, LENGTHS, true>(x, a, wi, wj, A.tab, lane, slots, live);
                 if (valid) {
 #pragma unroll
                     for (int rr = 0; rr < R; ++rr) {
+                        if (LENGTHS && rl * R + rr >= live) continue;
                         lds_store_frag<F>(xs + row[rr], x[rr]);
                         lds_store_frag<F>(as + row[rr], a[rr]);
                     }
@@ -322,8 +341,9 @@ __global__ void __launch_bounds__(64 * kFusedWavesFwd) fused_forward_kernel(cons
     }
 }
 
-template <int NC, int EC, int R, int F, bool TANH_ONLY, bool RADIX = false>
+template <int NC, int EC, int R, int F, bool TANH_ONLY, bool RADIX = false, bool LENGTHS = false>
 __global__ void __launch_bounds__(64 * kFusedWavesBwd, TANH_ONLY ? 4 : 1) fused_backward_kernel(const FusedArgs A) {
+    static_assert(!(RADIX && LENGTHS), "context lengths go with the stride permutation");
     constexpr int NW = kFusedWavesBwd;
     using T = Tile<NC, EC, R, F>;
     extern __shared__ float4 fused_lds4[];
@@ -387,6 +407,7 @@ __global__ void __launch_bounds__(64 * kFusedWavesBwd, TANH_ONLY ? 4 : 1) fused_
     __syncthreads();
     for (uint32_t item = blockIdx.x; item < A.total_items; item += gridDim.x) {
         const FusedItem it = fused_item<NC, EC, RADIX>(A, item);
+        const int32_t len = LENGTHS ? max(0, min(A.ctx_len[it.batch], (int32_t)A.N)) : 0;
         for (int st = A.n_stages - 1; st >= 0; --st) {
             const uint32_t ss = A.sub_stride[st];
             const uint32_t ngroups = A.closed ? A.window : A.window - (NC - 1) * ss;
@@ -409,11 +430,37 @@ __global__ void __launch_bounds__(64 * kFusedWavesBwd, TANH_ONLY ? 4 : 1) fused_
                     lds_load_frag<F>(gs + row[rr], G[rr]);
                     lds_load_frag<F>(ps + row[rr], P[rr]);
                 }
-                backward_core<NC, EC, R, F, true, TANH_ONLY, false, true>(Y, B, G, P, wi, wj, dwi, dwj, own, A.tab, (A.n_stages - 1 - st) * NC,
-                                                  lane, slots);
+                const int live = !LENGTHS ? NC : valid ? fused_live_rows<NC>(A, it, qg, len) : 0;
+                if (LENGTHS && live != NC) {
+                    // G, P carry m^-t: the steps this group skips still count.  Rows past the length only take the
+                    // factor of the whole stage and leave the sums of the group (zeros in the registers); the live
+                    // rows take the factor of the skipped steps here and that of their own steps in the step code.
+                    const float isc = pow_steps(A.tab.im, NC - live);
+#pragma unroll
+                    for (int rr = 0; rr < R; ++rr) {
+                        const bool dead = rl * R + rr >= live;
+#pragma unroll
+                        for (int f = 0; f < F; ++f) {
+                            const float sc = dead ? A.tab.inv_m_pow_n : isc;
+                            G[rr][f] *= sc;
+                            P[rr][f] *= sc;
+                        }
+                        if (dead) {
+                            if (valid) {
+                                lds_store_frag<F>(gs + row[rr], G[rr]);
+                                lds_store_frag<F>(ps + row[rr], P[rr]);
+                            }
+#pragma unroll
+                            for (int f = 0; f < F; ++f) Y[rr][f] = B[rr][f] = G[rr][f] = P[rr][f] = 0.f;
+                        }
+                    }
+                }
+                backward_core<NC, EC, R, F, true, TANH_ONLY, LENGTHS, true>(Y, B, G, P, wi, wj, dwi, dwj, own, A.tab,
+                                                                          (A.n_stages - 1 - st) * NC, lane, slots, live);
                 if (valid) {
 #pragma unroll
                     for (int rr = 0; rr < R; ++rr) {
+                        if (LENGTHS && rl * R + rr >= live) continue;
                         lds_store_frag<F>(ys + row[rr], Y[rr]);
                         lds_store_frag<F>(bs + row[rr], B[rr]);
                         lds_store_frag<F>(gs + row[rr], G[rr]);

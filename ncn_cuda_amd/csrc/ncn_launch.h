@@ -88,6 +88,8 @@ bool fused_supported(const ncn_shape* sh, int activation);
 std::vector<FusedPass> plan_fused(const ncn_shape* sh, int first, int count, bool backward);
 int fused_grid(const ncn_shape* sh, const FusedPass& p, bool backward);
 hipError_t launch_fused(Pass pass, FusedArgs& a, const ncn_shape* sh, const FusedPass& p, hipStream_t s);
+// the builds with context lengths (a.ctx_len set), ncn_fused_lengths.hip; launch_fused goes there by itself
+hipError_t launch_fused_lengths(Pass pass, const FusedArgs& a, int nc, int ec, int grid, size_t lds, hipStream_t s);
 
 
 // ---- multi-stage passes over radix-n levels, ncn_fused_radix.hip ---------------------------------------------

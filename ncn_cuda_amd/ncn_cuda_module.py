@@ -290,7 +290,11 @@ def backward_stages(y, ya, dy, dya, W, alpha, activation, cache_dim, nhead, firs
     dW = torch.empty(n_stages, 2 * E, dtype=torch.float32, device=dev)
     lib = _lib.load()
     if indexed:
-        ws_bytes = lib.ncn_workspace_bytes(ctypes.byref(shape))
+        # lengths without a table keep the stride permutation: with the multi-stage figure the library runs its
+        # multi-stage passes on them too
+        ws_bytes = (lib.ncn_workspace_bytes(ctypes.byref(shape)) if group_index is not None else
+                    lib.ncn_workspace_bytes_stages(ctypes.byref(shape), int(first_stage), int(n_stages),
+                                                   int(activation), 1))
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
         with torch.cuda.device(dev):
             rc = lib.ncn_backward_indexed(_ptr(y), _ptr(ya), y_code, _ptr(dy), _ptr(dya), _DTYPES[dy.dtype],

@@ -143,7 +143,57 @@ def test_context_lengths_without_table_and_inverse(M):
     assert O.rel_err(xi, x) < 3e-5 and O.rel_err(xai, xa) < 3e-5
     gt = torch.stack(tables).to(torch.int32).cuda()
     xi2, xai2 = M.inverse_stages(y, ya, gW, 0.9, 0, n, C, 0, L, group_index=gt, ctx_len=gl)
-    assert torch.equal(xi, xi2) and torch.equal(xai, xai2)
+    # lengths alone go through the multi-stage passes, a table through one launch per stage: equal to rounding
+    assert O.rel_err(xi, xi2) < TOL and O.rel_err(xai, xai2) < TOL
+
+
+LENGTH_PASS_CASES = [
+    (3, 1024, 64, 2, 2, 0, 11),    # halo passes, a closed pass, strides that wrap to 0
+    (2, 8192, 128, 4, 2, 0, 13),   # the deep small-group configuration at its real N
+    (4, 1024, 128, 4, 4, 0, 5),    # n = 4
+    (3, 2048, 64, 2, 2, 3, 6),     # range that starts at stage 3
+    (5, 64, 128, 4, 4, 0, 3),      # tiny ring
+]
+
+
+@pytest.mark.parametrize("case", LENGTH_PASS_CASES, ids=lambda c: "b%d_N%d_E%d_C%d_n%d_s%d_L%d" % c)
+def test_lengths_inside_multi_stage_passes(M, case):
+    """Context lengths with the stride permutation over a stage range: the library runs its multi-stage LDS passes
+    (rows past a length stay in LDS, the group a length cuts runs its live steps).  Checked against the same call with
+    the permutation given as a table, which runs one launch per stage (the path the oracle tests cover), and on the
+    smaller cases against the oracle itself."""
+    batch, N, E, C, n, first, L = case
+    x, xa, Ws, dy, dya = O.make_inputs(batch, N, E, L, n, seed=41, xa_zero=False)
+    lens = ([N // 2 + 1, 2 * n, N, 0, N + 5, 1, N - 1] * 2)[:batch]
+    tables = [O.stride_group_table(N, n, first + l) for l in range(L)]
+    gx, gxa, gdy, gdya = _dev(x, xa, dy, dya)
+    gW = torch.stack(Ws).cuda()
+    gt = torch.stack(tables).to(torch.int32).cuda()
+    gl = torch.tensor(lens, dtype=torch.int32).cuda()
+    amp = (1 / 0.9) ** (n * L)
+    tol, gtol = 1e-5, max(1e-5, 1e-6 * amp)
+    y, ya = M.forward_stages(gx, gxa, gW, 0.9, 0, n, C, first, L, ctx_len=gl)
+    ty, tya = M.forward_stages(gx, gxa, gW, 0.9, 0, n, C, 0, L, group_index=gt, ctx_len=gl)
+    assert O.rel_err(y, ty) < tol and O.rel_err(ya, tya) < tol
+    # rows past the lengths in every stage come out as they went in
+    for b, ln in enumerate(lens):
+        if ln == 0:
+            assert O.rel_err(y[b], gx[b]) < 1e-6 and O.rel_err(ya[b], gxa[b]) < 1e-6
+    got = M.backward_stages(y, ya, gdy, gdya, gW, 0.9, 0, n, C, first, L, ctx_len=gl)
+    ref = M.backward_stages(y, ya, gdy, gdya, gW, 0.9, 0, n, C, 0, L, group_index=gt, ctx_len=gl)
+    for name, u, v in zip(("x_rec", "xa_rec", "dx", "dxa", "dW"), got, ref):
+        assert O.rel_err(u, v) < gtol, name
+    xi, xai = M.inverse_stages(y, ya, gW, 0.9, 0, n, C, first, L, ctx_len=gl)
+    assert O.rel_err(xi, got[0]) < gtol and O.rel_err(xai, got[1]) < gtol
+    assert O.rel_err(xi, x) < max(3e-5, 3e-6 * amp)
+    if batch * N * E * L <= 3 * 1024 * 64 * 11:
+        d = torch.float64
+        ry, rya, rdx, rdxa, rdWs = O.net_autograd_indexed(x.to(d), xa.to(d), [w.to(d) for w in Ws], dy.to(d),
+                                                          dya.to(d), 0.9, n, C, tables, lens)
+        assert O.rel_err(y, ry) < tol and O.rel_err(ya, rya) < tol
+        assert O.rel_err(got[2], rdx) < gtol and O.rel_err(got[3], rdxa) < gtol
+        for l in range(L):
+            assert O.rel_err(got[4][l], rdWs[l]) < gtol, "dW%d" % l
 
 
 def test_bf16_and_other_activation_with_lengths(M):
