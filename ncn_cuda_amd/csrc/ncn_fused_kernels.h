@@ -131,6 +131,15 @@ __device__ __forceinline__ int64_t fused_row_offset(const FusedArgs& A, const Fu
     return it.base + ((int64_t)blk * NC + o) * A.E;
 }
 
+// Where window row `lr` lies in LDS.  The rows of one slot of neighbouring groups are NC rows apart, i.e. a multiple of
+// 256 bytes at these head widths: they would all start in the same LDS bank.  Flipping the row's lowest bit with the
+// bit above its slot number puts every other one of them half the banks further (rows stay whole, pairs swap places).
+template <int NC>
+__device__ __forceinline__ uint32_t fused_lds_place(uint32_t lr) {
+    constexpr uint32_t lg = NC == 2 ? 1u : NC == 4 ? 2u : 3u;
+    return lr ^ ((lr >> lg) & 1u);
+}
+
 // LDS row of slot i of the group whose slot-0 sub-block is window position qg
 // (RADIX: row of digit i at level log_n(sstride) of group qg; groups are numbered window by window)
 template <int NC, bool RADIX>
@@ -141,11 +150,11 @@ __device__ __forceinline__ uint32_t fused_lds_row(const FusedArgs& A, uint32_t q
         const uint32_t lg_span = log2u(A.ring), lg_sj = log2u(sstride);
         const uint32_t gpw = A.ring >> lg_nc;                       // groups per window
         const uint32_t wq = qg >> (lg_span - lg_nc), g = qg & (gpw - 1u);
-        return (wq << lg_span) + ((g >> lg_sj) << (lg_sj + lg_nc)) + (i << lg_sj) + (g & (sstride - 1u));
+        return fused_lds_place<NC>((wq << lg_span) + ((g >> lg_sj) << (lg_sj + lg_nc)) + (i << lg_sj) + (g & (sstride - 1u)));
     }
     uint32_t qi = qg + i * sstride;
     if (A.closed) qi = (qg & ~(A.ring - 1u)) | (qi & (A.ring - 1u));  // wrap inside the group's own ring
-    return qi * NC + i;
+    return fused_lds_place<NC>(qi * NC + i);
 }
 
 // Live rows of the group whose slot-0 sub-block is window position qg, for a batch entry with `len` live slots: the
@@ -217,7 +226,7 @@ __device__ __forceinline__ void fused_raw_to_float(const uint4& r, int dtype, fl
     }
 }
 
-template <int EC, int NW, int K>
+template <int NC, int EC, int NW, int K>
 __device__ __forceinline__ void fused_commit_rows(const uint4 (&raw)[K], int dtype, float* dst, uint32_t rows, float scale) {
     constexpr uint32_t CPR = EC / 4;
 #pragma unroll
@@ -228,7 +237,7 @@ __device__ __forceinline__ void fused_commit_rows(const uint4 (&raw)[K], int dty
             fused_raw_to_float(raw[k], dtype, v);
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[e] *= scale;
-            lds_store_frag<4>(dst + c * 4, v);   // c * 4 == lr * EC + c4 * 4
+            lds_store_frag<4>(dst + fused_lds_place<NC>(c / CPR) * EC + (c % CPR) * 4, v);
         }
     }
 }
@@ -242,7 +251,7 @@ __device__ __forceinline__ void fused_store_rows_scaled(const FusedArgs& A, cons
     for (uint32_t c = threadIdx.x; c < rows * CPR; c += 64 * NW) {
         const uint32_t lr = r0 + c / CPR, c4 = c % CPR;
         float v[4];
-        lds_load_frag<4>(src + lr * EC + c4 * 4, v);
+        lds_load_frag<4>(src + fused_lds_place<NC>(lr) * EC + c4 * 4, v);
 #pragma unroll
         for (int k = 0; k < 4; ++k) v[k] *= scale;
         const int64_t off = fused_row_offset<NC, RADIX>(A, it, lr) + c4 * 4;
@@ -292,8 +301,8 @@ __global__ void __launch_bounds__(64 * kFusedWavesFwd) fused_forward_kernel(cons
     for (uint32_t item = blockIdx.x; item < A.total_items; item += gridDim.x) {
         const FusedItem it = fused_item<NC, EC, RADIX>(A, item);
         const int32_t len = LENGTHS ? max(0, min(A.ctx_len[it.batch], (int32_t)A.N)) : 0;
-        fused_commit_rows<EC, NW, K>(rx, A.in_dtype, xs, rows, A.tab.kappa);
-        fused_commit_rows<EC, NW, K>(ra, A.in_dtype, as, rows, INVERSE ? A.tab.b_scale : A.tab.a_scale);
+        fused_commit_rows<NC, EC, NW, K>(rx, A.in_dtype, xs, rows, A.tab.kappa);
+        fused_commit_rows<NC, EC, NW, K>(ra, A.in_dtype, as, rows, INVERSE ? A.tab.b_scale : A.tab.a_scale);
         __syncthreads();
         if (item + gridDim.x < A.total_items) {   // the next window travels while this one is computed
             int64_t off[K];
@@ -382,9 +391,9 @@ __global__ void __launch_bounds__(64 * kFusedWavesBwd, TANH_ONLY ? 4 : 1) fused_
         fused_fetch_rows<K>(A.g1, A.g_dtype, off, r.h);
     };
     auto commit = [&](const Raw& r) {
-        fused_commit_rows<EC, NW, K>(r.y, A.in_dtype, ys, rows, A.tab.kappa);
-        fused_commit_rows<EC, NW, K>(r.b, A.in_dtype, bs, rows, A.tab.b_scale);
-        fused_commit_rows<EC, NW, K>(r.g, A.g_dtype, gs, rows, 1.0f);
+        fused_commit_rows<NC, EC, NW, K>(r.y, A.in_dtype, ys, rows, A.tab.kappa);
+        fused_commit_rows<NC, EC, NW, K>(r.b, A.in_dtype, bs, rows, A.tab.b_scale);
+        fused_commit_rows<NC, EC, NW, K>(r.g, A.g_dtype, gs, rows, 1.0f);
         constexpr uint32_t CPR = EC / 4;   // p = (1-m) g + h  (h = 0 when dya is null: the fetch left zeros)
 #pragma unroll
         for (int k = 0; k < K; ++k) {
@@ -395,7 +404,7 @@ __global__ void __launch_bounds__(64 * kFusedWavesBwd, TANH_ONLY ? 4 : 1) fused_
                 fused_raw_to_float(r.h[k], A.g_dtype, h);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) h[e] = fmaf(om, g[e], h[e]);
-                lds_store_frag<4>(ps + c * 4, h);
+                lds_store_frag<4>(ps + fused_lds_place<NC>(c / CPR) * EC + (c % CPR) * 4, h);
             }
         }
     };
@@ -496,8 +505,8 @@ __global__ void __launch_bounds__(64 * kFusedWavesBwd, TANH_ONLY ? 4 : 1) fused_
                 const uint32_t lr = r0 + c / CPR, c4 = c % CPR;
                 const int64_t off = fused_row_offset<NC, RADIX>(A, it, lr) + c4 * 4;
                 float g[4], h[4];
-                lds_load_frag<4>(gs + lr * EC + c4 * 4, g);
-                lds_load_frag<4>(ps + lr * EC + c4 * 4, h);
+                lds_load_frag<4>(gs + fused_lds_place<NC>(lr) * EC + c4 * 4, g);
+                lds_load_frag<4>(ps + fused_lds_place<NC>(lr) * EC + c4 * 4, h);
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     g[k] *= A.scale_dn;
