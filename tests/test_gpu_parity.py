@@ -260,3 +260,43 @@ def test_high_stage_numbers(M, stage):
     assert O.rel_err(y, ref_y) < TOL_F32 and O.rel_err(ya, ref_ya) < TOL_F32
     rx, rxa = M.inverse(y, ya, gw, 0.9, 0, n, C, stage)
     assert O.rel_err(rx, x) < TOL_F32 and O.rel_err(rxa, xa) < TOL_F32
+
+
+@pytest.mark.parametrize("alpha,m,with_backward", [(1e-4, 0.9, True), (0.9, 0.9995, True), (0.5, 5e-4, False)],
+                         ids=["alpha_near_0", "m_near_1", "m_near_0"])
+def test_scalars_the_scaled_state_cannot_carry_run_on_the_generic_kernels(M, alpha, m, with_backward):
+    """The register kernels carry x times alpha and xa times 1 - m (and divide by m): values next to zero are sent to
+    the generic kernels, which use alpha and m as they are.  Same results as the oracle either way.  (m next to 0 makes
+    the stage irreversible in float32, (1/m)^n, so only its forward is compared.)"""
+    import ctypes
+    from ncn_cuda_amd import _lib
+    batch, N, E, C, n, L = 2, 128, 128, 4, 16, 2
+    if not with_backward:
+        n, L = 4, 1     # with m next to 0 every step halves x (x' ~ tanh(alpha x ..)): few steps keep the outputs O(0.1)
+    shape = _lib.NcnShape(batch, N, E, C, n)
+    assert _lib.load().ncn_kernel_path(ctypes.byref(shape)) == 2
+    assert _lib.load().ncn_kernel_path_scalars(ctypes.byref(shape), alpha, m) == 1
+    assert _lib.load().ncn_kernel_path_scalars(ctypes.byref(shape), 0.9, 0.9) == 2
+    x, xa, Ws, dyi, dya = O.make_inputs(batch, N, E, L, n, seed=23, xa_zero=False)
+    d = torch.float64
+    gx, gxa, gdy, gdya = _dev(x, xa, dyi, dya)
+    gW = torch.stack(Ws).cuda()
+    # the C ABI takes float scalars: the oracle gets the values the library sees (1 - m differs by 5e-5 otherwise)
+    alpha, m = float(torch.tensor(alpha, dtype=torch.float32)), float(torch.tensor(m, dtype=torch.float32))
+    ry, rya = O.net_forward(x.to(d), xa.to(d), [w.to(d) for w in Ws], alpha, n, C, m=m)
+    y, ya = gx, gxa
+    outs = []
+    for l in range(L):
+        y, ya = M.forward_stages(y, ya, gW[l], alpha, 0, n, C, l, 1, m=m)
+        outs.append((y, ya))
+    assert O.rel_err(y, ry) < TOL_F32 and O.rel_err(ya, rya) < TOL_F32
+    if not with_backward:
+        return
+    _, _, rdx, rdxa, rdWs = O.net_autograd(x.to(d), xa.to(d), [w.to(d) for w in Ws], dyi.to(d), dya.to(d), alpha, n, C,
+                                           m=m)
+    g, h = gdy, gdya
+    for l in range(L - 1, -1, -1):
+        _, _, g, h, dW = M.backward_stages(outs[l][0], outs[l][1], g, h, gW[l], alpha, 0, n, C, l, 1, m=m)
+        assert O.rel_err(dW[0], rdWs[l]) < max(TOL_F32, 1e-6 * (1 / m) ** n), "dW%d" % l
+    gtol = max(TOL_F32, 1e-6 * (1 / m) ** n)
+    assert O.rel_err(g, rdx) < gtol and O.rel_err(h, rdxa) < gtol

@@ -79,6 +79,12 @@ def test_kernel_path_and_workspace(lib):
     assert h.ncn_workspace_bytes_stages(ctypes.byref(deep), 0, 1, 0, 0) == 0
     head = _shape(lib, 128, 4096, 128, 4, 16)
     assert h.ncn_workspace_bytes_stages(ctypes.byref(head), 0, 3, 0, 1) == h.ncn_workspace_bytes(ctypes.byref(head))
+    # scalars the register kernels' scaled state cannot carry go to the generic kernels, or nowhere for wide heads
+    for alpha, m, want in ((0.9, 0.9, 2), (1e-4, 0.9, 1), (0.9, 0.9995, 1), (0.9, 5e-4, 1), (40.0, 0.9, 2), (2000.0, 0.9, 1), (1e-3, 0.999, 2)):
+        assert h.ncn_kernel_path_scalars(ctypes.byref(head), alpha, m) == want, (alpha, m)
+    wide = _shape(lib, 2, 64, 256, 2, 8)        # heads of 128: register kernels only
+    assert h.ncn_kernel_path_scalars(ctypes.byref(wide), 0.9, 0.9) == 2
+    assert h.ncn_kernel_path_scalars(ctypes.byref(wide), 1e-4, 0.9) == 0
 
 
 def test_entry_points_reject_bad_arguments_before_touching_the_gpu(lib):
