@@ -269,3 +269,30 @@ def test_chunk_linear_surface_autograd(M):
         assert O.rel_err(yi, ref[0]) < TOL and O.rel_err(ya, ref[1]) < TOL
         assert O.rel_err(gx.grad, ref[2]) < TOL and O.rel_err(gxa.grad, ref[3]) < TOL
         assert gw.grad.shape == gw.shape and O.rel_err(gw.grad, ref[4][0]) < TOL
+
+
+@pytest.mark.parametrize("with_lengths", [False, True], ids=["table", "table_and_lengths"])
+def test_chunk_linear_bf16_storage_groups_of_16(M, with_lengths):
+    """fused_chunk_linear_ncn with bfloat16 tensors at groups of 16 rows: its autograd node has to keep more than the
+    bfloat16 outputs (the inversion amplifies their rounding by (1/m)^16 = 5.4).  bfloat16 storage with float32
+    arithmetic at 2e-2 against the float64 oracle on the same bfloat16-rounded inputs."""
+    from ncn_cuda_amd import chunk_linear as CL
+    batch, N, E, C, n = 3, 256, 128, 4, 16
+    x, xa, Ws, dy, dya = O.make_inputs(batch, N, E, 1, n, seed=43, xa_zero=False, dtype=torch.bfloat16)
+    lens = [N - 5, 3 * n, N] if with_lengths else None
+    table = CL.radix_group_table(N, n, 1, device="cuda")
+    d = torch.float64
+    ref = O.net_autograd_indexed(x.to(d), xa.to(d), [Ws[0].to(d)], dy.to(d), dya.to(d), 0.9, n, C,
+                                 [table.cpu().long()], lens)
+    gx = x.cuda().requires_grad_()
+    gxa = xa.cuda().requires_grad_()
+    gw = Ws[0].cuda().requires_grad_()
+    gl = torch.tensor(lens).cuda() if lens is not None else None
+    yi, ya = CL.fused_chunk_linear_ncn(gx, gxa, gw, table, gl, 0.9, "tanh", C, n, 0)
+    assert yi.dtype == torch.bfloat16
+    torch.autograd.backward([yi, ya], [dy.cuda(), dya.cuda()])
+    tol = 2e-2
+    assert O.rel_err(yi.float(), ref[0]) < tol and O.rel_err(ya.float(), ref[1]) < tol
+    assert gx.grad.dtype == torch.bfloat16
+    assert O.rel_err(gx.grad.float(), ref[2]) < tol and O.rel_err(gxa.grad.float(), ref[3]) < tol
+    assert O.rel_err(gw.grad.float(), ref[4][0]) < tol
