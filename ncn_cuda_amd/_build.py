@@ -21,6 +21,14 @@ HIPCC_FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 
+# Instruction scheduling per translation unit.  The multi-stage kernels wait on latency (LDS, barriers, dependent
+# chains of two-row tiles): LLVM's max-ILP strategy measured 2.5 % on the 13-stage configuration, and 1.5 % on the
+# one-stage forward; the one-stage backward is bound by issue slots and does not care.
+MAX_ILP = ["-mllvm", "-amdgpu-sched-strategy=max-ilp"]
+EXTRA_FLAGS = {"ncn_fused.hip": MAX_ILP, "ncn_fused_radix.hip": MAX_ILP, "ncn_fused_lengths.hip": MAX_ILP,
+               "ncn_fwd.hip": MAX_ILP}
+
+
 def _hipcc():
     exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(exe):
@@ -30,7 +38,7 @@ def _hipcc():
 
 def _compile(args):
     src, obj = args
-    cmd = [_hipcc(), *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [_hipcc(), *HIPCC_FLAGS, *EXTRA_FLAGS.get(src, []), "-c", os.path.join(CSRC, src), "-o", obj]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"hipcc failed on {src}:\n{proc.stdout}\n{proc.stderr}")
