@@ -63,7 +63,7 @@ std::vector<FusedPass> plan_fused(const ncn_shape* sh, int first, int count, boo
     std::vector<FusedPass> passes;
     const int nc = sh->n_cache, ec = (int)(sh->E / sh->n_head);
     const uint32_t groups = (uint32_t)(sh->N / nc);
-    const uint32_t cap_rows = (uint32_t)(kFusedStateBytes / ((backward ? 4 : 2) * ec * sizeof(float)));
+    const uint32_t cap_rows = (uint32_t)(fused_state_bytes(backward) / ((backward ? 4 : 2) * ec * sizeof(float)));
     uint32_t cap = floor_pow2(cap_rows / nc);
     if (cap > groups) cap = groups;
     if (cap < 4) return passes;

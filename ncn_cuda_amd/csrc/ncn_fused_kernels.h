@@ -40,8 +40,17 @@ namespace ncn {
 // The step code is instantiated with ROWS = true here: these kernels wait on latency rather than on issue slots, and
 // reductions through DPP row operations come back sooner than through the LDS crossbar (measured 2.5 % on 13 stages).
 constexpr int kFusedMaxStages = 8;
-constexpr size_t kFusedStateBytes = 64 * 1024;  // LDS for the row arrays of one workgroup (2 forward, 4 backward)
-constexpr int kFusedWavesFwd = 8;   // (16 waves per workgroup measured slower: all waves of a workgroup share its phases)
+// LDS for the row arrays of one workgroup (2 forward and inverse, 4 backward)
+#ifndef NCN_FUSED_STATE_FWD
+#define NCN_FUSED_STATE_FWD (64 * 1024)
+#endif
+constexpr size_t kFusedStateBytesFwd = NCN_FUSED_STATE_FWD;
+constexpr size_t kFusedStateBytesBwd = 64 * 1024;
+constexpr size_t fused_state_bytes(bool backward) { return backward ? kFusedStateBytesBwd : kFusedStateBytesFwd; }
+#ifndef NCN_FUSED_WAVES_FWD
+#define NCN_FUSED_WAVES_FWD 8
+#endif
+constexpr int kFusedWavesFwd = NCN_FUSED_WAVES_FWD;   // (16 waves per workgroup measured slower: all waves of a workgroup share its phases)
 constexpr int kFusedWavesBwd = 8;   // backward runs at 128 VGPRs: 4 waves per SIMD in all
 
 struct FusedArgs {
@@ -290,7 +299,7 @@ __global__ void __launch_bounds__(64 * kFusedWavesFwd) fused_forward_kernel(cons
     fused_load_weights<EC, NW>(A, blockIdx.x % A.n_head, w_lds);   // every item of this workgroup has this head
 
     // trips of 64 * NW threads over the float4 chunks of the largest window the LDS budget allows
-    constexpr int K = (int)((kFusedStateBytes / 2 / sizeof(float4) + 64 * NW - 1) / (64 * NW));
+    constexpr int K = (int)((kFusedStateBytesFwd / 2 / sizeof(float4) + 64 * NW - 1) / (64 * NW));
     uint4 rx[K], ra[K];
     if (blockIdx.x < A.total_items) {
         int64_t off[K];
@@ -378,7 +387,7 @@ __global__ void __launch_bounds__(64 * kFusedWavesBwd, TANH_ONLY ? 4 : 1) fused_
     // The step code leaves no registers to carry a window across the stages, but between two items they are free:
     // the window of the next item is requested (all loads of a thread back to back) before the owned rows of this one
     // are written out, and lands in LDS after them.
-    constexpr int K = (int)((kFusedStateBytes / 4 / sizeof(float4) + 64 * NW - 1) / (64 * NW));
+    constexpr int K = (int)((kFusedStateBytesBwd / 4 / sizeof(float4) + 64 * NW - 1) / (64 * NW));
     struct Raw {
         uint4 y[K], b[K], g[K], h[K];
     };

@@ -84,7 +84,7 @@ bool radix_fused_supported(const ncn_shape* sh) {
 std::vector<RadixPass> plan_radix(const ncn_shape* sh, int first, int count, bool backward, bool fused) {
     std::vector<RadixPass> passes;
     const int nc = sh->n_cache, ec = (int)(sh->E / sh->n_head);
-    const uint32_t cap_rows = floor_pow2((uint32_t)(kFusedStateBytes / ((backward ? 4 : 2) * ec * sizeof(float))));
+    const uint32_t cap_rows = floor_pow2((uint32_t)(fused_state_bytes(backward) / ((backward ? 4 : 2) * ec * sizeof(float))));
     int kmax = 0;
     while (ipow(nc, kmax + 1) <= (int64_t)cap_rows) ++kmax;
     const int max_stages = backward ? kFusedMaxStages - 1 : kFusedMaxStages;
