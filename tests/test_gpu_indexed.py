@@ -271,6 +271,32 @@ def test_chunk_linear_surface_autograd(M):
         assert gw.grad.shape == gw.shape and O.rel_err(gw.grad, ref[4][0]) < TOL
 
 
+@pytest.mark.parametrize("act", [2, 3, -1], ids=["sigmoid", "leaky_relu", "linear"])
+def test_lengths_inside_multi_stage_passes_other_activations(M, act):
+    """The builds of the multi-stage kernels that pick the activation at run time, with context lengths: against the
+    table path (one launch per stage) on the same lengths.  Leaky relu on inputs that keep T away from its kink."""
+    batch, N, E, C, n, first, L = 3, 512, 64, 2, 2, 0, 6
+    if act == 3:
+        x, xa, Ws, dy, dya = O.make_inputs_signed_regimes(batch, N, E, L, n, seed=47)
+    else:
+        x, xa, Ws, dy, dya = O.make_inputs(batch, N, E, L, n, seed=47, xa_zero=False)
+    lens = [N // 2 + 1, N - 1, 3]
+    gx, gxa, gdy, gdya = _dev(x, xa, dy, dya)
+    gW = torch.stack(Ws).cuda()
+    gt = torch.stack([O.stride_group_table(N, n, l) for l in range(L)]).to(torch.int32).cuda()
+    gl = torch.tensor(lens, dtype=torch.int32).cuda()
+    tol = max(1e-5, 1e-6 * (1 / 0.9) ** (n * L))
+    y, ya = M.forward_stages(gx, gxa, gW, 0.9, act, n, C, first, L, ctx_len=gl)
+    ty, tya = M.forward_stages(gx, gxa, gW, 0.9, act, n, C, 0, L, group_index=gt, ctx_len=gl)
+    assert O.rel_err(y, ty) < 1e-5 and O.rel_err(ya, tya) < 1e-5
+    got = M.backward_stages(y, ya, gdy, gdya, gW, 0.9, act, n, C, first, L, ctx_len=gl)
+    ref = M.backward_stages(y, ya, gdy, gdya, gW, 0.9, act, n, C, 0, L, group_index=gt, ctx_len=gl)
+    for name, u, v in zip(("x_rec", "xa_rec", "dx", "dxa", "dW"), got, ref):
+        assert O.rel_err(u, v) < (3 * tol if name == "xa_rec" else tol), name
+    xi, xai = M.inverse_stages(y, ya, gW, 0.9, act, n, C, first, L, ctx_len=gl)
+    assert O.rel_err(xi, got[0]) < tol and O.rel_err(xai, got[1]) < 3 * tol
+
+
 @pytest.mark.parametrize("with_lengths", [False, True], ids=["table", "table_and_lengths"])
 def test_chunk_linear_bf16_storage_groups_of_16(M, with_lengths):
     """fused_chunk_linear_ncn with bfloat16 tensors at groups of 16 rows: its autograd node has to keep more than the
