@@ -22,11 +22,12 @@ HIPCC_FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17",
 
 
 # Instruction scheduling per translation unit.  The multi-stage kernels wait on latency (LDS, barriers, dependent
-# chains of two-row tiles): LLVM's max-ILP strategy measured 2.5 % on the 13-stage configuration, and 1.5 % on the
-# one-stage forward; the one-stage backward is bound by issue slots and does not care.
+# chains of two-row tiles): LLVM's max-ILP strategy measured 2.5 % on the 13-stage configuration, 1.5 % on the
+# one-stage forward and 1.2 % on a step through the table builds; the plain one-stage backward is bound by issue slots
+# and does not care.
 MAX_ILP = ["-mllvm", "-amdgpu-sched-strategy=max-ilp"]
 EXTRA_FLAGS = {"ncn_fused.hip": MAX_ILP, "ncn_fused_radix.hip": MAX_ILP, "ncn_fused_lengths.hip": MAX_ILP,
-               "ncn_fwd.hip": MAX_ILP}
+               "ncn_fwd.hip": MAX_ILP, "ncn_fwd_indexed.hip": MAX_ILP, "ncn_bwd_indexed.hip": MAX_ILP}
 
 
 def _hipcc():
