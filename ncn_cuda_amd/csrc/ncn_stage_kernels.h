@@ -246,6 +246,9 @@ __device__ __forceinline__ void backward_core(float (&Y)[R][F], float (&B)[R][F]
                                               float4* slots, int live = NC) {
     using T = Tile<NC, EC, R, F>;
     const int rl = (lane / T::LF) % T::LR;
+    float wiku[F];   // ku Wi': G += rh (ku Wi') spares the product ku rh of every row and step
+#pragma unroll
+    for (int f = 0; f < F; ++f) wiku[f] = S.ku * wi[f];
 #pragma unroll 1
     for (int jo = T::LR - 1; jo >= 0; --jo) {
         const float selku = (T::LR == 1 || rl == jo) ? S.ku : 0.0f;  // this lane holds the pivot row
@@ -290,12 +293,11 @@ __device__ __forceinline__ void backward_core(float (&Y)[R][F], float (&B)[R][F]
 #pragma unroll
             for (int rr = 0; rr < R; ++rr) {
                 const float rho_w = krho * rh[rr];     // (1-alpha) r_i / kappa, weighted
-                const float kr = S.ku * rh[rr];
                 rhosum += rh[rr];
 #pragma unroll
                 for (int f = 0; f < F; ++f) {
                     dwi[f] = fmaf(rho_w, Y[rr][f], dwi[f]);
-                    G[rr][f] = fmaf(kr, wi[f], G[rr][f]);
+                    G[rr][f] = fmaf(rh[rr], wiku[f], G[rr][f]);
                     if (rr != jr) P[rr][f] = fmaf(S.om, G[rr][f], P[rr][f]);
                 }
             }
