@@ -419,7 +419,7 @@ __device__ __forceinline__ void backward_steps(float (&Y)[R][F], float (&B)[R][F
     }
 
 template <int NC, int EC, int R, int F, bool TANH_ONLY = true, bool INDEXED = false>
-__global__ void __launch_bounds__(kBlockThreads, (TANH_ONLY && !INDEXED && R == 4 && F == 4) ? 6 : 1) stage_forward_kernel(const StageArgs A) {
+__global__ void __launch_bounds__(kBlockThreads, (TANH_ONLY && !INDEXED && R == 4 && F == 4) ? 5 : 1) stage_forward_kernel(const StageArgs A) {
     NCN_WAVE_PROLOGUE
     for (uint32_t t = gwave / A.n_head; t < A.total_tiles; t += tile_step) {
         int64_t off[R];
