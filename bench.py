@@ -144,9 +144,10 @@ def main():
                 cx, cxa = M.forward_radix(cx, cxa, Wst[a:a + cnt], alpha, 0, n, C, a, cnt)
                 saved.append((cx, cxa))
             elif tables is not None:
-                cx, cxa, y32, ya32 = M.forward_stages(cx, cxa, Wst[a], alpha, 0, n, C, a, 1, save_fp32=True,
-                                                      group_index=tables[a], ctx_len=lens, check_tables=False)
-                saved.append((y32, ya32))
+                # what the table-grouped autograd node keeps: two bf16 planes for bf16 storage, the outputs otherwise
+                cx, cxa, sy, sya = M.forward_stages_saving(cx, cxa, Wst[a], alpha, 0, n, C, a, group_index=tables[a],
+                                                           ctx_len=lens, check_tables=False)
+                saved.append((sy, sya))
             elif bf16 and cnt == 1:
                 # bf16 outputs plus what their rounding took away (a second bf16 plane): what the backward inverts
                 cx, cxa, ys, yas = M.forward_stages(cx, cxa, Wst[a], alpha, 0, n, C, a, 1, save_residual=True,
