@@ -3,6 +3,7 @@
 #include <vector>
 
 #include "ncn_fused_kernels.h"
+#include "ncn_fused_pair_kernels.h"
 #include "ncn_launch.h"
 
 namespace ncn {
@@ -20,7 +21,8 @@ constexpr int kFusedMaxGridBwd = 4096;           // backward: one dW partial row
 size_t fused_lds_bytes(int nc, int ec, bool backward, uint32_t window, int n_stages) {
     const TileShape t = fast_tile(nc, ec);
     const int lr = nc / t.r;
-    size_t bytes = (size_t)(backward ? 4 : 2) * window * nc * ec * sizeof(float);
+    // groups of two rows keep their slot-0 rows in registers (ncn_fused_pair_kernels.h): one row per group in LDS
+    size_t bytes = (size_t)(backward ? 4 : 2) * window * (nc == 2 ? 1 : nc) * ec * sizeof(float);
     bytes += (size_t)kFusedMaxStages * 2 * ec * sizeof(float);  // the pass's weights
     const int nw = backward ? kFusedWavesBwd : kFusedWavesFwd;
     if (lr > 1) bytes += (size_t)nw * t.f * 64 * sizeof(float);
@@ -63,7 +65,8 @@ std::vector<FusedPass> plan_fused(const ncn_shape* sh, int first, int count, boo
     std::vector<FusedPass> passes;
     const int nc = sh->n_cache, ec = (int)(sh->E / sh->n_head);
     const uint32_t groups = (uint32_t)(sh->N / nc);
-    const uint32_t cap_rows = (uint32_t)(fused_state_bytes(backward) / ((backward ? 4 : 2) * ec * sizeof(float)));
+    const size_t state = nc == 2 ? pair_state_bytes(backward) : fused_state_bytes(backward);
+    const uint32_t cap_rows = (uint32_t)(state / ((backward ? 4 : 2) * ec * sizeof(float)));
     uint32_t cap = floor_pow2(cap_rows / nc);
     if (cap > groups) cap = groups;
     if (cap < 4) return passes;
@@ -146,6 +149,26 @@ static hipError_t launch_fused_t(Pass pass, const FusedArgs& a, int grid, size_t
     static_assert(t.r != 0, "multi-stage shapes must be one-stage shapes too");
     hipError_t err;
     const bool tanh_only = a.tab.activation == NCN_ACT_TANH;
+    if constexpr (NC == 2) {
+        static_assert(t.r == 2 && t.f == 4, "the two-row kernels are written for 2 x 4 tiles");
+        if (backward) {
+            auto k = tanh_only ? pair_backward_kernel<EC, true> : pair_backward_kernel<EC, false>;
+            err = ensure_dynamic_lds(reinterpret_cast<const void*>(k), lds);
+            if (err != hipSuccess) return err;
+            hipLaunchKernelGGL(k, dim3(grid), dim3(64 * kFusedWavesBwd), lds, s, a);
+        } else if (pass == kInverse) {
+            auto k = tanh_only ? pair_forward_kernel<EC, true, true> : pair_forward_kernel<EC, false, true>;
+            err = ensure_dynamic_lds(reinterpret_cast<const void*>(k), lds);
+            if (err != hipSuccess) return err;
+            hipLaunchKernelGGL(k, dim3(grid), dim3(64 * kFusedWavesFwd), lds, s, a);
+        } else {
+            auto k = tanh_only ? pair_forward_kernel<EC, true> : pair_forward_kernel<EC, false>;
+            err = ensure_dynamic_lds(reinterpret_cast<const void*>(k), lds);
+            if (err != hipSuccess) return err;
+            hipLaunchKernelGGL(k, dim3(grid), dim3(64 * kFusedWavesFwd), lds, s, a);
+        }
+        return hipGetLastError();
+    } else
     if (backward) {
         auto k = tanh_only ? fused_backward_kernel<NC, EC, t.r, t.f, true> : fused_backward_kernel<NC, EC, t.r, t.f, false>;
         err = ensure_dynamic_lds(reinterpret_cast<const void*>(k), lds);

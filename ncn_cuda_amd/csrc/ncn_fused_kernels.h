@@ -47,6 +47,16 @@ constexpr int kFusedMaxStages = 8;
 constexpr size_t kFusedStateBytesFwd = NCN_FUSED_STATE_FWD;
 constexpr size_t kFusedStateBytesBwd = 64 * 1024;
 constexpr size_t fused_state_bytes(bool backward) { return backward ? kFusedStateBytesBwd : kFusedStateBytesFwd; }
+// Groups of two rows under the stride permutation keep half of a window in registers (ncn_fused_pair_kernels.h): the
+// bytes of both halves that one workgroup holds
+#ifndef NCN_PAIR_STATE_FWD
+#define NCN_PAIR_STATE_FWD (128 * 1024)
+#endif
+#ifndef NCN_PAIR_STATE_BWD
+#define NCN_PAIR_STATE_BWD (128 * 1024)
+#endif
+constexpr size_t kPairStateBytesFwd = NCN_PAIR_STATE_FWD, kPairStateBytesBwd = NCN_PAIR_STATE_BWD;
+constexpr size_t pair_state_bytes(bool backward) { return backward ? kPairStateBytesBwd : kPairStateBytesFwd; }
 #ifndef NCN_FUSED_WAVES_FWD
 #define NCN_FUSED_WAVES_FWD 8
 #endif

@@ -1,6 +1,7 @@
 // The multi-stage (LDS-resident) passes with one context length per batch entry: the LENGTHS builds of
 // ncn_fused_kernels.h, in a translation unit of their own so that they compile beside the plain ones.
 #include "ncn_fused_kernels.h"
+#include "ncn_fused_pair_kernels.h"
 #include "ncn_launch.h"
 
 namespace ncn {
@@ -17,6 +18,25 @@ hipError_t launch_t(Pass pass, const FusedArgs& a, int grid, size_t lds, hipStre
     static_assert(t.r != 0, "multi-stage shapes must be one-stage shapes too");
     const bool tanh_only = a.tab.activation == NCN_ACT_TANH;
     hipError_t err;
+    if constexpr (NC == 2) {
+        if (pass == kBackward) {
+            auto k = tanh_only ? pair_backward_kernel<EC, true, true> : pair_backward_kernel<EC, false, true>;
+            err = ensure_dynamic_lds(reinterpret_cast<const void*>(k), lds);
+            if (err != hipSuccess) return err;
+            hipLaunchKernelGGL(k, dim3(grid), dim3(64 * kFusedWavesBwd), lds, s, a);
+        } else if (pass == kInverse) {
+            auto k = tanh_only ? pair_forward_kernel<EC, true, true, true> : pair_forward_kernel<EC, false, true, true>;
+            err = ensure_dynamic_lds(reinterpret_cast<const void*>(k), lds);
+            if (err != hipSuccess) return err;
+            hipLaunchKernelGGL(k, dim3(grid), dim3(64 * kFusedWavesFwd), lds, s, a);
+        } else {
+            auto k = tanh_only ? pair_forward_kernel<EC, true, false, true> : pair_forward_kernel<EC, false, false, true>;
+            err = ensure_dynamic_lds(reinterpret_cast<const void*>(k), lds);
+            if (err != hipSuccess) return err;
+            hipLaunchKernelGGL(k, dim3(grid), dim3(64 * kFusedWavesFwd), lds, s, a);
+        }
+        return hipGetLastError();
+    } else
     if (pass == kBackward) {
         auto k = tanh_only ? fused_backward_kernel<NC, EC, t.r, t.f, true, false, true>
                            : fused_backward_kernel<NC, EC, t.r, t.f, false, false, true>;
