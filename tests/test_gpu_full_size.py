@@ -214,6 +214,30 @@ def test_headline_shape_with_table_and_lengths_against_the_c_oracle(M):
         assert O.rel_err(dWs[l][0].cpu(), ref[4][l]) < tol, l
 
 
+def test_deep_shape_with_lengths_against_the_c_oracle(M):
+    """cfg4 with one context length per batch entry and no table: the multi-stage passes for groups of two rows in their
+    LENGTHS build (13 stages in two passes forward, three backward), every element against the C oracle in float64 on
+    the stride tables with the same lengths."""
+    from oracle import c_oracle as CO
+    batch, N, E, C, n, L, dtype, _ = CONFIGS["cfg4"]
+    x, xa, dy, W = _inputs("cfg4")
+    lens = (N - 1 - 61 * torch.arange(batch)) % (N + 1)
+    lens[0], lens[1], lens[2] = N, 0, 1
+    gl = lens.to(torch.int32).cuda()
+    y, ya = M.forward_stages(x, xa, W, 0.9, 0, n, C, 0, L, ctx_len=gl)
+    xr, xar, dx, dxa, dW = M.backward_stages(y, ya, dy, None, W, 0.9, 0, n, C, 0, L, ctx_len=gl)
+    tables = [O.stride_group_table(N, n, l) for l in range(L)]
+    d = torch.float64
+    ref = CO.net_forward_backward(x.cpu().to(d), xa.cpu().to(d), [w.cpu().to(d) for w in W], dy.cpu().to(d), None, 0.9, n,
+                                  C, tables=tables, ctx_len=lens, keep_outputs=False)
+    errs = {"y": O.rel_err(y.cpu(), ref[0]), "ya": O.rel_err(ya.cpu(), ref[1]), "dx": O.rel_err(dx.cpu(), ref[2]),
+            "dxa": O.rel_err(dxa.cpu(), ref[3]), "x_rec": O.rel_err(xr.cpu(), x.cpu().to(d)),
+            "dW_worst": max(O.rel_err(dW[l].cpu(), ref[4][l]) for l in range(L))}
+    print("measured errors cfg4 with lengths: " + json.dumps(errs))
+    for k, v in errs.items():
+        assert v < 1e-5, (k, v)
+
+
 def test_deep_shape_radix_levels_against_the_c_oracle(M):
     """cfg4's tensors through the 13 levels of the radix-2 grouping (two multi-level LDS passes each way), every element
     against the C oracle in float64 on the radix tables."""
