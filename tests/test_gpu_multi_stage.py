@@ -27,6 +27,8 @@ CASES = [
     (1, 256, 32, 1, 2, 0, 8),      # one head; whole ring fits the window from the start
     (5, 64, 128, 4, 4, 0, 3),      # tiny ring (16 groups)
     (2, 256, 64, 2, 2, 1000003, 3),  # a very high first stage: 2^(stage-1) mod groups is 0 from stage log2(groups)+1 on
+    (3, 2048, 64, 4, 2, 0, 10),    # n = 2, head width 16 (16 groups per wave tile, windows of 512 groups)
+    (2, 16, 32, 1, 2, 0, 3),       # n = 2, 8 groups: a window smaller than one wave tile per wave
 ]
 
 
