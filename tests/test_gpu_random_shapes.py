@@ -114,6 +114,8 @@ def test_random_problem(M, case):
         if (1 / 0.9) ** (n * levels) < 50:
             rxr, _, rdx, rdxa, rdW = M.backward_radix(ry, rya, gdy, gdya, W[:levels], alpha, act, n, C, 0, levels)
             tol = max(1e-5, 2e-6 * (1 / 0.9) ** (n * levels))
-            assert O.rel_err(rdx, rref[2]) < tol and O.rel_err(rdxa, rref[3]) < tol and O.rel_err(rxr, x) < tol
+            assert O.rel_err(rdx, rref[2]) < tol and O.rel_err(rdxa, rref[3]) < tol
+            # the reconstruction carries the rounding of every step it undoes: 1e-5 x (1/m)^(steps), as above
+            assert O.rel_err(rxr, x) < max(3e-5, 1e-5 * (1 / 0.9) ** (n * levels))
             for l in range(levels):
                 assert O.rel_err(rdW[l], rref[4][l]) < tol
