@@ -24,8 +24,9 @@
  *
  * Pinning: tests/test_oracle_c.py checks the double build against the float64 vectors the reference's own CPU code
  * produced (tests/golden, 1e-12), the float build against its float32 vectors and against the vectors of the
- * reference's Triton kernels, and both against oracle/ncn_oracle.py on random shapes.  Parity unpinned: relu and
- * sigmoid (no runnable reference statement), as in the Python oracle.
+ * reference's Triton kernels, and both against oracle/ncn_oracle.py on random shapes.  relu and sigmoid, which no
+ * vector of the reference covers, are held to the Python oracle there, which pins them by what the mathematics fixes
+ * (tests/test_oracle_properties.py).  Parity unpinned, as in the Python oracle: the pass-through of rows past a length.
  *
  * Built twice from this one file: -DREAL=float (suffix _f32, what the baseline times) and -DREAL=double (_f64).
  * Groups are independent, so the loops over them are OpenMP-parallel; dW is summed per thread in double and the
