@@ -286,7 +286,12 @@ size_t ncn_workspace_bytes(const ncn_shape* shape);
 
 /* Bytes of scratch that let ncn_forward (backward = 0) or ncn_backward (backward = 1) run stages
  * first_stage .. first_stage+n_stages-1 with the multi-stage passes; never less than what the call needs anyway
- * (0 for forward, ncn_workspace_bytes for backward).  No reference counterpart. */
+ * (0 for forward, ncn_workspace_bytes for backward).  For the backward that is, in this order: a dW partial row of
+ * 2E floats for every window and stage of every pass (at most 65536 rows, at least those of ncn_workspace_bytes)
+ * with their chunk sums, so that every window gets a workgroup of its own, and, with two passes or more, four
+ * float32 arrays of the tensors' size.  ncn_backward also takes ncn_workspace_bytes(shape) plus the four arrays
+ * (each padded to a multiple of 256 bytes) and then lets its workgroups walk over several windows, which is slower.
+ * No reference counterpart. */
 size_t ncn_workspace_bytes_stages(const ncn_shape* shape, int first_stage, int n_stages, int activation, int backward);
 
 /* How ncn_forward / ncn_backward would cut stages first_stage .. first_stage+n_stages-1 into passes, for

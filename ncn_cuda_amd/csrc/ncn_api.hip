@@ -230,9 +230,14 @@ int edge_rows(const ncn_shape* sh) { return (int)(sh->batch < kEdgeGridX ? sh->b
 
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
+// rows of chunk sums that the launches of one reduction job can need when they fill row_cap partial rows
+int level1_rows(int row_cap) {
+    const int r = row_cap / kReduceRowsPerBlock + kReduceMaxStages;
+    return r > kReduceLevel1Rows ? r : kReduceLevel1Rows;
+}
 // dW partial rows of the backward launches of a call, then the chunk sums of the first reduction level
 size_t partial_buffer_bytes(const ncn_shape* sh, int row_cap) {
-    return align256((size_t)(row_cap + kReduceLevel1Rows) * 2 * (size_t)sh->E * sizeof(float));
+    return align256((size_t)(row_cap + level1_rows(row_cap)) * 2 * (size_t)sh->E * sizeof(float));
 }
 size_t base_workspace_bytes(const ncn_shape* sh) { return partial_buffer_bytes(sh, kMaxGridX); }
 
@@ -245,6 +250,18 @@ std::vector<FusedPass> multi_stage_plan(const ncn_shape* sh, int first_stage, in
     bool any = false;
     for (const FusedPass& p : passes) any = any || !p.single;
     return any ? passes : none;
+}
+
+// Partial rows that the backward passes of a plan fill when every window has a workgroup of its own (rows * stages,
+// summed over the passes, which lie side by side in the buffer), between what every workspace holds and
+// kFusedRowCapMax (64 MB at E = 128).
+constexpr int kFusedRowCapMax = 65536;
+int fused_rows_wanted(const ncn_shape* sh, const std::vector<FusedPass>& passes) {
+    int64_t rows = 0;
+    for (const FusedPass& p : passes)
+        rows += p.single ? (int64_t)kMaxGridX : fused_items(sh, p) / sh->n_head * p.count;
+    if (rows > kFusedRowCapMax) rows = kFusedRowCapMax;
+    return rows < kMaxGridX ? kMaxGridX : (int)rows;
 }
 
 size_t temp_bytes(const ncn_shape* sh, bool backward) {
@@ -341,7 +358,7 @@ hipError_t static_scratch(float** out) {
 
 extern "C" {
 
-const char* ncn_version(void) { return "0.8"; }
+const char* ncn_version(void) { return "0.9"; }
 
 int ncn_plan_passes(const ncn_shape* shape, int first_stage, int n_stages, int activation, int backward, int32_t* out,
                     int max_passes) {
@@ -401,8 +418,9 @@ size_t ncn_workspace_bytes(const ncn_shape* shape) {
 
 size_t ncn_workspace_bytes_stages(const ncn_shape* shape, int first_stage, int n_stages, int activation, int backward) {
     if (check_shape(shape, first_stage, n_stages, activation) != NCN_OK) return 0;
-    const size_t base = backward ? base_workspace_bytes(shape) : 0;
     const std::vector<FusedPass> passes = multi_stage_plan(shape, first_stage, n_stages, activation, backward != 0);
+    const size_t base = !backward ? 0 : passes.empty() ? base_workspace_bytes(shape)
+                                                        : partial_buffer_bytes(shape, fused_rows_wanted(shape, passes));
     return passes.size() >= 2 ? base + temp_bytes(shape, backward != 0) : base;
 }
 
@@ -683,18 +701,26 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
         passes = multi_stage_plan(shape, first_stage, n_stages, activation, true, path);
     const size_t np = passes.size();
     bool fused_ok = np > 0;
-    if (np >= 2 && workspace_bytes < base_workspace_bytes(shape) + temp_bytes(shape, true)) fused_ok = false;
+    // a workspace of ncn_workspace_bytes_stages() holds a partial row for every window of every pass; a smaller one
+    // (ncn_workspace_bytes() and the four arrays) makes the workgroups loop over windows
+    int fused_cap = kMaxGridX;
+    if (np > 0) {
+        const int want = fused_rows_wanted(shape, passes);
+        if (workspace_bytes >= partial_buffer_bytes(shape, want) + (np >= 2 ? temp_bytes(shape, true) : 0)) fused_cap = want;
+    }
+    const size_t fused_base = partial_buffer_bytes(shape, fused_cap);
+    if (np >= 2 && workspace_bytes < fused_base + temp_bytes(shape, true)) fused_ok = false;
     if (np >= 1 && ((np - 1) % 2) == 0 && !passes[np - 1].closed && !passes[np - 1].single &&
         (y == x_rec || ya == xa_rec || dy == dx || (dya && dya == dxa)))
         fused_ok = false;  // the first pass to run is a halo pass and would write into its own input
     if (fused_ok) {
         const size_t one = temp_bytes(shape, true) / 4;
-        char* tb = static_cast<char*>(workspace) + base_workspace_bytes(shape);
+        char* tb = static_cast<char*>(workspace) + fused_base;
         float* t[4] = {reinterpret_cast<float*>(tb), reinterpret_cast<float*>(tb + one),
                        reinterpret_cast<float*>(tb + 2 * one), reinterpret_cast<float*>(tb + 3 * one)};
         const void* cy = y; const void* cya = ya; int cy_dtype = y_dtype;
         const void* cg = dy; const void* cga = dya; int cg_dtype = dy_dtype;
-        DwReducer reducer(partials, level1, wstride, s);
+        DwReducer reducer(partials, partials + (int64_t)fused_cap * wstride, wstride, s, fused_cap);
         for (size_t e = 0; e < np; ++e) {
             const FusedPass& ps = passes[np - 1 - e];
             const bool to_out = ((np - 1 - e) % 2) == 0;
@@ -704,7 +730,7 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
             void* ddxa = to_out ? dxa : static_cast<void*>(t[3]);
             const int d_dtype = to_out ? dx_dtype : NCN_F32;
             // a partial row of a multi-stage pass holds its stages side by side, as dW does
-            const int rows = ps.single ? p.partial_rows : fused_grid(shape, ps, true) / shape->n_head;
+            const int rows = ps.single ? p.partial_rows : fused_grid(shape, ps, true, fused_cap) / shape->n_head;
             float* region;
             hipError_t err = reducer.reserve(rows, ps.count, &region);
             if (err != hipSuccess) return (int)err;
@@ -731,7 +757,7 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
                 a.dw_partials = region;
                 a.ctx_len = grouping.ctx_len;
                 fill_step_table(a.tab, shape->n_cache, alpha, m, activation);
-                err = launch_fused(kBackward, a, shape, ps, s);
+                err = launch_fused(kBackward, a, shape, ps, s, fused_cap);
             }
             if (err != hipSuccess) return (int)err;
             reducer.add(region, rows, ps.count, dW + ps.first * wstride);

@@ -1,4 +1,5 @@
 // Planning and launching of the multi-stage (LDS-resident) passes; kernels in ncn_fused_kernels.h.
+#include <climits>
 #include <cmath>
 #include <vector>
 
@@ -15,8 +16,13 @@ namespace {
 #define NCN_FOR_EACH_FUSED_CONFIG(X) \
     X(2, 16) X(4, 16) X(2, 32) X(4, 32)
 
-constexpr int kFusedMaxGridFwd = 4096;           // forward: a few windows per workgroup, so that each can fetch its next one early
-constexpr int kFusedMaxGridBwd = 4096;           // backward: one dW partial row per n_head workgroups and stage
+// One window per workgroup wherever the problem allows: workgroups that start and end on their own fall out of step
+// with their neighbours on the CU, so that the loads and stores of one run under the stages of the other; a workgroup
+// that loops over several windows keeps the phase it started in (measured on the 13-stage configuration: grids of
+// 4096 workgroups, 4.5 windows each, 5.35 ms per step; one window each 4.94).  The backward is further bounded by its
+// dW partial rows (one per n_head workgroups and stage), see fused_grid.
+constexpr int kFusedMaxGridFwd = 1 << 16;
+constexpr int kFusedMaxGridBwd = 1 << 16;
 
 size_t fused_lds_bytes(int nc, int ec, bool backward, uint32_t window, int n_stages) {
     const TileShape t = fast_tile(nc, ec);
@@ -24,7 +30,7 @@ size_t fused_lds_bytes(int nc, int ec, bool backward, uint32_t window, int n_sta
     // groups of two rows keep their slot-0 rows in registers (ncn_fused_pair_kernels.h): one row per group in LDS
     size_t bytes = (size_t)(backward ? 4 : 2) * window * (nc == 2 ? 1 : nc) * ec * sizeof(float);
     bytes += (size_t)kFusedMaxStages * 2 * ec * sizeof(float);  // the pass's weights
-    const int nw = backward ? kFusedWavesBwd : kFusedWavesFwd;
+    const int nw = backward ? (nc == 2 ? kPairWavesBwd : kFusedWavesBwd) : kFusedWavesFwd;
     if (lr > 1) bytes += (size_t)nw * t.f * 64 * sizeof(float);
     if (backward) bytes += (size_t)nw * n_stages * 2 * ec * sizeof(float);
     return bytes;
@@ -151,11 +157,15 @@ static hipError_t launch_fused_t(Pass pass, const FusedArgs& a, int grid, size_t
     const bool tanh_only = a.tab.activation == NCN_ACT_TANH;
     if constexpr (NC == 2) {
         static_assert(t.r == 2 && t.f == 4, "the two-row kernels are written for 2 x 4 tiles");
+        if (!backward && (uint32_t)grid != a.total_items) return hipErrorInvalidConfiguration;   // one window each
         if (backward) {
-            auto k = tanh_only ? pair_backward_kernel<EC, true> : pair_backward_kernel<EC, false>;
+            // a workgroup per window when the dW scratch has the rows for it, else workgroups that loop over windows
+            const bool loop = (uint32_t)grid < a.total_items;
+            auto k = tanh_only ? (loop ? pair_backward_kernel<EC, true, false, true> : pair_backward_kernel<EC, true, false, false>)
+                               : (loop ? pair_backward_kernel<EC, false, false, true> : pair_backward_kernel<EC, false, false, false>);
             err = ensure_dynamic_lds(reinterpret_cast<const void*>(k), lds);
             if (err != hipSuccess) return err;
-            hipLaunchKernelGGL(k, dim3(grid), dim3(64 * kFusedWavesBwd), lds, s, a);
+            hipLaunchKernelGGL(k, dim3(grid), dim3(64 * kPairWavesBwd), lds, s, a);
         } else if (pass == kInverse) {
             auto k = tanh_only ? pair_forward_kernel<EC, true, true> : pair_forward_kernel<EC, false, true>;
             err = ensure_dynamic_lds(reinterpret_cast<const void*>(k), lds);
@@ -189,11 +199,17 @@ static hipError_t launch_fused_t(Pass pass, const FusedArgs& a, int grid, size_t
     return hipGetLastError();
 }
 
-int fused_grid(const ncn_shape* sh, const FusedPass& p, bool backward) {
-    const int64_t items = sh->batch * (int64_t)p.class_groups * p.tiles_per_ring * sh->n_head;
+int64_t fused_items(const ncn_shape* sh, const FusedPass& p) {
+    return sh->batch * (int64_t)p.class_groups * p.tiles_per_ring * sh->n_head;
+}
+
+int fused_grid(const ncn_shape* sh, const FusedPass& p, bool backward, int row_cap) {
+    const int64_t items = fused_items(sh, p);
+    // the forward kernels for groups of two rows take one window per workgroup and nothing else
+    if (!backward && sh->n_cache == 2) return items <= INT_MAX ? (int)items : 0;
     int64_t cap = backward ? kFusedMaxGridBwd : kFusedMaxGridFwd;
-    if (backward) {  // partial rows (grid / n_head) * stages must fit the kMaxGridX rows of the dW scratch
-        const int64_t by_rows = (int64_t)kMaxGridX / p.count * sh->n_head;
+    if (backward) {  // partial rows (grid / n_head) * stages must fit the row_cap rows of the dW scratch
+        const int64_t by_rows = (int64_t)row_cap / p.count * sh->n_head;
         if (by_rows < cap) cap = by_rows;
     }
     int64_t g = items < cap ? items : cap;
@@ -202,7 +218,7 @@ int fused_grid(const ncn_shape* sh, const FusedPass& p, bool backward) {
     return (int)g;
 }
 
-hipError_t launch_fused(Pass pass, FusedArgs& a, const ncn_shape* sh, const FusedPass& p, hipStream_t s) {
+hipError_t launch_fused(Pass pass, FusedArgs& a, const ncn_shape* sh, const FusedPass& p, hipStream_t s, int row_cap) {
     const bool backward = pass == kBackward;
     const int nc = sh->n_cache, ec = (int)(sh->E / sh->n_head);
     a.N = sh->N;
@@ -217,11 +233,11 @@ hipError_t launch_fused(Pass pass, FusedArgs& a, const ncn_shape* sh, const Fuse
     a.tiles_per_ring = p.tiles_per_ring;
     a.closed = p.closed;
     a.class_groups = p.class_groups;
-    a.total_items = (uint32_t)(sh->batch * (int64_t)p.class_groups * p.tiles_per_ring * sh->n_head);
+    a.total_items = (uint32_t)fused_items(sh, p);
     for (int k = 0; k < kFusedMaxStages; ++k) a.sub_stride[k] = k < p.count ? p.sub_stride[k] : 0;
     a.scale_dn = (float)std::pow((double)a.tab.m, (double)(nc * p.count));
     a.scale_up = (float)std::pow((double)a.tab.m, -(double)(nc * p.count));
-    const int grid = fused_grid(sh, p, backward);
+    const int grid = fused_grid(sh, p, backward, row_cap);
     const size_t lds = fused_lds_bytes(nc, ec, backward, p.window, p.count);
     if (a.ctx_len) return launch_fused_lengths(pass, a, nc, ec, grid, lds, s);
 #define NCN_CASE(NC, EC) \

@@ -19,11 +19,14 @@ hipError_t launch_t(Pass pass, const FusedArgs& a, int grid, size_t lds, hipStre
     const bool tanh_only = a.tab.activation == NCN_ACT_TANH;
     hipError_t err;
     if constexpr (NC == 2) {
+        if (pass != kBackward && (uint32_t)grid != a.total_items) return hipErrorInvalidConfiguration;
         if (pass == kBackward) {
-            auto k = tanh_only ? pair_backward_kernel<EC, true, true> : pair_backward_kernel<EC, false, true>;
+            const bool loop = (uint32_t)grid < a.total_items;   // see launch_fused_t
+            auto k = tanh_only ? (loop ? pair_backward_kernel<EC, true, true, true> : pair_backward_kernel<EC, true, true, false>)
+                               : (loop ? pair_backward_kernel<EC, false, true, true> : pair_backward_kernel<EC, false, true, false>);
             err = ensure_dynamic_lds(reinterpret_cast<const void*>(k), lds);
             if (err != hipSuccess) return err;
-            hipLaunchKernelGGL(k, dim3(grid), dim3(64 * kFusedWavesBwd), lds, s, a);
+            hipLaunchKernelGGL(k, dim3(grid), dim3(64 * kPairWavesBwd), lds, s, a);
         } else if (pass == kInverse) {
             auto k = tanh_only ? pair_forward_kernel<EC, true, true, true> : pair_forward_kernel<EC, false, true, true>;
             err = ensure_dynamic_lds(reinterpret_cast<const void*>(k), lds);

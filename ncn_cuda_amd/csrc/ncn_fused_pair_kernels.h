@@ -14,26 +14,31 @@
 
 namespace ncn {
 
-// Build parameters, with what was measured on the 13-stage configuration (x[128, 8192, 128], A/B on one box; the
-// general kernels 6.02 ms per step): windows as there (64 KB of rows counting both halves) with the next window
-// prefetched into registers 5.85; without the prefetch, which frees the registers for 6 waves per SIMD (three
-// workgroups per CU), 5.70; windows of 128 KB (the LDS holds half: two workgroups per CU as in the general kernels)
-// forward 5.51, backward too 5.33; the forward prefetch on top of that 5.58; a 256 KB forward window (one workgroup per
-// CU) 6.55; forcing 6 or 8 waves per SIMD where the code does not fit (spills) 6.2 - 11.6.
+// One window per workgroup: the forward is launched with as many workgroups as windows, the backward too whenever
+// the dW scratch has a partial row for each (LOOP = false).  Workgroups that come and go on their own fall out of step
+// with the other workgroup of their CU, so that the loads and stores of one run under the stages of the other, and
+// straight-line code needs no registers for what a loop over windows would carry around it (backward: 128 registers and
+// no spill, against 26 spilled registers inside the loop; forward 84 against 125).  The LOOP build of the backward, for
+// problems with more windows than partial rows, walks its windows with the next one's slot-1 rows requested before the
+// current one is written out.
+// Measured on the 13-stage configuration (x[128, 8192, 128], A/B on one box; the general kernels 6.02 ms per step):
+// windows as there (64 KB of rows counting both halves) 5.70 - 5.85; windows of 128 KB (the LDS holds half: two
+// workgroups per CU as in the general kernels) forward 5.51, backward too 5.33; a 256 KB forward window (one workgroup
+// per CU) 6.55; forcing 6 or 8 waves per SIMD where the code does not fit (spills) 6.2 - 11.6; all of these with grids
+// of 4096 workgroups that loop over 4.5 windows each.  One window per workgroup with the loop still compiled in 4.92;
+// without it 4.68.
 #ifndef NCN_PAIR_FWD_WAVES
 #define NCN_PAIR_FWD_WAVES 4     // waves per SIMD the forward is compiled for (register budget)
 #endif
 #ifndef NCN_PAIR_BWD_WAVES
 #define NCN_PAIR_BWD_WAVES 4
 #endif
-#ifndef NCN_PAIR_FWD_PREFETCH
-#define NCN_PAIR_FWD_PREFETCH 0  // 1: the forward requests its next window before it computes the current one
-#endif
+constexpr int kPairWavesBwd = kFusedWavesBwd;   // waves per workgroup of the backward
 
 // wave tiles per wave and stage at the largest window (forward: 128 KB of rows = 256 groups at Ec = 32 over 8 waves
 // of 8 groups = 4; backward: 128 groups = 2)
 constexpr int kPairTilesFwd = (int)(kPairStateBytesFwd / (2 * 2 * 4 * 4 * 64 * kFusedWavesFwd));
-constexpr int kPairTilesBwd = (int)(kPairStateBytesBwd / (4 * 2 * 4 * 4 * 64 * kFusedWavesBwd));
+constexpr int kPairTilesBwd = (int)((kPairStateBytesBwd + 4 * 2 * 4 * 4 * 64 * kPairWavesBwd - 1) / (4 * 2 * 4 * 4 * 64 * kPairWavesBwd));
 static_assert(kPairTilesFwd >= 1 && kPairTilesBwd >= 1, "a window holds at least one wave tile per wave");
 
 // Chunk offsets of the slot-1 rows of a window (row 1 of window sub-block qi is local row 2 qi + 1), for the
@@ -116,12 +121,12 @@ __global__ void __launch_bounds__(64 * kFusedWavesFwd, NCN_PAIR_FWD_WAVES) pair_
         fused_fetch_rows<KT>(A.in0, A.in_dtype, off0, r0x);
         fused_fetch_rows<KT>(A.in1, A.in_dtype, off0, r0a);
     };
-    if (NCN_PAIR_FWD_PREFETCH && blockIdx.x < A.total_items) fetch(blockIdx.x);
-    for (uint32_t item = blockIdx.x; item < A.total_items; item += gridDim.x) {
+    const uint32_t item = blockIdx.x;   // the launch has a workgroup for every window
+    if (item < A.total_items) {
         const FusedItem it = fused_item<NC, EC, false>(A, item);
         const int32_t len = LENGTHS ? max(0, min(A.ctx_len[it.batch], (int32_t)A.N)) : 0;
         float x0[KT][F], a0[KT][F];   // slot-0 rows of this lane's groups, scaled form
-        if (!NCN_PAIR_FWD_PREFETCH) fetch(item);
+        fetch(item);
         pair_commit_slot1<EC, NW, K1>(r1x, A.in_dtype, xs1, window, A.tab.kappa);
         pair_commit_slot1<EC, NW, K1>(r1a, A.in_dtype, as1, window, a_in);
 #pragma unroll
@@ -135,7 +140,6 @@ __global__ void __launch_bounds__(64 * kFusedWavesFwd, NCN_PAIR_FWD_WAVES) pair_
             }
         }
         __syncthreads();
-        if (NCN_PAIR_FWD_PREFETCH && item + gridDim.x < A.total_items) fetch(item + gridDim.x);   // travels while this window is computed
         for (int sq = 0; sq < A.n_stages; ++sq) {
             const int st = INVERSE ? A.n_stages - 1 - sq : sq;
             const uint32_t ss = A.sub_stride[st];
@@ -212,13 +216,12 @@ __global__ void __launch_bounds__(64 * kFusedWavesFwd, NCN_PAIR_FWD_WAVES) pair_
                 }
             }
         }
-        __syncthreads();   // every thread has read the LDS rows it writes out: the next window may land
     }
 }
 
-template <int EC, bool TANH_ONLY, bool LENGTHS = false>
-__global__ void __launch_bounds__(64 * kFusedWavesBwd, TANH_ONLY ? NCN_PAIR_BWD_WAVES : 1) pair_backward_kernel(const FusedArgs A) {
-    constexpr int NC = 2, R = 2, F = 4, NW = kFusedWavesBwd, KT = kPairTilesBwd;
+template <int EC, bool TANH_ONLY, bool LENGTHS = false, bool LOOP = false>
+__global__ void __launch_bounds__(64 * kPairWavesBwd, TANH_ONLY ? NCN_PAIR_BWD_WAVES : 1) pair_backward_kernel(const FusedArgs A) {
+    constexpr int NC = 2, R = 2, F = 4, NW = kPairWavesBwd, KT = kPairTilesBwd;
     using T = Tile<NC, EC, R, F>;
     static_assert(T::LR == 1, "both rows of a group in one lane");
     constexpr uint32_t CPR = EC / 4;
@@ -305,7 +308,8 @@ __global__ void __launch_bounds__(64 * kFusedWavesBwd, TANH_ONLY ? NCN_PAIR_BWD_
         commit(first);
     }
     __syncthreads();
-    for (uint32_t item = blockIdx.x; item < A.total_items; item += gridDim.x) {
+    uint32_t item = blockIdx.x;
+    if (item < A.total_items) do {
         const FusedItem it = fused_item<NC, EC, false>(A, item);
         const int32_t len = LENGTHS ? max(0, min(A.ctx_len[it.batch], (int32_t)A.N)) : 0;
         for (int st = A.n_stages - 1; st >= 0; --st) {
@@ -453,7 +457,7 @@ __global__ void __launch_bounds__(64 * kFusedWavesBwd, TANH_ONLY ? NCN_PAIR_BWD_
                 }
             }
         };
-        if (item + gridDim.x < A.total_items) {   // the same for the whole workgroup
+        if (LOOP && item + gridDim.x < A.total_items) {   // the same for the whole workgroup
             Raw next;
             fetch(item + gridDim.x, next);
             write_out();
@@ -464,7 +468,7 @@ __global__ void __launch_bounds__(64 * kFusedWavesBwd, TANH_ONLY ? NCN_PAIR_BWD_
             write_out();
         }
         __syncthreads();
-    }
+    } while (LOOP && (item += gridDim.x) < A.total_items);
     // one partial row per workgroup and stage; workgroup b owns slot (b / n_head, head b % n_head)
     float* prow = A.dw_partials + (int64_t)(blockIdx.x / A.n_head) * A.n_stages * (2 * A.E);
     for (int k = threadIdx.x; k < A.n_stages * 2 * EC; k += 64 * NW) {

@@ -86,8 +86,12 @@ struct FusedPass {
 };
 bool fused_supported(const ncn_shape* sh, int activation);
 std::vector<FusedPass> plan_fused(const ncn_shape* sh, int first, int count, bool backward);
-int fused_grid(const ncn_shape* sh, const FusedPass& p, bool backward);
-hipError_t launch_fused(Pass pass, FusedArgs& a, const ncn_shape* sh, const FusedPass& p, hipStream_t s);
+// windows of a pass (== workgroups, when every workgroup takes one)
+int64_t fused_items(const ncn_shape* sh, const FusedPass& p);
+// row_cap: rows of the dW partial buffer a backward pass may fill (grid / n_head rows per stage)
+int fused_grid(const ncn_shape* sh, const FusedPass& p, bool backward, int row_cap = kMaxGridX);
+hipError_t launch_fused(Pass pass, FusedArgs& a, const ncn_shape* sh, const FusedPass& p, hipStream_t s,
+                        int row_cap = kMaxGridX);
 // the builds with context lengths (a.ctx_len set), ncn_fused_lengths.hip; launch_fused goes there by itself
 hipError_t launch_fused_lengths(Pass pass, const FusedArgs& a, int nc, int ec, int grid, size_t lds, hipStream_t s);
 

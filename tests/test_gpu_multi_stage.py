@@ -213,3 +213,42 @@ def test_dw_of_a_call_equals_dw_of_its_stages(M, case):
     # and a second identical call reproduces every bit
     _, _, _, _, dW2 = M.backward_stages(outs[-1][0], outs[-1][1], gdy, None, torch.stack(gWs), alpha, 0, n, C, first, L)
     assert torch.equal(dW, dW2)
+
+
+def test_backward_with_the_smaller_workspace_loops_over_windows(M):
+    """ncn_backward gives every window of a multi-stage pass a workgroup of its own when the workspace has a dW partial
+    row for each (ncn_workspace_bytes_stages); with ncn_workspace_bytes plus the four float32 arrays, which every
+    version of the library accepted, the workgroups of a pass that does not fit walk over several windows (the other
+    build of the kernel).  Same windows, same arithmetic: dx, dxa and the reconstructed inputs must be bit-identical,
+    dW equal up to the order of its partial sums."""
+    import ctypes
+    from ncn_cuda_amd import _lib
+    batch, N, E, C, n, L = 80, 8192, 128, 4, 2, 13     # 80 x 32 closed windows per head x 7 stages > 16384 partial rows
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(3)
+    x = torch.randn(batch, N, E, device=dev, generator=g)
+    xa = torch.randn(batch, N, E, device=dev, generator=g) * 0.1
+    dy = torch.randn(batch, N, E, device=dev, generator=g)
+    dya = torch.randn(batch, N, E, device=dev, generator=g)
+    W = torch.randn(L, 2 * E, device=dev, generator=g) * (E // C) ** -0.5
+    y, ya = M.forward_stages(x, xa, W, 0.9, 0, n, C, 0, L)
+    ref = M.backward_stages(y, ya, dy, dya, W, 0.9, 0, n, C, 0, L)
+
+    lib = _lib.load()
+    shape = _lib.NcnShape(batch, N, E, C, n)
+    plane = (batch * N * E * 4 + 255) // 256 * 256
+    small = lib.ncn_workspace_bytes(ctypes.byref(shape)) + 4 * plane
+    assert small < lib.ncn_workspace_bytes_stages(ctypes.byref(shape), 0, L, 0, 1)
+    ws = torch.empty(small, dtype=torch.uint8, device=dev)
+    out = [torch.empty_like(x) for _ in range(4)]       # dx, dxa, x_rec, xa_rec
+    dW = torch.empty(L, 2 * E, device=dev)
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    rc = lib.ncn_backward(p(y), p(ya), 0, p(dy), p(dya), 0, p(out[0]), p(out[1]), 0, p(out[2]), p(out[3]), p(W), p(dW),
+                          p(ws), ctypes.c_size_t(small), ctypes.byref(shape), 0, L, 0.9, 0.9, 0,
+                          ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream))
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out[2], ref[0]) and torch.equal(out[3], ref[1])
+    assert torch.equal(out[0], ref[2]) and torch.equal(out[1], ref[3])
+    assert O.rel_err(dW, ref[4]) < 1e-6
+    assert O.rel_err(ref[0], x) < 1e-4      # and both are the inputs again (26 steps undone)
