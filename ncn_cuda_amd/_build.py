@@ -13,8 +13,8 @@ from concurrent.futures import ThreadPoolExecutor
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libncn_hip.so")
-SOURCES = ["ncn_api.hip", "ncn_fwd.hip", "ncn_bwd.hip", "ncn_fwd_indexed.hip", "ncn_bwd_indexed.hip", "ncn_generic.hip",
-           "ncn_fused.hip", "ncn_fused_radix.hip", "ncn_fused_lengths.hip"]
+SOURCES = ["ncn_api.hip", "ncn_fwd.hip", "ncn_bwd.hip", "ncn_bwd_once.hip", "ncn_fwd_indexed.hip", "ncn_bwd_indexed.hip",
+           "ncn_generic.hip", "ncn_fused.hip", "ncn_fused_radix.hip", "ncn_fused_lengths.hip"]
 # packed-fp32 VALU instructions are switched off for device code on purpose (flag is device-only;
 # the host pass prints a harmless "not a recognized feature" note).
 HIPCC_FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17",
@@ -23,11 +23,12 @@ HIPCC_FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17",
 
 # Instruction scheduling per translation unit.  The multi-stage kernels wait on latency (LDS, barriers, dependent
 # chains of two-row tiles): LLVM's max-ILP strategy measured 2.5 % on the 13-stage configuration, 1.5 % on the
-# one-stage forward and 1.2 % on a step through the table builds; the plain one-stage backward is bound by issue slots
-# and does not care.
+# one-stage forward and 1.2 % on a step through the table builds; the plain one-stage backward with its loop over
+# tiles is bound by issue slots and does not care, its form without the loop gains 2.5 % at 16 rows per group.
 MAX_ILP = ["-mllvm", "-amdgpu-sched-strategy=max-ilp"]
 EXTRA_FLAGS = {"ncn_fused.hip": MAX_ILP, "ncn_fused_radix.hip": MAX_ILP, "ncn_fused_lengths.hip": MAX_ILP,
-               "ncn_fwd.hip": MAX_ILP, "ncn_fwd_indexed.hip": MAX_ILP, "ncn_bwd_indexed.hip": MAX_ILP}
+               "ncn_fwd.hip": MAX_ILP, "ncn_fwd_indexed.hip": MAX_ILP, "ncn_bwd_indexed.hip": MAX_ILP,
+               "ncn_bwd_once.hip": MAX_ILP}
 
 
 def _hipcc():

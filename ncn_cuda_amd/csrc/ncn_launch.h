@@ -68,6 +68,8 @@ hipError_t ensure_dynamic_lds(const void* kernel, size_t bytes);
 
 hipError_t launch_fast_forward(Pass pass, const StageArgs& a, int n_head, int grid_x, hipStream_t s);
 hipError_t launch_fast_backward(const StageArgs& a, int n_head, int grid_x, hipStream_t s);
+// the same for a grid that has a wave for every tile (ncn_bwd_once.hip); launch_fast_backward goes there by itself
+hipError_t launch_fast_backward_once(const StageArgs& a, int n_head, int grid_x, hipStream_t s);
 // the same kernels built to honour a.table and a.ctx_len (the plain builds ignore both)
 hipError_t launch_fast_forward_indexed(Pass pass, const StageArgs& a, int n_head, int grid_x, hipStream_t s);
 hipError_t launch_fast_backward_indexed(const StageArgs& a, int n_head, int grid_x, hipStream_t s);

@@ -474,14 +474,18 @@ __global__ void __launch_bounds__(kBlockThreads) stage_inverse_kernel(const Stag
 
 // Tiles of up to 16 elements per lane fit 128 VGPRs (4 waves per SIMD) when the compiler is asked to.  Larger tiles,
 // the multi-activation build and the builds that mask steps would spill, so they are left alone.
-template <int NC, int EC, int R, int F, bool TANH_ONLY = true, bool INDEXED = false>
+// LOOP = false is for launches with a wave for every tile: without the loop around them the tile's addresses and
+// offsets are not carried in registers across it (the loop build spills 6 of them per lane at R x F = 16, which a
+// launch bound by its traffic pays for), and the steps come out in an order that issues better.
+template <int NC, int EC, int R, int F, bool TANH_ONLY = true, bool INDEXED = false, bool LOOP = true>
 __global__ void __launch_bounds__(kBlockThreads, (TANH_ONLY && R * F <= 16 && F == 4) ? 4 : 1) stage_backward_kernel(const StageArgs A) {
     NCN_WAVE_PROLOGUE
     float dwi[F], dwj[F];
 #pragma unroll
     for (int f = 0; f < F; ++f) dwi[f] = dwj[f] = 0.f;
 
-    for (uint32_t t = gwave / A.n_head; t < A.total_tiles; t += tile_step) {
+    uint32_t t = gwave / A.n_head;
+    if (t < A.total_tiles) do {
         int64_t off[R];
         const int live = tile_offsets<NC, EC, R, F, INDEXED>(A, t, lane, head, off);
         float Y[R][F], B[R][F], G[R][F], H[R][F];
@@ -520,7 +524,7 @@ __global__ void __launch_bounds__(kBlockThreads, (TANH_ONLY && R * F <= 16 && F 
                 store_frag<F>(A.aux1, NCN_F32, off[rr], valid, B[rr]);
             }
         }
-    }
+    } while (LOOP && (t += tile_step) < A.total_tiles);
 
     // dW: lanes holding the same feature chunk -> one value; this wave owns slot (gwave / n_head, head).
 #pragma unroll

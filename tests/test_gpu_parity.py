@@ -300,3 +300,29 @@ def test_scalars_the_scaled_state_cannot_carry_run_on_the_generic_kernels(M, alp
         assert O.rel_err(dW[0], rdWs[l]) < max(TOL_F32, 1e-6 * (1 / m) ** n), "dW%d" % l
     gtol = max(TOL_F32, 1e-6 * (1 / m) ** n)
     assert O.rel_err(g, rdx) < gtol and O.rel_err(h, rdxa) < gtol
+
+
+def test_backward_with_more_tiles_than_waves_loops_and_agrees_with_smaller_calls():
+    """ncn_backward launches at most 16384 workgroups (one dW partial row per n_head waves): up to that size every wave
+    takes one tile and the kernel is the build without a loop over tiles, beyond it the build with the loop.  160 batch
+    entries of the headline shape need 81920 waves (the loop build); the same entries in two calls of 80 (the other
+    build) must give the same dx, dxa and reconstructed inputs, and dW as the sum of the two."""
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from ncn_cuda_amd import ncn_cuda_module as M
+    batch, N, E, C, n = 160, 4096, 128, 4, 16
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(5)
+    x = torch.randn(batch, N, E, device=dev, generator=g)
+    xa = torch.randn(batch, N, E, device=dev, generator=g) * 0.1
+    dy = torch.randn(batch, N, E, device=dev, generator=g)
+    dya = torch.randn(batch, N, E, device=dev, generator=g)
+    W = torch.randn(2 * E, device=dev, generator=g) * (E // C) ** -0.5
+    y, ya = M.forward(x, xa, W, 0.9, 0, n, C, 1)
+    whole = M.backward_stages(y, ya, dy, dya, W, 0.9, 0, n, C, 1, 1)
+    h = batch // 2
+    parts = [M.backward_stages(y[s], ya[s], dy[s], dya[s], W, 0.9, 0, n, C, 1, 1) for s in (slice(0, h), slice(h, batch))]
+    for k in range(4):
+        assert O.rel_err(whole[k], torch.cat([parts[0][k], parts[1][k]])) < 1e-6
+    assert O.rel_err(whole[4], parts[0][4] + parts[1][4]) < 1e-6
+    assert O.rel_err(whole[0], x) < 1e-4
