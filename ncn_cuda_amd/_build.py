@@ -13,7 +13,7 @@ from concurrent.futures import ThreadPoolExecutor
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libncn_hip.so")
-SOURCES = ["ncn_api.hip", "ncn_fwd.hip", "ncn_bwd.hip", "ncn_bwd_once.hip", "ncn_fwd_indexed.hip", "ncn_bwd_indexed.hip",
+SOURCES = ["ncn_api.hip", "ncn_fwd.hip", "ncn_bwd.hip", "ncn_bwd_once.hip", "ncn_fwd_indexed.hip", "ncn_bwd_indexed.hip", "ncn_bwd_indexed_once.hip",
            "ncn_generic.hip", "ncn_fused.hip", "ncn_fused_radix.hip", "ncn_fused_lengths.hip"]
 # packed-fp32 VALU instructions are switched off for device code on purpose (flag is device-only;
 # the host pass prints a harmless "not a recognized feature" note).
@@ -28,7 +28,7 @@ HIPCC_FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17",
 MAX_ILP = ["-mllvm", "-amdgpu-sched-strategy=max-ilp"]
 EXTRA_FLAGS = {"ncn_fused.hip": MAX_ILP, "ncn_fused_radix.hip": MAX_ILP, "ncn_fused_lengths.hip": MAX_ILP,
                "ncn_fwd.hip": MAX_ILP, "ncn_fwd_indexed.hip": MAX_ILP, "ncn_bwd_indexed.hip": MAX_ILP,
-               "ncn_bwd_once.hip": MAX_ILP}
+               "ncn_bwd_once.hip": MAX_ILP, "ncn_bwd_indexed_once.hip": MAX_ILP}
 
 
 def _hipcc():

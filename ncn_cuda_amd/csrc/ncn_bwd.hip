@@ -1,7 +1,8 @@
 // Instantiations and dispatch of the register-resident reversible backward stage kernel.
-// Compiled three times: as it stands for the stride permutation; through ncn_bwd_once.hip (NCN_ONCE_BUILD = 1) in the
-// form without a loop over tiles, which launch_fast_backward picks by itself when the grid has a wave for every tile;
-// and through ncn_bwd_indexed.hip (NCN_INDEXED_BUILD = 1) for launches that carry a grouping table or context lengths.
+// Compiled four times: as it stands for the stride permutation; through ncn_bwd_indexed.hip (NCN_INDEXED_BUILD = 1)
+// for launches that carry a grouping table or context lengths; and each of the two once more (ncn_bwd_once.hip,
+// ncn_bwd_indexed_once.hip: NCN_ONCE_BUILD = 1) in the form without a loop over tiles, which the launchers pick by
+// themselves when the grid has a wave for every tile.
 #include "ncn_configs.h"
 #include "ncn_launch.h"
 #include "ncn_stage_kernels.h"
@@ -15,8 +16,12 @@
 
 namespace ncn {
 
-#if NCN_INDEXED_BUILD
-hipError_t launch_fast_backward_indexed(const StageArgs& a, int /*n_head*/, int grid_x, hipStream_t s) {
+#if NCN_INDEXED_BUILD && NCN_ONCE_BUILD
+hipError_t launch_fast_backward_indexed_once(const StageArgs& a, int /*n_head*/, int grid_x, hipStream_t s) {
+#elif NCN_INDEXED_BUILD
+hipError_t launch_fast_backward_indexed(const StageArgs& a, int n_head, int grid_x, hipStream_t s) {
+    if ((uint64_t)a.total_tiles * (uint64_t)a.n_head <= (uint64_t)grid_x * kWavesPerBlock)
+        return launch_fast_backward_indexed_once(a, n_head, grid_x, s);   // a wave for every tile
 #elif NCN_ONCE_BUILD
 hipError_t launch_fast_backward_once(const StageArgs& a, int /*n_head*/, int grid_x, hipStream_t s) {
 #else

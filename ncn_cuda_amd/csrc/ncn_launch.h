@@ -73,6 +73,7 @@ hipError_t launch_fast_backward_once(const StageArgs& a, int n_head, int grid_x,
 // the same kernels built to honour a.table and a.ctx_len (the plain builds ignore both)
 hipError_t launch_fast_forward_indexed(Pass pass, const StageArgs& a, int n_head, int grid_x, hipStream_t s);
 hipError_t launch_fast_backward_indexed(const StageArgs& a, int n_head, int grid_x, hipStream_t s);
+hipError_t launch_fast_backward_indexed_once(const StageArgs& a, int n_head, int grid_x, hipStream_t s);
 hipError_t launch_generic(Pass pass, const StageArgs& a, int n_head, int grid_x, hipStream_t s);
 // Rows past the context length of their batch entry: copied through (a.ctx_len must be set).
 hipError_t launch_pass_through(Pass pass, const StageArgs& a, int64_t batch, hipStream_t s);
