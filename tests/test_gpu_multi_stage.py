@@ -252,3 +252,16 @@ def test_backward_with_the_smaller_workspace_loops_over_windows(M):
     assert torch.equal(out[0], ref[2]) and torch.equal(out[1], ref[3])
     assert O.rel_err(dW, ref[4]) < 1e-6
     assert O.rel_err(ref[0], x) < 1e-4      # and both are the inputs again (26 steps undone)
+
+    # the same with one context length per batch entry (the LENGTHS builds of both forms of the kernel)
+    lens = torch.tensor([(37 * b * b + 11) % (N + 1) for b in range(batch)], dtype=torch.int32, device=dev)
+    y, ya = M.forward_stages(x, xa, W, 0.9, 0, n, C, 0, L, ctx_len=lens)
+    ref = M.backward_stages(y, ya, dy, dya, W, 0.9, 0, n, C, 0, L, ctx_len=lens)
+    rc = lib.ncn_backward_indexed(p(y), p(ya), 0, p(dy), p(dya), 0, p(out[0]), p(out[1]), 0, p(out[2]), p(out[3]), p(W),
+                                  p(dW), p(ws), ctypes.c_size_t(small), None, p(lens), ctypes.byref(shape), 0, L, 0.9,
+                                  0.9, 0, ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream))
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out[2], ref[0]) and torch.equal(out[3], ref[1])
+    assert torch.equal(out[0], ref[2]) and torch.equal(out[1], ref[3])
+    assert O.rel_err(dW, ref[4]) < 1e-6
