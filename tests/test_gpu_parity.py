@@ -326,3 +326,13 @@ def test_backward_with_more_tiles_than_waves_loops_and_agrees_with_smaller_calls
         assert O.rel_err(whole[k], torch.cat([parts[0][k], parts[1][k]])) < 1e-6
     assert O.rel_err(whole[4], parts[0][4] + parts[1][4]) < 1e-6
     assert O.rel_err(whole[0], x) < 1e-4
+    # the same through the builds that take context lengths (and a table: the stride permutation written out)
+    lens = torch.tensor([(53 * b * b + 7) % (N + 1) for b in range(batch)], dtype=torch.int32, device=dev)
+    table = O.stride_group_table(N, n, 1).to(torch.int32).cuda()
+    y, ya = M.forward_stages(x, xa, W, 0.9, 0, n, C, 0, 1, group_index=table, ctx_len=lens)
+    whole = M.backward_stages(y, ya, dy, dya, W, 0.9, 0, n, C, 0, 1, group_index=table, ctx_len=lens)
+    parts = [M.backward_stages(y[s], ya[s], dy[s], dya[s], W, 0.9, 0, n, C, 0, 1, group_index=table, ctx_len=lens[s])
+             for s in (slice(0, h), slice(h, batch))]
+    for k in range(4):
+        assert O.rel_err(whole[k], torch.cat([parts[0][k], parts[1][k]])) < 1e-6
+    assert O.rel_err(whole[4], parts[0][4] + parts[1][4]) < 1e-6
