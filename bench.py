@@ -173,7 +173,7 @@ def main():
                 _, _, dy, dya_, dWs[k] = M.backward_stages(saved[k][0], saved[k][1], dy, dya_, Wst[a:a + cnt], alpha,
                                                            0, n, C, a, cnt,
                                                            grad_dtype=io_dtype if cnt == 1 else torch.float32,
-                                                           want_inputs=cnt > 1, **extra)
+                                                           want_inputs=False, **extra)
             if events is not None:
                 e1.record()
                 events.append((e0, e1, cnt))

@@ -116,9 +116,12 @@ int ncn_forward(const void* x, const void* xa, int in_dtype,
  *                  amplifies rounding by (1/m)^n_cache per stage)
  * dy, dya     in   [batch,N,E] of dy_dtype; dya may be NULL, meaning zeros
  * dx, dxa     out  [batch,N,E] of dx_dtype
- * x_rec,xa_rec out float32 [batch,N,E], reconstructed inputs of first_stage; may be NULL when
- *                  n_stages == 1.  With n_stages > 1 they are required, dx_dtype must be NCN_F32, and
- *                  the four of x_rec, xa_rec, dx, dxa carry the state between stages in place.
+ * x_rec,xa_rec out float32 [batch,N,E], reconstructed inputs of first_stage, or both NULL when the caller does not
+ *                  want them (an autograd node does not).  With n_stages > 1 dx_dtype must be NCN_F32 and the
+ *                  four of x_rec, xa_rec, dx, dxa carry the state between stages in place; without x_rec, xa_rec
+ *                  two arrays of the workspace do (ncn_workspace_bytes_stages(.., backward = 2) bytes) and the
+ *                  last stage to run writes no reconstructed inputs at all (NCN_ERR_ALIAS if the workspace is
+ *                  smaller).
  * W           in   [n_stages, 2E] float32
  * dW          out  [n_stages, 2E] float32, overwritten (summed over batch, groups and rows)
  * workspace        scratch of at least ncn_workspace_bytes(shape) bytes; with n_stages > 1,
@@ -202,7 +205,8 @@ int ncn_inverse_ws(const void* y, const void* ya, int in_dtype,
  *                 (forward, inverse: out = in; backward: dx = dy, dxa = dya, x_rec = y, no share in dW).  Values are
  *                 clamped to [0, N].
  * Everything else as in ncn_forward / ncn_backward / ncn_inverse.  With a table these run stage by stage and
- * ncn_backward_indexed needs ncn_workspace_bytes(shape).  With lengths only (group_index NULL) the grouping is the
+ * ncn_backward_indexed needs ncn_workspace_bytes(shape) (followed, for several stages without x_rec, xa_rec, by two
+ * float32 arrays of the tensors' size, each padded to a multiple of 256 bytes).  With lengths only (group_index NULL) the grouping is the
  * stride permutation and several stages use the multi-stage LDS passes where ncn_forward / ncn_inverse / ncn_backward
  * would (float32 between passes): forward and inverse take no workspace, so their first pass goes from the inputs to
  * the outputs and the others work in place on the outputs, where the stages of a halo pass run one launch each;
@@ -291,6 +295,8 @@ size_t ncn_workspace_bytes(const ncn_shape* shape);
  * with their chunk sums, so that every window gets a workgroup of its own, and, with two passes or more, four
  * float32 arrays of the tensors' size.  ncn_backward also takes ncn_workspace_bytes(shape) plus the four arrays
  * (each padded to a multiple of 256 bytes) and then lets its workgroups walk over several windows, which is slower.
+ * backward = 2: the same for a call without x_rec, xa_rec, which takes the two arrays that carry the reconstructed
+ * state between stages from the end of the workspace (none when one multi-stage pass covers the range).
  * No reference counterpart. */
 size_t ncn_workspace_bytes_stages(const ncn_shape* shape, int first_stage, int n_stages, int activation, int backward);
 

@@ -358,7 +358,7 @@ hipError_t static_scratch(float** out) {
 
 extern "C" {
 
-const char* ncn_version(void) { return "0.9"; }
+const char* ncn_version(void) { return "0.10"; }
 
 int ncn_plan_passes(const ncn_shape* shape, int first_stage, int n_stages, int activation, int backward, int32_t* out,
                     int max_passes) {
@@ -388,7 +388,7 @@ const char* ncn_error_string(int code) {
         case NCN_ERR_WORKSPACE: return "workspace is NULL or smaller than ncn_workspace_bytes()";
         case NCN_ERR_UNSUPPORTED: return "unsupported shape: n_cache must be <= 64 and the head width <= 64 (128 for power-of-two n_cache <= 16)";
         case NCN_ERR_ALIGN: return "a pointer is not 16-byte aligned (4-byte for group_index and ctx_len)";
-        case NCN_ERR_ALIAS: return "n_stages > 1 needs float32 x_rec, xa_rec, dx, dxa to carry the state";
+        case NCN_ERR_ALIAS: return "n_stages > 1 needs float32 dx, dxa and either x_rec, xa_rec or the workspace of ncn_workspace_bytes_stages(.., 2) to carry the state";
         case NCN_ERR_STATIC_LIMIT: return "ncn_backward_static: E is above 256, the limit of the library's own scratch";
         default: break;
     }
@@ -421,7 +421,10 @@ size_t ncn_workspace_bytes_stages(const ncn_shape* shape, int first_stage, int n
     const std::vector<FusedPass> passes = multi_stage_plan(shape, first_stage, n_stages, activation, backward != 0);
     const size_t base = !backward ? 0 : passes.empty() ? base_workspace_bytes(shape)
                                                         : partial_buffer_bytes(shape, fused_rows_wanted(shape, passes));
-    return passes.size() >= 2 ? base + temp_bytes(shape, backward != 0) : base;
+    // backward == 2: the call will pass no x_rec, xa_rec, so the two arrays that carry the reconstructed state from
+    // stage to stage come out of the workspace (a single multi-stage pass carries nothing)
+    const size_t carriers = (backward == 2 && n_stages > 1 && passes.size() != 1) ? temp_bytes(shape, true) / 2 : 0;
+    return (passes.size() >= 2 ? base + temp_bytes(shape, backward != 0) : base) + carriers;
 }
 
 static int forward_impl(const void* x, const void* xa, int in_dtype, void* y, void* ya, int out_dtype, float* y32,
@@ -681,8 +684,13 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
     const int path = kernel_path_for(shape, activation, alpha, m);
     if (path == 0) return NCN_ERR_UNSUPPORTED;
     if (!known_dtype_or_x2(y_dtype, n_stages, path) || !known_dtype(dy_dtype) || !known_dtype(dx_dtype)) return NCN_ERR_DTYPE;
-    if (n_stages > 1 && (!x_rec || dx_dtype != NCN_F32)) return NCN_ERR_ALIAS;
+    if (n_stages > 1 && dx_dtype != NCN_F32) return NCN_ERR_ALIAS;
     if (!workspace || workspace_bytes < partial_buffer_bytes(shape, row_cap)) return NCN_ERR_WORKSPACE;
+    // Several stages without x_rec, xa_rec: the caller does not want the reconstructed inputs.  The stages before the
+    // last one to run still hand their reconstructed inputs on, through two arrays taken from the end of the
+    // workspace (ncn_workspace_bytes_stages(.., backward = 2)); the last one does not write them at all.
+    const bool no_rec = n_stages > 1 && !x_rec;
+    const size_t plane_bytes = temp_bytes(shape, true) / 4;
     if (!aligned16(y) || !aligned16(ya) || !aligned16(dy) || !aligned16(dya) || !aligned16(dx) || !aligned16(dxa) ||
         !aligned16(x_rec) || !aligned16(xa_rec) || !aligned16(W) || !aligned16(dW) || !aligned16(workspace))
         return NCN_ERR_ALIGN;
@@ -704,12 +712,13 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
     // a workspace of ncn_workspace_bytes_stages() holds a partial row for every window of every pass; a smaller one
     // (ncn_workspace_bytes() and the four arrays) makes the workgroups loop over windows
     int fused_cap = kMaxGridX;
+    const size_t fused_extra = np >= 2 ? temp_bytes(shape, true) + (no_rec ? 2 * plane_bytes : 0) : 0;
     if (np > 0) {
         const int want = fused_rows_wanted(shape, passes);
-        if (workspace_bytes >= partial_buffer_bytes(shape, want) + (np >= 2 ? temp_bytes(shape, true) : 0)) fused_cap = want;
+        if (workspace_bytes >= partial_buffer_bytes(shape, want) + fused_extra) fused_cap = want;
     }
     const size_t fused_base = partial_buffer_bytes(shape, fused_cap);
-    if (np >= 2 && workspace_bytes < fused_base + temp_bytes(shape, true)) fused_ok = false;
+    if (np >= 2 && workspace_bytes < fused_base + fused_extra) fused_ok = false;
     if (np >= 1 && ((np - 1) % 2) == 0 && !passes[np - 1].closed && !passes[np - 1].single &&
         (y == x_rec || ya == xa_rec || dy == dx || (dya && dya == dxa)))
         fused_ok = false;  // the first pass to run is a halo pass and would write into its own input
@@ -718,14 +727,18 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
         char* tb = static_cast<char*>(workspace) + fused_base;
         float* t[4] = {reinterpret_cast<float*>(tb), reinterpret_cast<float*>(tb + one),
                        reinterpret_cast<float*>(tb + 2 * one), reinterpret_cast<float*>(tb + 3 * one)};
+        // where the passes that write "to the outputs" leave the reconstructed inputs
+        float* rec = no_rec ? (np >= 2 ? reinterpret_cast<float*>(tb + 4 * one) : nullptr) : x_rec;
+        float* reca = no_rec ? (np >= 2 ? reinterpret_cast<float*>(tb + 5 * one) : nullptr) : xa_rec;
         const void* cy = y; const void* cya = ya; int cy_dtype = y_dtype;
         const void* cg = dy; const void* cga = dya; int cg_dtype = dy_dtype;
         DwReducer reducer(partials, partials + (int64_t)fused_cap * wstride, wstride, s, fused_cap);
         for (size_t e = 0; e < np; ++e) {
             const FusedPass& ps = passes[np - 1 - e];
             const bool to_out = ((np - 1 - e) % 2) == 0;
-            float* dxr = to_out ? x_rec : t[0];
-            float* dxar = to_out ? xa_rec : t[1];
+            const bool last = e + 1 == np;   // writes to the outputs by construction
+            float* dxr = to_out ? ((last && no_rec) ? nullptr : rec) : t[0];
+            float* dxar = to_out ? ((last && no_rec) ? nullptr : reca) : t[1];
             void* ddx = to_out ? dx : static_cast<void*>(t[2]);
             void* ddxa = to_out ? dxa : static_cast<void*>(t[3]);
             const int d_dtype = to_out ? dx_dtype : NCN_F32;
@@ -767,6 +780,12 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
         return (int)reducer.flush();
     }
 
+    if (no_rec) {   // the state between the stages lives behind the partial rows
+        if (workspace_bytes < partial_buffer_bytes(shape, row_cap) + 2 * plane_bytes) return NCN_ERR_ALIAS;
+        char* cb = static_cast<char*>(workspace) + partial_buffer_bytes(shape, row_cap);
+        x_rec = reinterpret_cast<float*>(cb);
+        xa_rec = reinterpret_cast<float*>(cb + plane_bytes);
+    }
     DwReducer reducer(partials, level1, wstride, s, row_cap);
     for (int k = n_stages - 1; k >= 0; --k) {
         float* region;
@@ -784,8 +803,8 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
         a.out0 = dx;
         a.out1 = dxa;
         a.out_dtype = dx_dtype;
-        a.aux0 = x_rec;
-        a.aux1 = xa_rec;
+        a.aux0 = (no_rec && k == 0) ? nullptr : x_rec;   // the last stage to run hands nothing on
+        a.aux1 = (no_rec && k == 0) ? nullptr : xa_rec;
         a.W = W + (int64_t)k * 2 * shape->E;
         a.dw_partials = region;
         err = (p.path != 2)      ? launch_generic(kBackward, a, shape->n_head, p.grid_x, s)

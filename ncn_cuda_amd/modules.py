@@ -93,7 +93,7 @@ class NCNNetFunction(torch.autograd.Function):
             a, cnt = segs[k]
             _, _, g, ga, dW = ncn_cuda_module.backward_stages(
                 saved[2 * k], saved[2 * k + 1], g, ga, W[a:a + cnt], alpha, activation, n_cache, n_head,
-                first_stage + a, cnt, grad_dtype=torch.float32, want_inputs=cnt > 1)
+                first_stage + a, cnt, grad_dtype=torch.float32, want_inputs=False)
             for j in range(cnt):
                 dWs[a + j] = dW[j].reshape(w_shapes[a + j]).to(w_dtypes[a + j])
         return (g.to(io_dtype), ga.to(io_dtype), None, None, None, None, None, None, *dWs)

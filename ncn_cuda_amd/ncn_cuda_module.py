@@ -255,7 +255,8 @@ def backward_stages(y, ya, dy, dya, W, alpha, activation, cache_dim, nhead, firs
     """Reversible backward of stages first_stage+n_stages-1 .. first_stage from the outputs y, ya of the last one.
     dya may be None (zeros).  y, ya may be the two-plane tensors [2, batch, N, E] of forward_stages(save_residual=True)
     (one stage).  Returns (x_rec, xa_rec, dx, dxa, dW[n_stages, 2E]); x_rec/xa_rec are None when
-    want_inputs is False and n_stages == 1."""
+    want_inputs is False (with several stages the state between them then travels through the workspace and the
+    last stage to run writes no reconstructed inputs)."""
     two_plane = _is_two_plane(y) and _is_two_plane(ya)
     if two_plane and n_stages != 1:
         raise ValueError("two-plane saved outputs hold one stage: n_stages must be 1")
@@ -279,7 +280,8 @@ def backward_stages(y, ya, dy, dya, W, alpha, activation, cache_dim, nhead, firs
     dy, w = _prep(dy.detach()), _w32(W)
     dya = _prep(dya.detach()) if dya is not None else None
     grad_dtype = dy.dtype if grad_dtype is None else grad_dtype
-    need_state = want_inputs or n_stages > 1
+    need_state = want_inputs
+    ws_mode = 1 if want_inputs else 2
     if n_stages > 1 and grad_dtype != torch.float32:
         raise ValueError("multi-stage backward carries its state in float32: use grad_dtype=torch.float32")
     dx = torch.empty(dy.shape, dtype=grad_dtype, device=dev)
@@ -292,9 +294,14 @@ def backward_stages(y, ya, dy, dya, W, alpha, activation, cache_dim, nhead, firs
     if indexed:
         # lengths without a table keep the stride permutation: with the multi-stage figure the library runs its
         # multi-stage passes on them too
-        ws_bytes = (lib.ncn_workspace_bytes(ctypes.byref(shape)) if group_index is not None else
-                    lib.ncn_workspace_bytes_stages(ctypes.byref(shape), int(first_stage), int(n_stages),
-                                                   int(activation), 1))
+        if group_index is not None:
+            # a table never uses the multi-stage passes: the partial rows of one launch, plus the two float32 arrays
+            # (each padded to 256 bytes) that carry the state between stages when no reconstructed inputs are wanted
+            plane = (dy.numel() * 4 + 255) // 256 * 256
+            ws_bytes = lib.ncn_workspace_bytes(ctypes.byref(shape)) + (2 * plane if ws_mode == 2 and n_stages > 1 else 0)
+        else:
+            ws_bytes = lib.ncn_workspace_bytes_stages(ctypes.byref(shape), int(first_stage), int(n_stages),
+                                                      int(activation), ws_mode)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
         with torch.cuda.device(dev):
             rc = lib.ncn_backward_indexed(_ptr(y), _ptr(ya), y_code, _ptr(dy), _ptr(dya), _DTYPES[dy.dtype],
@@ -304,7 +311,8 @@ def backward_stages(y, ya, dy, dya, W, alpha, activation, cache_dim, nhead, firs
                                           int(activation), _stream(dev))
         _lib.check(rc, "ncn_backward_indexed")
         return x_rec, xa_rec, dx, dxa, dW
-    ws_bytes = lib.ncn_workspace_bytes_stages(ctypes.byref(shape), int(first_stage), int(n_stages), int(activation), 1)
+    ws_bytes = lib.ncn_workspace_bytes_stages(ctypes.byref(shape), int(first_stage), int(n_stages), int(activation),
+                                              ws_mode)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
         rc = lib.ncn_backward(_ptr(y), _ptr(ya), y_code, _ptr(dy), _ptr(dya), _DTYPES[dy.dtype],

@@ -265,3 +265,47 @@ def test_backward_with_the_smaller_workspace_loops_over_windows(M):
     assert torch.equal(out[2], ref[0]) and torch.equal(out[3], ref[1])
     assert torch.equal(out[0], ref[2]) and torch.equal(out[1], ref[3])
     assert O.rel_err(dW, ref[4]) < 1e-6
+
+
+@pytest.mark.parametrize("case", [
+    (3, 1024, 64, 2, 2, 0, 11),    # several multi-stage passes (halo and closed)
+    (1, 256, 32, 1, 2, 0, 8),      # one pass covers the range
+    (2, 1024, 128, 4, 4, 0, 5),    # multi-stage passes and one-stage launches mixed
+    (2, 512, 32, 2, 8, 0, 4),      # one-stage launches only
+    (2, 96, 20, 2, 3, 1, 3),       # the generic kernels
+], ids=lambda c: "b%d_N%d_E%d_C%d_n%d_s%d_L%d" % c)
+@pytest.mark.parametrize("grouping", ["closed", "lengths", "table"])
+def test_backward_without_reconstructed_inputs(M, case, grouping):
+    """x_rec = xa_rec = NULL with several stages: the state between the stages travels through the workspace and the
+    last stage to run writes no reconstructed inputs.  Same kernels on the same values: dx, dxa, dW bit-identical to
+    the call that returns them."""
+    batch, N, E, C, n, first, L = case
+    x, xa, Ws, dy, dya = O.make_inputs(batch, N, E, L, n, seed=29, xa_zero=False)
+    gx, gxa, gdy, gdya = x.cuda(), xa.cuda(), dy.cuda(), dya.cuda()
+    W = torch.stack(Ws).cuda()
+    kw = {}
+    if grouping == "lengths":
+        kw["ctx_len"] = torch.tensor(([N // 2 + 1, N, 3, 0, N - 1])[:batch], dtype=torch.int32).cuda()
+    if grouping == "table":
+        kw["group_index"] = torch.stack([O.stride_group_table(N, n, first + l) for l in range(L)]).to(torch.int32).cuda()
+        first = 0
+    y, ya = M.forward_stages(gx, gxa, W, 0.9, 0, n, C, first, L, **kw)
+    full = M.backward_stages(y, ya, gdy, gdya, W, 0.9, 0, n, C, first, L, **kw)
+    lean = M.backward_stages(y, ya, gdy, gdya, W, 0.9, 0, n, C, first, L, want_inputs=False, **kw)
+    assert lean[0] is None and lean[1] is None
+    for k in (2, 3, 4):
+        assert torch.equal(full[k], lean[k])
+    # and without the workspace for it the call says so instead of running
+    import ctypes
+    from ncn_cuda_amd import _lib
+    lib = _lib.load()
+    shape = _lib.NcnShape(batch, N, E, C, n)
+    small = lib.ncn_workspace_bytes(ctypes.byref(shape))
+    ws = torch.empty(small, dtype=torch.uint8, device="cuda")
+    dx, dxa, dW = torch.empty_like(gx), torch.empty_like(gx), torch.empty(L, 2 * E, device="cuda")
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    if grouping == "closed" and lib.ncn_plan_passes(ctypes.byref(shape), first, L, 0, 1, None, 0) != 1:
+        rc = lib.ncn_backward(p(y), p(ya), 0, p(gdy), p(gdya), 0, p(dx), p(dxa), 0, None, None, p(W), p(dW), p(ws),
+                              ctypes.c_size_t(small), ctypes.byref(shape), first, L, 0.9, 0.9, 0,
+                              ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert rc == -8
