@@ -168,7 +168,7 @@ def main():
                      dict(ctx_len=lens))
             if args.grouping == "radix":
                 _, _, dy, dya_, dWs[k] = M.backward_radix(saved[k][0], saved[k][1], dy, dya_, Wst[a:a + cnt], alpha, 0,
-                                                          n, C, a, cnt)
+                                                          n, C, a, cnt, want_inputs=False)
             else:
                 _, _, dy, dya_, dWs[k] = M.backward_stages(saved[k][0], saved[k][1], dy, dya_, Wst[a:a + cnt], alpha,
                                                            0, n, C, a, cnt,

@@ -251,7 +251,9 @@ int ncn_inverse_indexed(const void* y, const void* ya, int in_dtype,
  * n_cache^(first_level+n_levels) must divide N (NCN_ERR_SHAPE otherwise).  W, dW: [n_levels, 2E].
  * Arguments as in ncn_forward / ncn_backward.  Levels after the first pass run in place on y, ya (forward) and on
  * x_rec, xa_rec, dx, dxa (backward): use float32 outputs when more than one pass is needed, or the values between
- * passes are rounded to the output type.  ncn_backward_radix needs ncn_workspace_bytes(shape) of scratch.
+ * passes are rounded to the output type.  ncn_backward_radix needs ncn_workspace_bytes(shape) of scratch; with several
+ * levels x_rec, xa_rec may both be NULL when that scratch is followed by two float32 arrays of the tensors' size (each
+ * padded to a multiple of 256 bytes): the last pass to run then writes no reconstructed inputs.
  */
 int ncn_forward_radix(const void* x, const void* xa, int in_dtype,
                       void* y, void* ya, int out_dtype,

@@ -949,8 +949,18 @@ int ncn_backward_radix(const void* y, const void* ya, int y_dtype, const void* d
     if (!y || !ya || !dy || !dx || !dxa || !W || !dW) return NCN_ERR_NULL;
     if ((x_rec == nullptr) != (xa_rec == nullptr)) return NCN_ERR_NULL;
     if (!known_dtype(y_dtype) || !known_dtype(dy_dtype) || !known_dtype(dx_dtype)) return NCN_ERR_DTYPE;
-    if (n_levels > 1 && (!x_rec || dx_dtype != NCN_F32)) return NCN_ERR_ALIAS;
+    if (n_levels > 1 && dx_dtype != NCN_F32) return NCN_ERR_ALIAS;
     if (!workspace || workspace_bytes < ncn_workspace_bytes(shape)) return NCN_ERR_WORKSPACE;
+    // several levels without x_rec, xa_rec: as in ncn_backward, the state travels through two arrays behind the partial
+    // rows and the last pass to run writes no reconstructed inputs
+    const bool no_rec = n_levels > 1 && !x_rec;
+    if (no_rec) {
+        const size_t plane_bytes = temp_bytes(shape, true) / 4;
+        if (workspace_bytes < base_workspace_bytes(shape) + 2 * plane_bytes) return NCN_ERR_ALIAS;
+        char* cb = static_cast<char*>(workspace) + base_workspace_bytes(shape);
+        x_rec = reinterpret_cast<float*>(cb);
+        xa_rec = reinterpret_cast<float*>(cb + plane_bytes);
+    }
     if (!aligned16(y) || !aligned16(ya) || !aligned16(dy) || !aligned16(dya) || !aligned16(dx) || !aligned16(dxa) ||
         !aligned16(x_rec) || !aligned16(xa_rec) || !aligned16(W) || !aligned16(dW) || !aligned16(workspace))
         return NCN_ERR_ALIGN;
@@ -967,6 +977,7 @@ int ncn_backward_radix(const void* y, const void* ya, int y_dtype, const void* d
     for (size_t e = 0; e < passes.size(); ++e) {
         const RadixPass& ps = passes[passes.size() - 1 - e];
         const bool top = (e == 0);
+        const bool drop_rec = no_rec && e + 1 == passes.size();
         const int rows = ps.single ? p.partial_rows : radix_grid(shape, ps, true) / shape->n_head;
         float* region;
         hipError_t err = reducer.reserve(rows, ps.count, &region);
@@ -978,7 +989,7 @@ int ncn_backward_radix(const void* y, const void* ya, int y_dtype, const void* d
             a.in0 = top ? y : x_rec; a.in1 = top ? ya : xa_rec; a.in_dtype = top ? y_dtype : NCN_F32;
             a.g0 = top ? dy : dx; a.g1 = top ? dya : dxa; a.g_dtype = top ? dy_dtype : NCN_F32;
             a.out0 = dx; a.out1 = dxa; a.out_dtype = dx_dtype;
-            a.aux0 = x_rec; a.aux1 = xa_rec;
+            a.aux0 = drop_rec ? nullptr : x_rec; a.aux1 = drop_rec ? nullptr : xa_rec;
             a.W = W + ps.first * wstride;
             a.dw_partials = region;
             err = (p.path != 2) ? launch_generic(kBackward, a, shape->n_head, p.grid_x, s)
@@ -988,7 +999,7 @@ int ncn_backward_radix(const void* y, const void* ya, int y_dtype, const void* d
             a.in0 = top ? y : x_rec; a.in1 = top ? ya : xa_rec; a.in_dtype = top ? y_dtype : NCN_F32;
             a.g0 = top ? dy : dx; a.g1 = top ? dya : dxa; a.g_dtype = top ? dy_dtype : NCN_F32;
             a.out0 = dx; a.out1 = dxa; a.out_dtype = dx_dtype;
-            a.aux0 = x_rec; a.aux1 = xa_rec;
+            a.aux0 = drop_rec ? nullptr : x_rec; a.aux1 = drop_rec ? nullptr : xa_rec;
             a.W = W + ps.first * wstride;
             a.dw_partials = region;
             fill_step_table(a.tab, shape->n_cache, alpha, m, activation);

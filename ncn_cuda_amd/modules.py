@@ -129,7 +129,8 @@ class NCNRadixNetFunction(torch.autograd.Function):
         for k in range(len(segs) - 1, -1, -1):
             a, cnt = segs[k]
             _, _, g, ga, dW = ncn_cuda_module.backward_radix(saved[2 * k], saved[2 * k + 1], g, ga, W[a:a + cnt], alpha,
-                                                             activation, n_cache, n_head, first_level + a, cnt)
+                                                             activation, n_cache, n_head, first_level + a, cnt,
+                                                             want_inputs=False)
             for j in range(cnt):
                 dWs[a + j] = dW[j].reshape(w_shapes[a + j]).to(w_dtypes[a + j])
         return (g.to(io_dtype), ga.to(io_dtype), None, None, None, None, None, None, *dWs)

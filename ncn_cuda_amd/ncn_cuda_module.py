@@ -404,9 +404,10 @@ def inverse_radix(y, ya, W, alpha, activation, cache_dim, nhead, first_level, n_
     return x, xa
 
 
-def backward_radix(y, ya, dy, dya, W, alpha, activation, cache_dim, nhead, first_level, n_levels, *, m=M_DEFAULT):
+def backward_radix(y, ya, dy, dya, W, alpha, activation, cache_dim, nhead, first_level, n_levels, *, m=M_DEFAULT,
+                   want_inputs=True):
     """Reversible backward of forward_radix from its outputs.  Returns (x_rec, xa_rec, dx, dxa, dW[n_levels, 2E]), all
-    float32."""
+    float32; x_rec, xa_rec are None when want_inputs is False (the library then does not write them)."""
     shape = validate(y, ya, W, cache_dim, nhead, activation, 0, n_levels, what="y")
     if dy.shape != y.shape or (dya is not None and dya.shape != y.shape):
         raise ValueError("dy/dya must have the shape of y")
@@ -417,10 +418,13 @@ def backward_radix(y, ya, dy, dya, W, alpha, activation, cache_dim, nhead, first
     dya = _prep(dya.detach()) if dya is not None else None
     f32 = torch.float32
     dx, dxa = torch.empty(y.shape, dtype=f32, device=dev), torch.empty(y.shape, dtype=f32, device=dev)
-    x_rec, xa_rec = torch.empty(y.shape, dtype=f32, device=dev), torch.empty(y.shape, dtype=f32, device=dev)
+    x_rec = torch.empty(y.shape, dtype=f32, device=dev) if want_inputs else None
+    xa_rec = torch.empty(y.shape, dtype=f32, device=dev) if want_inputs else None
     dW = torch.empty(n_levels, 2 * y.shape[2], dtype=f32, device=dev)
     lib = _lib.load()
     ws_bytes = lib.ncn_workspace_bytes(ctypes.byref(shape))
+    if not want_inputs and n_levels > 1:   # two float32 arrays (padded to 256 bytes) carry the state between the passes
+        ws_bytes += 2 * ((y.numel() * 4 + 255) // 256 * 256)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
         rc = lib.ncn_backward_radix(_ptr(y), _ptr(ya), _DTYPES[y.dtype], _ptr(dy), _ptr(dya), _DTYPES[dy.dtype],

@@ -63,6 +63,9 @@ def test_radix_levels_vs_oracle_tables(M, case):
     for l in range(L):
         assert O.rel_err(dW[l], ref[4][l]) < tol, f"dW{l}"
     assert O.rel_err(xr, x) < tol and O.rel_err(xar, xa) < tol
+    # without the reconstructed inputs (state through the workspace, the last pass writes gradients only): same bits
+    lean = M.backward_radix(y, ya, gdy, gdya, W, alpha, 0, n, C, first, L, want_inputs=False)
+    assert lean[0] is None and torch.equal(lean[2], dx) and torch.equal(lean[3], dxa) and torch.equal(lean[4], dW)
     ix, ixa = M.inverse_radix(y, ya, W, alpha, 0, n, C, first, L)
     assert O.rel_err(ix, x) < tol and O.rel_err(ixa, xa) < tol
     # the table path of the library on the same levels (one launch per level): rounding-level agreement
