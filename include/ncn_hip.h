@@ -298,7 +298,7 @@ size_t ncn_workspace_bytes(const ncn_shape* shape);
  * float32 arrays of the tensors' size.  ncn_backward also takes ncn_workspace_bytes(shape) plus the four arrays
  * (each padded to a multiple of 256 bytes) and then lets its workgroups walk over several windows, which is slower.
  * backward = 2: the same for a call without x_rec, xa_rec, which takes the two arrays that carry the reconstructed
- * state between stages from the end of the workspace (none when one multi-stage pass covers the range).
+ * state between stages from the end of the workspace (none when one pass over closed rings covers the range).
  * No reference counterpart. */
 size_t ncn_workspace_bytes_stages(const ncn_shape* shape, int first_stage, int n_stages, int activation, int backward);
 

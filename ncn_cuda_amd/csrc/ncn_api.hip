@@ -422,8 +422,10 @@ size_t ncn_workspace_bytes_stages(const ncn_shape* shape, int first_stage, int n
     const size_t base = !backward ? 0 : passes.empty() ? base_workspace_bytes(shape)
                                                         : partial_buffer_bytes(shape, fused_rows_wanted(shape, passes));
     // backward == 2: the call will pass no x_rec, xa_rec, so the two arrays that carry the reconstructed state from
-    // stage to stage come out of the workspace (a single multi-stage pass carries nothing)
-    const size_t carriers = (backward == 2 && n_stages > 1 && passes.size() != 1) ? temp_bytes(shape, true) / 2 : 0;
+    // stage to stage come out of the workspace (a single pass over closed rings carries nothing; a single halo pass
+    // may have to give way to one launch per stage when the caller's buffers alias, and those carry)
+    const bool one_closed_pass = passes.size() == 1 && passes[0].closed && !passes[0].single;
+    const size_t carriers = (backward == 2 && n_stages > 1 && !one_closed_pass) ? temp_bytes(shape, true) / 2 : 0;
     return (passes.size() >= 2 ? base + temp_bytes(shape, backward != 0) : base) + carriers;
 }
 
