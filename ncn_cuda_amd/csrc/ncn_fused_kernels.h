@@ -145,7 +145,7 @@ __device__ __forceinline__ int64_t fused_row_offset(const FusedArgs& A, const Fu
     }
     const uint32_t qi = lr / NC, o = lr - qi * NC;
     const uint32_t sub = (it.sub0 + qi) & (A.ring - 1u);
-    const uint32_t cls = A.closed ? it.cls + qi / A.ring : it.cls;
+    const uint32_t cls = A.closed ? it.cls + (qi >> log2u(A.ring)) : it.cls;   // rings are powers of two
     const uint32_t blk = sub * A.class_stride + cls;
     return it.base + ((int64_t)blk * NC + o) * A.E;
 }
@@ -182,7 +182,7 @@ __device__ __forceinline__ uint32_t fused_lds_row(const FusedArgs& A, uint32_t q
 template <int NC>
 __device__ __forceinline__ int fused_live_rows(const FusedArgs& A, const FusedItem& it, uint32_t qg, int32_t len) {
     const uint32_t sub = (it.sub0 + qg) & (A.ring - 1u);
-    const uint32_t cls = A.closed ? it.cls + qg / A.ring : it.cls;
+    const uint32_t cls = A.closed ? it.cls + (qg >> log2u(A.ring)) : it.cls;
     const int64_t r = (int64_t)len - (int64_t)(sub * A.class_stride + cls) * NC;
     return (int)max((int64_t)0, min(r, (int64_t)NC));
 }
