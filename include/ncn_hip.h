@@ -67,7 +67,8 @@ extern "C" {
 #define NCN_ERR_DTYPE (-3)       /* unknown element type */
 #define NCN_ERR_ACTIVATION (-4)  /* unknown activation code */
 #define NCN_ERR_WORKSPACE (-5)   /* workspace missing or smaller than ncn_workspace_bytes() */
-#define NCN_ERR_UNSUPPORTED (-6) /* n_cache > 64, or head width too large for the generic kernel */
+#define NCN_ERR_UNSUPPORTED (-6) /* n_cache > 64, or head width too large for the generic kernel; also alpha outside
+                                    [1e-3, 1e3] or m outside [1e-3, 0.999] at head widths above 64 (see ncn_kernel_path_scalars) */
 #define NCN_ERR_ALIGN (-7)       /* a pointer is not 16-byte aligned (4-byte for the int32 tables) */
 #define NCN_ERR_ALIAS (-8)       /* n_stages > 1 needs the state buffers the call would carry it in */
 #define NCN_ERR_STATIC_LIMIT (-9) /* ncn_backward_static: the shape needs more scratch than the library holds */
@@ -148,7 +149,13 @@ int ncn_backward(const void* y, const void* ya, int y_dtype,
  * one stage are bit-identical to ncn_backward's, dW sums the same terms over fewer partial rows.
  * Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (different streams or threads) race;
  * calls on one stream are ordered.  Nothing in the array has to be cleared between calls.
- * Arguments as ncn_backward.
+ * Arguments as ncn_backward, with one difference: with n_stages > 1, x_rec and xa_rec are REQUIRED (NCN_ERR_ALIAS when
+ * they are NULL).  The stages of a call hand their reconstructed inputs on through them; ncn_backward takes two
+ * float32 [batch, N, E] arrays from its workspace for that when they are NULL, and the library's array is far too
+ * small to hold those.  With n_stages == 1 they may be NULL as there.
+ * Before a stream capture: make one call of the same shape class on the device outside the capture.  The first call
+ * per device resolves the array's address (hipGetSymbolAddress) and the first launch of a kernel that needs more than
+ * 64 KB of LDS raises its limit (hipFuncSetAttribute); neither can be recorded into a graph.  Later calls only launch.
  */
 int ncn_backward_static(const void* y, const void* ya, int y_dtype,
                         const void* dy, const void* dya, int dy_dtype,
@@ -322,8 +329,10 @@ int ncn_kernel_path(const ncn_shape* shape);
  * than those take. */
 int ncn_kernel_path_scalars(const ncn_shape* shape, float alpha, float m);
 
-/* Validates arguments exactly as the entry points do, without touching the GPU.  Returns NCN_OK or
- * the error the corresponding call would return before launching.  No reference counterpart (the
+/* Validates the shape, stage range and activation exactly as the entry points do, without touching the GPU.  Returns
+ * NCN_OK or the error the corresponding call would return before launching.  It takes no scalars: an entry point
+ * additionally returns NCN_ERR_UNSUPPORTED when ncn_kernel_path_scalars(shape, alpha, m) is 0 (alpha or m outside the
+ * range of the register kernels at a head width the generic kernels do not take).  No reference counterpart (the
  * reference validates nothing). */
 int ncn_check_shape(const ncn_shape* shape, int first_stage, int n_stages, int activation);
 
@@ -332,6 +341,20 @@ const char* ncn_error_string(int code);
 
 /* Library version, "major.minor". */
 const char* ncn_version(void);
+
+/* Build id: 16 hex digits, a hash of every source file, header and compiler flag the library was made from.  The
+ * Python loader compares it with the hash of the sources it finds beside the library and rebuilds when they differ
+ * (file times play no part).  No reference counterpart. */
+const char* ncn_build_id(void);
+
+/* Measurement aid, no part of the layer and no reference counterpart: launches `blocks` workgroups of 256 threads in
+ * which every thread executes ncn_probe_fma_per_thread(iters) independent float32 FMAs (8 chains per lane, plain
+ * v_fma_f32: the library is built without packed FP32) and writes one float to out[blocks * 256].  Timed by the
+ * caller (HIP events on `stream`), blocks = 8 x the number of CUs gives the FP32 vector rate this GPU sustains
+ * without packed instructions, which bench.py quotes beside the published 157.3 TFLOP/s (that figure counts packed
+ * FP32). */
+int ncn_probe_fma_stream(float* out, int blocks, int iters, void* stream);
+int ncn_probe_fma_per_thread(int iters);
 
 #ifdef __cplusplus
 }

@@ -1,7 +1,7 @@
 """ctypes binding of libncn_hip.so (C ABI declared in include/ncn_hip.h).
 
-There is no CPU or PyTorch fallback.  A library that is missing, or older than one of its sources, is built on the
-spot with hipcc (ncn_cuda_amd/_build.py, about a minute); if that cannot be done, loading raises.
+There is no CPU or PyTorch fallback.  A library that is missing, or was made from other sources than those beside it
+(compared by content, see _build.py), is built on the spot with hipcc; if that cannot be done, loading raises.
 """
 import ctypes
 import os
@@ -15,7 +15,8 @@ ACT_TANH, ACT_RELU, ACT_SIGMOID, ACT_LEAKY_RELU, ACT_LINEAR = 0, 1, 2, 3, -1
 EXPORTS = ("ncn_forward", "ncn_backward", "ncn_inverse", "ncn_forward_indexed", "ncn_backward_indexed",
            "ncn_inverse_indexed", "ncn_inverse_ws", "ncn_forward_radix", "ncn_backward_radix", "ncn_inverse_radix", "ncn_plan_radix", "ncn_workspace_bytes", "ncn_workspace_bytes_stages",
            "ncn_plan_passes", "ncn_kernel_path",
-           "ncn_check_shape", "ncn_error_string", "ncn_version", "ncn_backward_static", "ncn_static_scratch_bytes", "ncn_kernel_path_scalars")
+           "ncn_check_shape", "ncn_error_string", "ncn_version", "ncn_backward_static", "ncn_static_scratch_bytes", "ncn_kernel_path_scalars",
+           "ncn_build_id", "ncn_probe_fma_stream", "ncn_probe_fma_per_thread")
 
 
 class NcnShape(ctypes.Structure):
@@ -27,17 +28,17 @@ _lib = None
 
 
 def _stale_reason():
-    """Why the shared library has to be built before it can be loaded, or None."""
+    """Why the shared library has to be built before it can be loaded, or None.  Decided by content: the library carries
+    a hash of the sources it was made from (ncn_build_id), compared here with the hash of the sources beside it.  File
+    times play no part, so a copy or checkout that disturbs them changes nothing."""
+    from . import _build
     if not os.path.exists(LIB_PATH):
         return "libncn_hip.so is missing"
-    built = os.path.getmtime(LIB_PATH)
-    roots = [os.path.join(PKG_DIR, "csrc"), os.path.join(os.path.dirname(PKG_DIR), "include")]
-    for root in roots:
-        if not os.path.isdir(root):
-            continue                      # an installed copy without sources: take the library as it is
-        for name in os.listdir(root):
-            if name.endswith((".hip", ".h")) and os.path.getmtime(os.path.join(root, name)) > built:
-                return f"libncn_hip.so is older than {name}"
+    if not _build.have_sources():
+        return None                       # an installed copy without sources: take the library as it is
+    have, want = _build.library_build_id(LIB_PATH), _build.source_build_id()
+    if have != want:
+        return f"libncn_hip.so was built from other sources (build id {have}, sources {want})"
     return None
 
 
@@ -50,13 +51,17 @@ def load():
     if reason:
         import sys
         from . import _build
-        print(f"ncn_cuda_amd: {reason}: building it with hipcc (about a minute)", file=sys.stderr)
-        try:
-            _build.build()
-        except Exception as exc:
-            raise RuntimeError(
-                f"{LIB_PATH}: {reason}, and building it failed ({exc}); build it with `python -m ncn_cuda_amd._build` "
-                "(or __graft_entry__.build()): there is no CPU or PyTorch fallback for the NCN kernels") from exc
+        if os.path.exists(LIB_PATH) and not _build.have_hipcc():
+            print(f"ncn_cuda_amd: warning: {reason}, and there is no hipcc here to rebuild it: loading it as it is",
+                  file=sys.stderr)
+        else:
+            print(f"ncn_cuda_amd: {reason}: building what changed with hipcc (up to a minute)", file=sys.stderr)
+            try:
+                _build.build(force=False)   # under a file lock; checks again whether another process has built it
+            except Exception as exc:
+                raise RuntimeError(
+                    f"{LIB_PATH}: {reason}, and building it failed ({exc}); build it with `python -m ncn_cuda_amd._build` "
+                    "(or __graft_entry__.build()): there is no CPU or PyTorch fallback for the NCN kernels") from exc
     lib = ctypes.CDLL(LIB_PATH)
     vp, f32p, shp = ctypes.c_void_p, ctypes.c_void_p, ctypes.POINTER(NcnShape)
     i, fl = ctypes.c_int, ctypes.c_float
@@ -105,6 +110,12 @@ def load():
     lib.ncn_error_string.argtypes = [i]
     lib.ncn_version.restype = ctypes.c_char_p
     lib.ncn_version.argtypes = []
+    lib.ncn_build_id.restype = ctypes.c_char_p
+    lib.ncn_build_id.argtypes = []
+    lib.ncn_probe_fma_stream.restype = i
+    lib.ncn_probe_fma_stream.argtypes = [vp, i, i, vp]
+    lib.ncn_probe_fma_per_thread.restype = i
+    lib.ncn_probe_fma_per_thread.argtypes = [i]
     _lib = lib
     return lib
 

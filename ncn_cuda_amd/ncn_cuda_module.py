@@ -29,8 +29,9 @@ _DTYPES = {torch.float32: _lib.NCN_F32, torch.bfloat16: _lib.NCN_BF16}
 _ACT_CODES = (_lib.ACT_TANH, _lib.ACT_RELU, _lib.ACT_SIGMOID, _lib.ACT_LEAKY_RELU, _lib.ACT_LINEAR)
 
 
-def validate(x, xa, W, n_cache, n_head, activation, module_l=0, n_stages=1, what="x"):
-    """Host-side argument checks (no GPU needed).  Raises TypeError / ValueError."""
+def validate(x, xa, W, n_cache, n_head, activation, module_l=0, n_stages=1, what="x", alpha=None, m=None):
+    """Host-side argument checks (no GPU needed).  Raises TypeError / ValueError.  With alpha (and m) also checks that
+    some kernel takes these scalars at this head width."""
     if not (isinstance(x, torch.Tensor) and isinstance(xa, torch.Tensor) and isinstance(W, torch.Tensor)):
         raise TypeError("x, xa and W must be torch tensors")
     if x.dim() != 3:
@@ -60,6 +61,12 @@ def validate(x, xa, W, n_cache, n_head, activation, module_l=0, n_stages=1, what
     if rc != 0:
         raise ValueError(f"unsupported NCN problem {tuple(x.shape)}, n_cache={n_cache}, n_head={n_head}: "
                          f"{_lib.error_string(rc)}")
+    if alpha is not None:
+        mm = M_DEFAULT if m is None else float(m)
+        if _lib.load().ncn_kernel_path_scalars(ctypes.byref(shape), float(alpha), mm) == 0:
+            raise ValueError(f"alpha={alpha}, m={mm} with heads of {E // n_head} features: the register kernels take "
+                             "alpha in [1e-3, 1e3] and m in [1e-3, 0.999], and the generic kernels, which take any "
+                             "scalars, only heads of up to 64 features")
     return shape
 
 
@@ -182,7 +189,7 @@ def forward_stages(x, xa, W, alpha, activation, cache_dim, nhead, first_stage, n
     group_index [n_stages, N] replaces the stride permutation by a table of positions in (group, slot) order and
     ctx_len [batch] gives every batch entry its own number of live slots (the group_tensor / ctxlen_tensor of
     ncn_triton/ncn_triton_old.py:362-387); rows past the length pass through."""
-    shape = validate(x, xa, W, cache_dim, nhead, activation, first_stage, n_stages)
+    shape = validate(x, xa, W, cache_dim, nhead, activation, first_stage, n_stages, alpha=alpha, m=m)
     dev = _require_gpu(x, xa, W)
     indexed = group_index is not None or ctx_len is not None
     gi, cl = _grouping(group_index, ctx_len, x.shape[0], x.shape[1], n_stages, dev, check_tables)
@@ -263,7 +270,7 @@ def backward_stages(y, ya, dy, dya, W, alpha, activation, cache_dim, nhead, firs
     ys_full, yas_full = y, ya
     if two_plane:
         y, ya = ys_full[0], yas_full[0]
-    shape = validate(y, ya, W, cache_dim, nhead, activation, first_stage, n_stages, what="y")
+    shape = validate(y, ya, W, cache_dim, nhead, activation, first_stage, n_stages, what="y", alpha=alpha, m=m)
     if dy.shape != y.shape or (dya is not None and dya.shape != y.shape):
         raise ValueError("dy/dya must have the shape of y")
     if dy.dtype not in _DTYPES or (dya is not None and dya.dtype != dy.dtype):
@@ -327,7 +334,7 @@ def inverse_stages(y, ya, W, alpha, activation, cache_dim, nhead, first_stage, n
                    out_dtype=None, group_index=None, ctx_len=None, check_tables=True, scratch=True):
     """x, xa with forward_stages(x, xa, ...) == (y, ya).  scratch: with several stages, allocate the scratch that lets
     every multi-stage pass run as one (ncn_inverse_ws); without it the stages of a halo pass run one launch each."""
-    shape = validate(y, ya, W, cache_dim, nhead, activation, first_stage, n_stages, what="y")
+    shape = validate(y, ya, W, cache_dim, nhead, activation, first_stage, n_stages, what="y", alpha=alpha, m=m)
     dev = _require_gpu(y, ya, W)
     indexed = group_index is not None or ctx_len is not None
     gi, cl = _grouping(group_index, ctx_len, y.shape[0], y.shape[1], n_stages, dev, check_tables)
@@ -369,7 +376,7 @@ def forward_radix(x, xa, W, alpha, activation, cache_dim, nhead, first_level, n_
     """Levels first_level .. first_level+n_levels-1 of the radix-n digit grouping (ncn_triton/group_tensors.py:8-18)
     without index tensors; W: [n_levels, 2E].  Several levels per pass stay in LDS for n_cache 2 and 4.  Outputs are
     float32 unless out_dtype says otherwise (values between passes live in the outputs)."""
-    shape = validate(x, xa, W, cache_dim, nhead, activation, 0, n_levels)
+    shape = validate(x, xa, W, cache_dim, nhead, activation, 0, n_levels, alpha=alpha, m=m)
     dev = _require_gpu(x, xa, W)
     x, xa, w = _prep(x.detach()), _prep(xa.detach()), _w32(W)
     out_dtype = torch.float32 if out_dtype is None else out_dtype
@@ -388,7 +395,7 @@ def forward_radix(x, xa, W, alpha, activation, cache_dim, nhead, first_level, n_
 
 def inverse_radix(y, ya, W, alpha, activation, cache_dim, nhead, first_level, n_levels, *, m=M_DEFAULT):
     """x, xa (float32) with forward_radix(x, xa, ...) == (y, ya)."""
-    shape = validate(y, ya, W, cache_dim, nhead, activation, 0, n_levels, what="y")
+    shape = validate(y, ya, W, cache_dim, nhead, activation, 0, n_levels, what="y", alpha=alpha, m=m)
     dev = _require_gpu(y, ya, W)
     y, ya, w = _prep(y.detach()), _prep(ya.detach()), _w32(W)
     x = torch.empty(y.shape, dtype=torch.float32, device=dev)
@@ -408,7 +415,7 @@ def backward_radix(y, ya, dy, dya, W, alpha, activation, cache_dim, nhead, first
                    want_inputs=True):
     """Reversible backward of forward_radix from its outputs.  Returns (x_rec, xa_rec, dx, dxa, dW[n_levels, 2E]), all
     float32; x_rec, xa_rec are None when want_inputs is False (the library then does not write them)."""
-    shape = validate(y, ya, W, cache_dim, nhead, activation, 0, n_levels, what="y")
+    shape = validate(y, ya, W, cache_dim, nhead, activation, 0, n_levels, what="y", alpha=alpha, m=m)
     if dy.shape != y.shape or (dya is not None and dya.shape != y.shape):
         raise ValueError("dy/dya must have the shape of y")
     if dy.dtype not in _DTYPES or (dya is not None and dya.dtype != dy.dtype):

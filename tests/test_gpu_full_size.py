@@ -45,8 +45,11 @@ def _segment(n):
     return default_save_every(n)
 
 
-def _run(M, x, xa, dy, W, C, n, L, dtype):
-    """Forward + reversible backward the way bench.py runs the configuration: segments of default_save_every(n) stages."""
+def _run(M, x, xa, dy, W, C, n, L, dtype, want_inputs=False, with_inputs=False):
+    """Forward + reversible backward the way bench.py's timed step and the autograd nodes run the configuration:
+    segments of default_save_every(n) stages, and no reconstructed inputs asked of the backward (want_inputs=False: the
+    state between the stages of a segment travels through the workspace and the last pass writes gradients only).
+    want_inputs=True is the other form of the call, which also returns the reconstructed inputs of every segment."""
     seg = _segment(n)
     saved, spans = [], []
     cx, cxa = x, xa
@@ -61,11 +64,37 @@ def _run(M, x, xa, dy, W, C, n, L, dtype):
         spans.append((a, cnt))
     g, h = dy, None
     dWs = [None] * len(spans)
+    xr = xar = None
     for k in range(len(spans) - 1, -1, -1):
         a, cnt = spans[k]
-        _, _, g, h, dWs[k] = M.backward_stages(saved[k][0], saved[k][1], g, h, W[a:a + cnt], 0.9, 0, n, C, a, cnt,
-                                               grad_dtype=dtype if cnt == 1 else torch.float32, want_inputs=cnt > 1)
+        xr, xar, g, h, dWs[k] = M.backward_stages(saved[k][0], saved[k][1], g, h, W[a:a + cnt], 0.9, 0, n, C, a, cnt,
+                                                  grad_dtype=dtype if cnt == 1 else torch.float32,
+                                                  want_inputs=want_inputs)
+    if with_inputs:
+        return cx, cxa, g, h, torch.cat(dWs), xr, xar
     return cx, cxa, g, h, torch.cat(dWs)
+
+
+@pytest.mark.parametrize("name", ["cfg2", "cfg4", "cfg5"])
+def test_full_size_with_and_without_reconstructed_inputs(M, name):
+    """The two forms of the backward call at full size: the one that is timed (no reconstructed inputs) and the one
+    that also writes them.  They run the same kernels on the same values, so the gradients must agree bit for bit; the
+    reconstructed inputs of the first segment are the network inputs, to the rounding that reversing
+    default_save_every(n) stages amplifies."""
+    batch, N, E, C, n, L, dtype, _ = CONFIGS[name]
+    x, xa, dy, W = _inputs(name)
+    timed = _run(M, x, xa, dy, W, C, n, L, dtype)
+    other = _run(M, x, xa, dy, W, C, n, L, dtype, want_inputs=True, with_inputs=True)
+    for a, b in zip(timed, other[:5]):
+        assert torch.equal(a, b)
+    amp = (1 / 0.9) ** (n * min(_segment(n), L))
+    errs = {"x_rec": O.rel_err(other[5], x.float()), "xa_rec": O.rel_err(other[6], xa.float())}
+    print(f"measured reconstruction errors {name} (want_inputs=True): " + json.dumps(errs))
+    if os.environ.get("NCN_ERROR_REPORT"):
+        with open(os.environ["NCN_ERROR_REPORT"], "a") as fh:
+            fh.write(json.dumps({"config": name, "form": "want_inputs", **errs}) + "\n")
+    for v in errs.values():
+        assert v < max(1e-5, 1e-6 * amp)
 
 
 @pytest.mark.parametrize("name", list(CONFIGS))
@@ -156,7 +185,8 @@ def test_more_than_2_31_elements_per_array(M, case):
 
 @pytest.mark.parametrize("name,entries", [("cfg2", None), ("cfg5", None), ("cfg3", None), ("cfg4", None)])
 def test_whole_tensor_against_the_c_oracle(M, name, entries):
-    """Every element, not a slice: the configuration as bench.py runs it against the plain C restatement in float64
+    """Every element, not a slice: the configuration as bench.py's timed step runs it (backward without reconstructed
+    inputs) against the plain C restatement in float64
     (oracle/ncn_oracle.c on the host threads: about 25 s for the four configurations on 16 threads).  `entries` cuts
     the comparison to that many batch entries spread over the batch, for a machine where that is too long."""
     from oracle import c_oracle as CO

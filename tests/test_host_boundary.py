@@ -362,11 +362,60 @@ def test_header_is_valid_c(tmp_path):
 
 
 def test_library_staleness_check(lib, monkeypatch, tmp_path):
-    """load() builds a library that is missing or older than a source instead of failing: the check behind it."""
-    assert lib._stale_reason() is None                      # what build() left is newer than every source
+    """load() builds a library that is missing or was made from other sources instead of failing: the check behind it
+    compares contents (the build id compiled into the library against a hash of the sources), never file times."""
+    import shutil
+    from ncn_cuda_amd import _build
+    assert lib._stale_reason() is None                      # what build() left carries the hash of these sources
+    assert lib.load().ncn_build_id().decode() == _build.source_build_id() == _build.library_build_id()
+    # a source whose time stamp is newer than the library, content unchanged: not stale, and nothing to compile
+    src = os.path.join(_build.CSRC, "ncn_device.h")
+    before = os.stat(src)
+    try:
+        os.utime(src, None)
+        assert os.path.getmtime(src) > os.path.getmtime(_build.LIB_PATH)
+        assert lib._stale_reason() is None
+        assert _build.build(force=False) == []
+    finally:
+        os.utime(src, (before.st_atime, before.st_mtime))
+    # a library older than everything (as after a copy that keeps no times) is still current
+    lib_before = os.stat(_build.LIB_PATH)
+    try:
+        os.utime(_build.LIB_PATH, (1, 1))
+        assert lib._stale_reason() is None
+    finally:
+        os.utime(_build.LIB_PATH, (lib_before.st_atime, lib_before.st_mtime))
+    # changed content is what makes it stale: the same sources with one byte more in a header
+    copy = tmp_path / "csrc"
+    shutil.copytree(_build.CSRC, copy)
+    with open(copy / "ncn_device.h", "a") as fh:
+        fh.write("\n")
+    monkeypatch.setattr(_build, "CSRC", str(copy))
+    assert _build.source_build_id() != _build.library_build_id()
+    assert "other sources" in lib._stale_reason()
+    monkeypatch.undo()
+    # no library at all
     monkeypatch.setattr(lib, "LIB_PATH", str(tmp_path / "libncn_hip.so"))
     assert "missing" in lib._stale_reason()
-    (tmp_path / "libncn_hip.so").write_bytes(b"")
-    import os
-    os.utime(tmp_path / "libncn_hip.so", (1, 1))            # older than any source file
-    assert "older than" in lib._stale_reason()
+
+
+def test_stale_library_without_compiler_loads_with_a_warning(lib, monkeypatch, capsys):
+    """A box without hipcc and a library that does not match its sources: load it and say so, rather than fail."""
+    from ncn_cuda_amd import _build
+    monkeypatch.setattr(lib, "_lib", None)
+    monkeypatch.setattr(lib, "_stale_reason", lambda: "libncn_hip.so was built from other sources (test)")
+    monkeypatch.setattr(_build, "have_hipcc", lambda: False)
+    monkeypatch.setattr(_build, "build", lambda **kw: (_ for _ in ()).throw(AssertionError("must not build")))
+    assert lib.load() is not None
+    assert "no hipcc here" in capsys.readouterr().err
+
+
+def test_python_validation_rejects_scalars_no_kernel_takes(lib):
+    """alpha next to zero runs on the generic kernels, which take heads of up to 64 features: a clear error beyond."""
+    from ncn_cuda_amd import ncn_cuda_module as M
+    x = torch.zeros(1, 16, 256)
+    W = torch.zeros(512)
+    M.validate(x, x, W, 4, 2, 0, alpha=0.9, m=0.9)            # heads of 128: register kernels
+    M.validate(torch.zeros(1, 16, 64), torch.zeros(1, 16, 64), torch.zeros(128), 4, 2, 0, alpha=1e-5)   # generic
+    with pytest.raises(ValueError, match="generic kernels"):
+        M.validate(x, x, W, 4, 2, 0, alpha=1e-5, m=0.9)

@@ -62,11 +62,18 @@ def test_backward_static_matches_backward_on_two_calls_in_a_row():
     from ncn_cuda_amd import _lib
     lib = _lib.load()
     assert 0 < lib.ncn_static_scratch_bytes() <= 16 << 20
-    # first call: more tiles than the scratch has partial rows (a persistent loop over 4096 blocks), bf16 gradients
-    a, b = _call_both(lib, _lib, (24, 4096, 128, 4, 16), 1, seed=3, dtype=torch.bfloat16)
+    # first call: more wave tiles (40 * 128 = 5120) than the scratch has partial rows (4096): the grid is capped at
+    # 4096 partial rows and its waves loop over tiles, where ncn_backward launches a wave per tile; bf16 gradients
+    a, b = _call_both(lib, _lib, (40, 4096, 128, 4, 16), 1, seed=3, dtype=torch.bfloat16)
     for u, v in zip(a[:4], b[:4]):
         assert torch.equal(u, v)                         # dx, dxa, x_rec, xa_rec do not depend on the grid
     assert O.rel_err(b[4], a[4]) < 1e-5 and torch.isfinite(b[4]).all()   # the same terms summed over fewer partial rows
+    # the capped grid is rounded to whole multiples of n_head waves: three heads (blocks in threes) and two
+    for shape5 in ((40, 4096, 96, 3, 16), (40, 4096, 64, 2, 16)):
+        a, b = _call_both(lib, _lib, shape5, 1, seed=6)
+        for u, v in zip(a[:4], b[:4]):
+            assert torch.equal(u, v)
+        assert O.rel_err(b[4], a[4]) < 1e-5 and torch.isfinite(b[4]).all()
     # second call, smaller, three stages: what the first call left in the scratch must not show
     a, b = _call_both(lib, _lib, (2, 96, 32, 4, 4), 3, seed=4)
     for u, v in zip(a, b):
@@ -86,3 +93,29 @@ def test_backward_static_rejects_what_its_scratch_cannot_hold():
     p = ctypes.c_void_p(4096)                             # never dereferenced: the size check comes first
     rc = lib.ncn_backward_static(p, p, 0, p, p, 0, p, p, 0, None, None, p, p, ctypes.byref(sh), 0, 1, 0.9, 0.9, 0, None)
     assert rc == -9 and "scratch" in _lib.error_string(rc)
+
+
+def test_backward_static_needs_the_state_buffers_for_several_stages():
+    """With n_stages > 1 the stages hand their reconstructed inputs on through x_rec, xa_rec; ncn_backward takes two
+    arrays from its workspace when they are NULL, the static scratch has no room for them: NCN_ERR_ALIAS."""
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from ncn_cuda_amd import _lib
+    lib = _lib.load()
+    batch, N, E, C, n, L = 2, 64, 32, 4, 4, 3
+    dev = torch.device("cuda:0")
+    sh = _lib.NcnShape(batch, N, E, C, n)
+    t = [torch.randn(batch, N, E, device=dev) for _ in range(3)]
+    out = [torch.empty(batch, N, E, device=dev) for _ in range(2)]
+    W = torch.randn(L, 2 * E, device=dev) * 0.3
+    dW = torch.empty(L, 2 * E, device=dev)
+    rc = lib.ncn_backward_static(t[0].data_ptr(), t[1].data_ptr(), 0, t[2].data_ptr(), None, 0, out[0].data_ptr(),
+                                 out[1].data_ptr(), 0, None, None, W.data_ptr(), dW.data_ptr(), ctypes.byref(sh), 0, L,
+                                 0.9, 0.9, 0, None)
+    assert rc == -8 and "x_rec" in _lib.error_string(rc)
+    # one stage takes the NULLs, as ncn_backward does
+    rc = lib.ncn_backward_static(t[0].data_ptr(), t[1].data_ptr(), 0, t[2].data_ptr(), None, 0, out[0].data_ptr(),
+                                 out[1].data_ptr(), 0, None, None, W.data_ptr(), dW.data_ptr(), ctypes.byref(sh), 0, 1,
+                                 0.9, 0.9, 0, None)
+    torch.cuda.synchronize()
+    assert rc == 0 and torch.isfinite(out[0]).all() and torch.isfinite(dW[0]).all()
