@@ -2,7 +2,8 @@
 """Headline benchmark: NCN forward + backward of the full stage stack on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg3|cfg2|cfg4|cfg5] [--no-cpu]
-                    [--grouping closed|stride-table|radix-table|ragged|radix]
+                    [--grouping closed|stride-table|radix-table|ragged|radix] [--save-every K] [--scalar-heads]
+                    [--no-surface]
 
 One step = forward of all L stages (each stage saving its outputs, like the reference's autograd
 node) + reversible backward of all L stages producing dx, dxa and every dW_l, on inputs that are
@@ -15,6 +16,13 @@ backward call over a segment of stages where several stages run per launch) agai
 it: float32 vector arithmetic for groups of 8 rows and more (each element takes n_cache sequential tanh
 steps per stage), HBM bandwidth for smaller groups.  Its duration is measured with HIP events on the
 launch stream inside the timed region; the figures for the other roof ride along as hbm_* / valu_*.
+`roofline.frac` is against the published peak (157.3 TFLOP/s, which counts packed FP32 instructions; 8 TB/s); what
+this GPU sustains is measured in the same run and quoted beside it: `attainable_valu_TFLOPs` (a stream of independent
+plain v_fma_f32, the library's ncn_probe_fma_stream; the library is built without packed FP32) and
+`attainable_copy_GBps` (a 1 GiB device copy).
+`stack.autograd_*` time the same workload through the reference's own surface (NCNNetTestCuda + yi.backward(dyi),
+grad_test_bench.py:116-134) and through the one-node form of the stack, `stack.graph_ms_per_step` replays the timed
+step from a HIP graph; all three outside the headline timed region.
 `roofline.traffic` is read from profiles/traffic.json (rocprofv3 FETCH_SIZE + WRITE_SIZE of that kernel,
 recorded for one library version) and is null when that file has no entry for this library version.
 `cpu_baseline` times the checker's plain C restatement (and, beside it, the PyTorch one) on a bounded
@@ -40,7 +48,6 @@ CONFIGS = {
 }
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 VALU_PEAK_TFLOPS = 157.3   # MI355X FP32 vector peak, which counts packed FP32 instructions
-VALU_PEAK_TFLOPS_UNPACKED = 78.6   # the same without them (this build does not use packed FP32)
 # float32 operations per element and step of the kernels as written in ncn_stage_kernels.h (FMA = 2, exp2 and
 # rcp = 1 each), without the per-row and per-lane bookkeeping: forward 5 FMA (row sum, z, two for xa, x) + the
 # +1 before the reciprocal + exp2 + rcp = 13; backward 12 FMA (inversion of x, row sum, z, two for xa, F'/4, the
@@ -79,6 +86,14 @@ def main():
                          "lengths and no table, whole segments per call (multi-stage LDS passes for small groups).  radix: levels 0 .. L-1 of the radix-n digit grouping "
                          "through ncn_forward_radix / ncn_backward_radix (needs n_cache^L to divide N; several levels "
                          "per LDS pass for n_cache 2 and 4; float32 between calls)")
+    ap.add_argument("--save-every", type=int, default=0,
+                    help="stages per saved checkpoint (0: what the whole-net autograd node chooses, "
+                         "modules.default_save_every)")
+    ap.add_argument("--scalar-heads", action="store_true",
+                    help="the literal scalar reading of x[B, D]: one feature per head (n_head = E), a different shape "
+                         "from the one the metric is quoted on; runs on the generic kernels")
+    ap.add_argument("--no-surface", action="store_true",
+                    help="skip the legs outside the timed region that go through the autograd surface and a HIP graph")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one plain 1 GiB device copy, so that a rocprofv3 --pmc run has a kernel of known "
                          "traffic to calibrate FETCH_SIZE / WRITE_SIZE against")
@@ -97,6 +112,8 @@ def main():
         sys.exit(2)
     cfg = CONFIGS[args.config]
     batch, N, E, C, n, L = cfg["batch"], cfg["N"], cfg["E"], cfg["C"], cfg["n"], cfg["L"]
+    if args.scalar_heads:
+        C = E
     io_dtype = torch.bfloat16 if cfg["dtype"] == "bf16" else torch.float32
     alpha = 0.9
     tokens = batch * E
@@ -118,7 +135,10 @@ def main():
     # Stages per saved checkpoint: 1 for the headline shape (every stage saves its outputs, like the reference's
     # autograd node); small groups run whole segments per call (multi-stage LDS passes) and reverse them from the
     # segment's outputs: rounding grows like (1/m)^(n_cache * stages), kept below 16x.
-    save_every = max(1, 26 // n) if args.grouping in ("closed", "radix", "lengths") else 1   # tables run stage by stage
+    from ncn_cuda_amd.modules import default_save_every
+    save_every = 1   # tables run stage by stage
+    if args.grouping in ("closed", "radix", "lengths"):
+        save_every = args.save_every if args.save_every > 0 else default_save_every(n, L, batch * N * E)
     tables = lens = None
     if args.grouping == "lengths":   # the closed-form permutation with one context length per batch entry
         lens = (N - 1 - torch.arange(batch, device=dev) % n).to(torch.int32)
@@ -216,6 +236,80 @@ def main():
     copy_gbps = 5 * 2.0 * src.numel() * 4 / (c0.elapsed_time(c1) * 1e-3) / 1e9
     del src, dst
 
+    # what this GPU sustains on plain float32 FMAs (no packed instructions, as the library is built): a stream of
+    # independent v_fma_f32, 8 waves per SIMD, timed here with events on the launch stream
+    lib = M._lib.load()
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    fma_blocks, fma_iters = 8 * cus, 2048
+    probe_out = torch.empty(fma_blocks * 256, dtype=torch.float32, device=dev)
+    stream_ptr = torch.cuda.current_stream(dev).cuda_stream
+    M._lib.check(lib.ncn_probe_fma_stream(probe_out.data_ptr(), fma_blocks, fma_iters, stream_ptr), "ncn_probe_fma_stream")
+    f0, f1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    f0.record()
+    for _ in range(3):
+        M._lib.check(lib.ncn_probe_fma_stream(probe_out.data_ptr(), fma_blocks, fma_iters, stream_ptr), "ncn_probe_fma_stream")
+    f1.record()
+    torch.cuda.synchronize()
+    fma_flops = 2.0 * lib.ncn_probe_fma_per_thread(fma_iters) * fma_blocks * 256
+    attainable_valu = 3 * fma_flops / (f0.elapsed_time(f1) * 1e-3) / 1e12
+    del probe_out
+
+    # The same workload through the autograd surface the reference times (NCNNetTestCuda(...)(x, xa); yi.backward(dyi),
+    # grad_test_bench.py:116-134: one node per stage) and through the one-node form of the stack; then the timed step
+    # replayed from a HIP graph (launch gaps taken out).  Medians of HIP-event brackets, outside the timed region.
+    surface = {"autograd_per_stage_nodes_ms_per_step": None, "autograd_one_node_ms_per_step": None,
+               "graph_ms_per_step": None}
+    if not args.no_surface and args.grouping == "closed":
+        import ncn_cuda_amd
+
+        def timed_median(fn, reps):
+            for _ in range(3):
+                fn()
+            ev = [torch.cuda.Event(enable_timing=True) for _ in range(reps + 1)]
+            ev[0].record()
+            for k in range(reps):
+                fn()
+                ev[k + 1].record()
+            torch.cuda.synchronize()
+            t = sorted(ev[k].elapsed_time(ev[k + 1]) for k in range(reps))
+            return t[len(t) // 2]
+
+        ax, axa = gx.clone().requires_grad_(), gxa.clone().requires_grad_()
+        aWs = [w.clone().requires_grad_() for w in gWs]
+
+        def through(net):
+            def run():
+                ax.grad = axa.grad = None
+                for w in aWs:
+                    w.grad = None
+                yi, _ = net(ax, axa)
+                yi.backward(gdyi)
+            return run
+
+        reps = max(5, min(args.steps, 20))
+        surface["autograd_per_stage_nodes_ms_per_step"] = timed_median(
+            through(ncn_cuda_amd.NCNNetTestCuda(alpha, "tanh", n, C, L, aWs)), reps)
+        surface["autograd_one_node_ms_per_step"] = timed_median(
+            through(ncn_cuda_amd.NCNNetTestCuda(alpha, "tanh", n, C, L, aWs, fuse_stages=True,
+                                                save_every=save_every)), reps)
+        del ax, axa, aWs
+        try:
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                step()                       # every kernel's attributes are set before the capture
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                graph_out = step()
+            surface["graph_ms_per_step"] = timed_median(graph.replay, reps)
+            surface["graph_replay_matches_eager"] = bool(
+                torch.equal(graph_out[2], out[2]) and all(torch.equal(a, b) for a, b in zip(graph_out[4], out[4])))
+            del graph, graph_out
+        except RuntimeError as exc:      # a capture the runtime refuses is reported, not fatal to the headline figure
+            surface["graph_error"] = str(exc).splitlines()[0][:200]
+
     # the invertible-inverse pass over the whole stack (not part of the step; the invertible configuration, cfg5, is quoted with it):
     # from the final outputs back to the inputs, segment by segment as the backward reverses them
     inverse_ms = None
@@ -267,7 +361,7 @@ def main():
     # bytes from 8 rows per group on (one launch per stage); the multi-stage passes of small groups are built to be
     # limited by their HBM round trips
     valu_bound = n >= 8
-    version = M._lib.load().ncn_version().decode()
+    version = lib.ncn_version().decode()
     kernel = (f"stage_backward_kernel<{n},{E // C}>" + (" (indexed build)" if tables else "") if not lds_passes else
               f"backward call over a segment of up to {save_every} stages (multi-stage passes)")
     roof = {"bound": "fp32_valu" if valu_bound else "hbm",
@@ -280,7 +374,7 @@ def main():
             "algorithmic_flops_per_launch": flops_bwd_unit,
             "algorithmic_bytes_per_launch": bytes_bwd_launch,
             "valu_achieved_TFLOPs": valu_achieved, "valu_frac_of_packed_peak": valu_achieved / VALU_PEAK_TFLOPS,
-            "valu_frac_of_unpacked_peak": valu_achieved / VALU_PEAK_TFLOPS_UNPACKED,
+            "attainable_valu_TFLOPs": attainable_valu, "valu_frac_of_attainable": valu_achieved / attainable_valu,
             "hbm_achieved_GBps": hbm_achieved, "hbm_frac": hbm_achieved / HBM_PEAK_GBS,
             "attainable_copy_GBps": copy_gbps, "hbm_frac_of_attainable_copy": hbm_achieved / copy_gbps,
             "ncn_version": version}
@@ -311,7 +405,8 @@ def main():
                   "fp32_flops_per_step": flops_step,
                   "achieved_TFLOPs": flops_step / (ms_per_step * 1e-3) / 1e12,
                   "frac_of_fp32_vector_peak": flops_step / (ms_per_step * 1e-3) / 1e12 / VALU_PEAK_TFLOPS,
-                  "frac_of_fp32_vector_peak_unpacked": flops_step / (ms_per_step * 1e-3) / 1e12 / VALU_PEAK_TFLOPS_UNPACKED,
+                  "frac_of_attainable_valu": flops_step / (ms_per_step * 1e-3) / 1e12 / attainable_valu,
+                  **surface,
                   "inverse_ms_per_stack": inverse_ms,
                   "inverse_reconstruction_rel_err": recon_err if inverse_ms is not None else None},
     }

@@ -36,6 +36,9 @@ class NCNFunction(torch.autograd.Function):
     def forward(ctx, x, xa, W, alpha, activation, n_cache, n_head, module_l):
         yi, ya, sy, sya = ncn_cuda_module.forward_stages_saving(x, xa, W, alpha, activation, n_cache, n_head, module_l)
         ctx.save_for_backward(sy, sya, W)
+        # an output nobody differentiates (ya of the last stage under yi.backward(dyi), grad_test_bench.py:121) arrives
+        # as None instead of a tensor of zeros that autograd would have to fill and the kernel to read
+        ctx.set_materialize_grads(False)
         ctx.alpha = alpha
         ctx.activation = activation
         ctx.n_cache = n_cache
@@ -47,6 +50,10 @@ class NCNFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dyi, dya):
         (yi, ya, W) = ctx.saved_tensors
+        if dyi is None:
+            if dya is None:
+                return (None,) * 8
+            dyi = torch.zeros_like(dya)
         _, _, dx, dxa, dW = ncn_cuda_module.backward_stages(
             yi, ya, dyi, dya, W, ctx.alpha, ctx.activation, ctx.n_cache, ctx.n_head, ctx.module_l, 1,
             grad_dtype=ctx.io_dtype, want_inputs=False)
@@ -54,31 +61,54 @@ class NCNFunction(torch.autograd.Function):
         return dx, dxa, sum_dW, None, None, None, None, None
 
 
-def default_save_every(n_cache: int) -> int:
-    """Stages per saved checkpoint of the whole-net node: the reversible backward amplifies float32 rounding by
-    (1/m)^(n_cache * stages) between checkpoints; 26 steps keep that below 16x at m = 0.9."""
-    return max(1, 26 // max(1, int(n_cache)))
+# Saved activations that the whole-net node may keep before it trades memory for time (see default_save_every).
+SAVE_BUDGET_BYTES = 32 << 30
+
+
+def default_save_every(n_cache: int, n_stages: int = None, elements: int = None, budget_bytes: int = None) -> int:
+    """Stages per saved checkpoint of the whole-net node.
+
+    Groups of 2 and 4 rows run several stages per launch out of LDS, so long segments save HBM round trips; the
+    reversible backward amplifies float32 rounding by (1/m)^(n_cache * stages) between checkpoints, and 26 steps keep
+    that below 16x at m = 0.9: segments of 26 // n_cache stages.
+    Larger groups run one launch per stage whatever the segment, and a backward launch that need not hand the
+    reconstructed inputs on to the next stage moves 6 instead of 7-8 arrays: every stage's outputs are kept (which the
+    forward writes anyway) as long as they fit the budget, 2 float32 arrays of `elements` values per stage against
+    `budget_bytes` (default SAVE_BUDGET_BYTES); beyond it, or when the sizes are not given, segments as above."""
+    by_rounding = max(1, 26 // max(1, int(n_cache)))
+    if int(n_cache) <= 4 or n_stages is None or elements is None:
+        return by_rounding
+    budget = SAVE_BUDGET_BYTES if budget_bytes is None else int(budget_bytes)
+    return 1 if 2 * 4 * int(elements) * int(n_stages) <= budget else by_rounding
 
 
 class NCNNetFunction(torch.autograd.Function):
     """The whole stage stack as ONE autograd node (no counterpart in the reference, which chains one NCNFunction
     per stage, ncn_pytorch_wrapper_v2.py:107-117).  Stages run `save_every` at a time through the library's
-    multi-stage calls; only the float32 outputs of every `save_every`-th stage are kept for backward, which
-    reverses each segment from its outputs.  Inter-stage activations stay float32 whatever the I/O dtype."""
+    multi-stage calls; only the outputs of every `save_every`-th stage are kept for backward, which reverses each
+    segment from its outputs.  Segments of several stages keep float32 between the stages whatever the I/O dtype;
+    segments of one stage keep the I/O dtype and save what NCNFunction saves (for bfloat16 the outputs plus what
+    their rounding took away, as two bfloat16 planes)."""
 
     @staticmethod
     def forward(ctx, x, xa, alpha, activation, n_cache, n_head, first_stage, save_every, *weights):
         L = len(weights)
-        save_every = default_save_every(n_cache) if not save_every else int(save_every)
+        save_every = default_save_every(n_cache, L, x.numel()) if not save_every else int(save_every)
         W = torch.stack([w.detach().reshape(-1).to(torch.float32) for w in weights])
         saved = []
         cx, cxa = x, xa
         segs = [(a, min(save_every, L - a)) for a in range(0, L, save_every)]
         for a, cnt in segs:
-            cx, cxa = ncn_cuda_module.forward_stages(cx, cxa, W[a:a + cnt], alpha, activation, n_cache, n_head,
-                                                     first_stage + a, cnt, out_dtype=torch.float32)
-            saved.extend([cx, cxa])
+            if cnt == 1 and cx.dtype == x.dtype:
+                cx, cxa, sy, sya = ncn_cuda_module.forward_stages_saving(cx, cxa, W[a], alpha, activation, n_cache,
+                                                                         n_head, first_stage + a)
+                saved.extend([sy, sya])
+            else:
+                cx, cxa = ncn_cuda_module.forward_stages(cx, cxa, W[a:a + cnt], alpha, activation, n_cache, n_head,
+                                                         first_stage + a, cnt, out_dtype=torch.float32)
+                saved.extend([cx, cxa])
         ctx.save_for_backward(W, *saved)
+        ctx.set_materialize_grads(False)   # a missing upstream gradient stays None (see NCNFunction)
         ctx.cfg = (alpha, activation, n_cache, n_head, first_stage, segs, x.dtype, [w.dtype for w in weights],
                    [w.shape for w in weights])
         return cx.to(x.dtype), cxa.to(x.dtype)
@@ -88,12 +118,19 @@ class NCNNetFunction(torch.autograd.Function):
         W, *saved = ctx.saved_tensors
         alpha, activation, n_cache, n_head, first_stage, segs, io_dtype, w_dtypes, w_shapes = ctx.cfg
         dWs = [None] * W.shape[0]
+        if dyi is None:
+            if dya is None:
+                return (None,) * (8 + W.shape[0])
+            dyi = torch.zeros_like(dya)
         g, ga = dyi, dya
         for k in range(len(segs) - 1, -1, -1):
             a, cnt = segs[k]
+            # a one-stage segment hands its gradients on in the dtype they came in (bfloat16 stays bfloat16)
+            gd = g.dtype if cnt == 1 else torch.float32
+            Wk = W[a] if cnt == 1 else W[a:a + cnt]
             _, _, g, ga, dW = ncn_cuda_module.backward_stages(
-                saved[2 * k], saved[2 * k + 1], g, ga, W[a:a + cnt], alpha, activation, n_cache, n_head,
-                first_stage + a, cnt, grad_dtype=torch.float32, want_inputs=False)
+                saved[2 * k], saved[2 * k + 1], g, ga, Wk, alpha, activation, n_cache, n_head,
+                first_stage + a, cnt, grad_dtype=gd, want_inputs=False)
             for j in range(cnt):
                 dWs[a + j] = dW[j].reshape(w_shapes[a + j]).to(w_dtypes[a + j])
         return (g.to(io_dtype), ga.to(io_dtype), None, None, None, None, None, None, *dWs)
@@ -116,6 +153,7 @@ class NCNRadixNetFunction(torch.autograd.Function):
                                                     first_level + a, cnt)
             saved.extend([cx, cxa])
         ctx.save_for_backward(W, *saved)
+        ctx.set_materialize_grads(False)   # a missing upstream gradient stays None (see NCNFunction)
         ctx.cfg = (alpha, activation, n_cache, n_head, first_level, segs, x.dtype, [w.dtype for w in weights],
                    [w.shape for w in weights])
         return cx.to(x.dtype), cxa.to(x.dtype)
@@ -125,6 +163,10 @@ class NCNRadixNetFunction(torch.autograd.Function):
         W, *saved = ctx.saved_tensors
         alpha, activation, n_cache, n_head, first_level, segs, io_dtype, w_dtypes, w_shapes = ctx.cfg
         dWs = [None] * W.shape[0]
+        if dyi is None:
+            if dya is None:
+                return (None,) * (8 + W.shape[0])
+            dyi = torch.zeros_like(dya)
         g, ga = dyi, dya
         for k in range(len(segs) - 1, -1, -1):
             a, cnt = segs[k]

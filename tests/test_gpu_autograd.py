@@ -117,6 +117,9 @@ def test_whole_net_node_matches_oracle_and_per_stage_nodes(pkg, cfg):
             assert got[4][l].dtype == dtype
             assert O.rel_err(got[4][l], ref[4][l]) < tol, f"dW{l}"
     assert pkg.default_save_every(2) == 13 and pkg.default_save_every(16) == 1
+    # groups of 8 rows and more keep every stage's outputs while they fit the memory budget, segments beyond it
+    assert pkg.default_save_every(8) == 3 and pkg.default_save_every(8, 4, 1 << 24) == 1
+    assert pkg.default_save_every(8, 4, 1 << 24, budget_bytes=1 << 20) == 3 and pkg.default_save_every(2, 13, 1 << 24) == 13
 
 
 def test_net_cuda_fuse_stages_flag_keeps_parameters(pkg):
@@ -160,3 +163,30 @@ def test_triton_named_surface_matches_cuda_named_surface(pkg):
     d = torch.float64
     ref = O.net_autograd(x.to(d), xa.to(d), [w.to(d) for w in Ws], dy.to(d), dya.to(d), 0.9, n, C, activation=-1)
     assert O.rel_err(res[0][0], ref[0]) < 1e-5 and O.rel_err(res[0][2], ref[2]) < 1e-5
+
+
+@pytest.mark.parametrize("fuse", [False, True], ids=["per_stage_nodes", "one_node"])
+def test_missing_upstream_gradients_are_not_materialised(pkg, fuse):
+    """yi.backward(dyi) (grad_test_bench.py:121) leaves ya without a gradient: the nodes take None for it (no tensor of
+    zeros is made) and give what explicit zeros give, bit for bit; only dya works too, and neither gives no gradient."""
+    batch, N, E, C, n, L = 2, 128, 128, 4, 4, 3
+    x, xa, Ws, dyi, dya = O.make_inputs(batch, N, E, L, n, seed=5, xa_zero=False)
+
+    def run(which):
+        gx, gxa = x.cuda().requires_grad_(), xa.cuda().requires_grad_()
+        gWs = [w.cuda().requires_grad_() for w in Ws]
+        yi, ya = pkg.NCNNetTestCuda(0.9, "tanh", n, C, L, gWs, fuse_stages=fuse)(gx, gxa)
+        if which == "yi":
+            yi.backward(dyi.cuda())
+        elif which == "ya":
+            ya.backward(dya.cuda())
+        elif which == "yi_zeros":
+            torch.autograd.backward([yi, ya], [dyi.cuda(), torch.zeros_like(ya)])
+        else:
+            torch.autograd.backward([yi, ya], [torch.zeros_like(yi), dya.cuda()])
+        return [gx.grad, gxa.grad] + [w.grad for w in gWs]
+
+    for a, b in zip(run("yi"), run("yi_zeros")):
+        assert torch.equal(a, b)
+    for a, b in zip(run("ya"), run("zeros_ya")):
+        assert torch.equal(a, b)

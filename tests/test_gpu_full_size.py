@@ -39,10 +39,10 @@ def _inputs(name):
     return x, xa, dy, W
 
 
-def _segment(n):
+def _segment(n, L=None, elements=None):
     """Stages per saved checkpoint, as bench.py and the whole-net autograd node choose it."""
     from ncn_cuda_amd.modules import default_save_every
-    return default_save_every(n)
+    return default_save_every(n, L, elements)
 
 
 def _run(M, x, xa, dy, W, C, n, L, dtype, want_inputs=False, with_inputs=False):
@@ -50,7 +50,7 @@ def _run(M, x, xa, dy, W, C, n, L, dtype, want_inputs=False, with_inputs=False):
     segments of default_save_every(n) stages, and no reconstructed inputs asked of the backward (want_inputs=False: the
     state between the stages of a segment travels through the workspace and the last pass writes gradients only).
     want_inputs=True is the other form of the call, which also returns the reconstructed inputs of every segment."""
-    seg = _segment(n)
+    seg = _segment(n, L, x.numel())
     saved, spans = [], []
     cx, cxa = x, xa
     for a in range(0, L, seg):
@@ -87,7 +87,7 @@ def test_full_size_with_and_without_reconstructed_inputs(M, name):
     other = _run(M, x, xa, dy, W, C, n, L, dtype, want_inputs=True, with_inputs=True)
     for a, b in zip(timed, other[:5]):
         assert torch.equal(a, b)
-    amp = (1 / 0.9) ** (n * min(_segment(n), L))
+    amp = (1 / 0.9) ** (n * min(_segment(n, L, x.numel()), L))
     errs = {"x_rec": O.rel_err(other[5], x.float()), "xa_rec": O.rel_err(other[6], xa.float())}
     print(f"measured reconstruction errors {name} (want_inputs=True): " + json.dumps(errs))
     if os.environ.get("NCN_ERROR_REPORT"):
@@ -133,7 +133,7 @@ def test_full_size_inverse_round_trip(M, name):
     batch, N, E, C, n, L, dtype, _ = CONFIGS[name]
     x, xa, _, W = _inputs(name)
     x, xa = x.float(), xa.float()
-    seg = _segment(n)
+    seg = _segment(n, L, x.numel())
     for a in range(0, L, seg):            # reversal is only asked over what one saved checkpoint covers
         cnt = min(seg, L - a)
         y, ya = M.forward_stages(x, xa, W[a:a + cnt], 0.9, 0, n, C, a, cnt)
@@ -207,10 +207,10 @@ def test_whole_tensor_against_the_c_oracle(M, name, entries):
     if entries is None:                                            # dW sums over the whole batch
         per_stage = [O.rel_err(dW[l].cpu(), ref[4][l]) for l in range(L)]
         report["dW_worst"] = {"max": max(per_stage), "rms": max(O.rms_err(dW[l].cpu(), ref[4][l]) for l in range(L))}
-    print(f"measured errors {name} (segments of {_segment(n)} stages): " + json.dumps(report))
+    print(f"measured errors {name} (segments of {_segment(n, L, x.numel())} stages): " + json.dumps(report))
     if os.environ.get("NCN_ERROR_REPORT"):                         # a file to read the figures from after a run
         with open(os.environ["NCN_ERROR_REPORT"], "a") as fh:
-            fh.write(json.dumps({"config": name, "segment": _segment(n), **report}) + "\n")
+            fh.write(json.dumps({"config": name, "segment": _segment(n, L, x.numel()), **report}) + "\n")
     for k, v in report.items():
         assert v["max"] < tol, (k, v)
 
