@@ -28,7 +28,8 @@ size_t fused_lds_bytes(int nc, int ec, bool backward, uint32_t window, int n_sta
     const TileShape t = fast_tile(nc, ec);
     const int lr = nc / t.r;
     // groups of two rows keep their slot-0 rows in registers (ncn_fused_pair_kernels.h): one row per group in LDS
-    size_t bytes = (size_t)(backward ? 4 : 2) * window * (nc == 2 ? 1 : nc) * ec * sizeof(float);
+    size_t bytes = nc == 2 ? pair_state_bytes(backward) / 2   // the arrays of the largest window, whatever this one's size
+                           : (size_t)(backward ? 4 : 2) * window * nc * ec * sizeof(float);
     bytes += (size_t)kFusedMaxStages * 2 * ec * sizeof(float);  // the pass's weights
     const int nw = backward ? (nc == 2 ? kPairWavesBwd : kFusedWavesBwd) : kFusedWavesFwd;
     if (lr > 1) bytes += (size_t)nw * t.f * 64 * sizeof(float);
@@ -156,7 +157,7 @@ static hipError_t launch_fused_t(Pass pass, const FusedArgs& a, int grid, size_t
     hipError_t err;
     const bool tanh_only = a.tab.activation == NCN_ACT_TANH;
     if constexpr (NC == 2) {
-        static_assert(t.r == 2 && t.f == 4, "the two-row kernels are written for 2 x 4 tiles");
+        static_assert(t.r == 2, "the two-row kernels keep both rows of a group in one lane");
         if (!backward && (uint32_t)grid != a.total_items) return hipErrorInvalidConfiguration;   // one window each
         if (backward) {
             // a workgroup per window when the dW scratch has the rows for it, else workgroups that loop over windows

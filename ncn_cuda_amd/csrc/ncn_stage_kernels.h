@@ -239,16 +239,20 @@ __device__ __forceinline__ void inverse_core(float (&y)[R][F], float (&b)[R][F],
 // group whose dW another tile accounts for).
 // STEP_MASK: steps j >= live leave the registers as they are (the caller scales G, P as if they had been done).
 // ---------------------------------------------------------------------------------------------
-template <int NC, int EC, int R, int F, bool MASKED, bool TANH_ONLY = true, bool STEP_MASK = false, bool ROWS = false>
+// KU_W: the products ku Wi' are kept beside the weights (F more registers, one multiplication less per row and step).
+template <int NC, int EC, int R, int F, bool MASKED, bool TANH_ONLY = true, bool STEP_MASK = false, bool ROWS = false,
+          bool KU_W = true>
 __device__ __forceinline__ void backward_core(float (&Y)[R][F], float (&B)[R][F], float (&G)[R][F], float (&P)[R][F],
                                               const float (&wi)[F], const float (&wj)[F], float (&dwi)[F],
                                               float (&dwj)[F], float own, const StepTable& S, int step_base, int lane,
                                               float4* slots, int live = NC) {
     using T = Tile<NC, EC, R, F>;
     const int rl = (lane / T::LF) % T::LR;
-    float wiku[F];   // ku Wi': G += rh (ku Wi') spares the product ku rh of every row and step
+    float wiku[KU_W ? F : 1];   // ku Wi': G += rh (ku Wi') spares the product ku rh of every row and step
+    if constexpr (KU_W) {
 #pragma unroll
-    for (int f = 0; f < F; ++f) wiku[f] = S.ku * wi[f];
+        for (int f = 0; f < F; ++f) wiku[f] = S.ku * wi[f];
+    }
 #pragma unroll 1
     for (int jo = T::LR - 1; jo >= 0; --jo) {
         const float selku = (T::LR == 1 || rl == jo) ? S.ku : 0.0f;  // this lane holds the pivot row
@@ -261,9 +265,62 @@ __device__ __forceinline__ void backward_core(float (&Y)[R][F], float (&B)[R][F]
             for (int rr = 0; rr < R; ++rr)
 #pragma unroll
                 for (int f = 0; f < F; ++f) Y[rr][f] = fmaf(S.im, Y[rr][f], -B[rr][f]);  // xs before this step
-            float xj[F], v[F], c[R], rh[R];
+            float xj[F], c[R], rh[R];
             row_lane_broadcast<T::LF, T::LR, F>(Y[jr], xj, jo, lane, slots);
             row_sums<T::LF, R, F, ROWS>(Y, wi, dot_chain<F>(xj, wj), c);
+            if constexpr (T::LR == 1) {
+                // The whole group is in this lane: the pivot row's share sum_i c_i U_i goes straight into its gradient
+                // (no sum across lanes to wait for), with the pivot's own two terms merged into one coefficient.
+                float kc[R];
+#pragma unroll
+                for (int rr = 0; rr < R; ++rr) kc[rr] = (rr == jr) ? fmaf(S.ku, c[rr], S.ku) : S.ku * c[rr];
+#pragma unroll
+                for (int rr = 0; rr < R; ++rr) {
+                    rh[rr] = 0.f;
+#pragma unroll
+                    for (int f = 0; f < F; ++f) {
+                        const float z = fmaf(c[rr], xj[f], Y[rr][f]);
+                        float w;
+                        if constexpr (TANH_ONLY) {
+                            const float r = __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(z) + 1.0f);
+                            B[rr][f] = fmaf(S.bk1, r, fmaf(S.im, B[rr][f], S.bk0));   // bh before this step
+                            w = fmaf(-r, r, r);
+                        } else {
+                            float Fv;
+                            act_Fw(z, S.activation, Fv, w);
+                            B[rr][f] = fmaf(S.bk0, Fv, S.im * B[rr][f]);
+                        }
+                        const float U = P[rr][f] * w;
+                        rh[rr] = fmaf(U, xj[f], rh[rr]);
+                        if (rr != jr) G[rr][f] = fmaf(S.ku, U, G[rr][f]);
+                        G[jr][f] = fmaf(kc[rr], U, G[jr][f]);
+                    }
+                }
+                lane_sum_n<1, T::LF, ROWS, R>(rh);
+                float rhosum = 0.f;
+#pragma unroll
+                for (int rr = 0; rr < R; ++rr) {
+                    const float rho_w = krho * rh[rr];     // (1-alpha) r_i / kappa, weighted
+                    const float rho_ku = KU_W ? rh[rr] : S.ku * rh[rr];
+                    rhosum += rh[rr];
+#pragma unroll
+                    for (int f = 0; f < F; ++f) {
+                        dwi[f] = fmaf(rho_w, Y[rr][f], dwi[f]);
+                        G[rr][f] = fmaf(rho_ku, KU_W ? wiku[f] : wi[f], G[rr][f]);
+                    }
+                }
+                const float rhosum_w = krho * rhosum, rhosum_ku = S.ku * rhosum;
+#pragma unroll
+                for (int f = 0; f < F; ++f) {
+                    dwj[f] = fmaf(rhosum_w, xj[f], dwj[f]);
+                    G[jr][f] = fmaf(rhosum_ku, wj[f], G[jr][f]);
+                }
+#pragma unroll
+                for (int rr = 0; rr < R; ++rr)
+#pragma unroll
+                    for (int f = 0; f < F; ++f) P[rr][f] = fmaf(S.om, G[rr][f], P[rr][f]);
+            } else {
+            float v[F];
 #pragma unroll
             for (int f = 0; f < F; ++f) v[f] = 0.f;
 #pragma unroll
@@ -293,11 +350,12 @@ __device__ __forceinline__ void backward_core(float (&Y)[R][F], float (&B)[R][F]
 #pragma unroll
             for (int rr = 0; rr < R; ++rr) {
                 const float rho_w = krho * rh[rr];     // (1-alpha) r_i / kappa, weighted
+                const float rho_ku = KU_W ? rh[rr] : S.ku * rh[rr];
                 rhosum += rh[rr];
 #pragma unroll
                 for (int f = 0; f < F; ++f) {
                     dwi[f] = fmaf(rho_w, Y[rr][f], dwi[f]);
-                    G[rr][f] = fmaf(rh[rr], wiku[f], G[rr][f]);
+                    G[rr][f] = fmaf(rho_ku, KU_W ? wiku[f] : wi[f], G[rr][f]);
                     if (rr != jr) P[rr][f] = fmaf(S.om, G[rr][f], P[rr][f]);
                 }
             }
@@ -313,6 +371,7 @@ __device__ __forceinline__ void backward_core(float (&Y)[R][F], float (&B)[R][F]
             for (int f = 0; f < F; ++f) {
                 G[jr][f] = fmaf(selku, t[f], G[jr][f]);
                 P[jr][f] = fmaf(S.om, G[jr][f], P[jr][f]);
+            }
             }
             __builtin_amdgcn_sched_barrier(0);  // keep steps apart: interleaving them only costs registers
         }
