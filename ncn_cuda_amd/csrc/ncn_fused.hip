@@ -11,10 +11,8 @@ namespace ncn {
 
 namespace {
 
-// shapes the multi-stage kernels are built for; tile shapes as in the one-stage table
-// (n_cache = 8 and up is bound by arithmetic even stage by stage: measured 10 % slower through LDS)
-#define NCN_FOR_EACH_FUSED_CONFIG(X) \
-    X(2, 16) X(4, 16) X(2, 32) X(4, 32)
+// the shapes the multi-stage kernels are built for: NCN_FOR_EACH_FUSED_CONFIG (ncn_configs.h), tile shapes as in the
+// one-stage table
 
 // One window per workgroup wherever the problem allows: workgroups that start and end on their own fall out of step
 // with their neighbours on the CU, so that the loads and stores of one run under the stages of the other; a workgroup
@@ -59,7 +57,8 @@ bool fused_supported(const ncn_shape* sh, int activation) {
     (void)activation;  // every activation has a build (tanh its own, without the branch on the code)
     const int64_t ec = sh->E / sh->n_head;
     const uint32_t groups = (uint32_t)(sh->N / sh->n_cache);
-    if ((groups & (groups - 1)) != 0 || groups < 2) return false;
+    // classes are residues modulo a power of two that divides the number of groups: an odd number of groups has none
+    if (groups < 2 || (groups & 1u)) return false;
 #define NCN_MATCH(NC, EC) \
     if (sh->n_cache == NC && ec == EC) return true;
     NCN_FOR_EACH_FUSED_CONFIG(NCN_MATCH)
@@ -75,20 +74,38 @@ std::vector<FusedPass> plan_fused(const ncn_shape* sh, int first, int count, boo
     const size_t state = nc == 2 ? pair_state_bytes(backward) : fused_state_bytes(backward);
     const uint32_t cap_rows = (uint32_t)(state / ((backward ? 4 : 2) * ec * sizeof(float)));
     uint32_t cap = floor_pow2(cap_rows / nc);
-    if (cap > groups) cap = groups;
+    if (cap > groups) cap = floor_pow2(groups);
     if (cap < 4) return passes;
+    const uint32_t groups_pow2 = groups & (~groups + 1u);   // the power of two in the number of groups
     std::vector<uint32_t> s(count);
     for (int k = 0; k < count; ++k) s[k] = stage_stride_of(first + k, groups);
 
-    // backward keeps a dW slot per wave and stage in LDS: 7 stages leave room for two workgroups per CU
-    const int max_stages = backward ? kFusedMaxStages - 1 : kFusedMaxStages;
+    // backward keeps a dW slot per wave and stage in LDS: 7 stages leave room for two workgroups per CU at heads of up
+    // to 32 features; the two-row kernels at wider heads take as many stages as still let two workgroups share a CU
+    int max_stages = backward ? kFusedMaxStages - 1 : kFusedMaxStages;
+    if (backward && nc == 2) {
+        const size_t budget = 80 * 1024, fixed = pair_state_bytes(true) / 2 + (size_t)kFusedMaxStages * 2 * ec * sizeof(float);
+        const size_t per_stage = (size_t)kPairWavesBwd * 2 * ec * sizeof(float);
+        const int fit = fixed < budget ? (int)((budget - fixed) / per_stage) : 0;
+        if (fit >= 2 && fit < max_stages) max_stages = fit;
+    }
     // stages [a, b) as one pass; returns its cost in "full passes over the data" (read + write), or < 0 if impossible
     auto make = [&](int a, int b, FusedPass& p) -> double {
         if (b - a > max_stages || b - a < 2) return -1.0;
+        // S0: the largest power of two that divides every non-zero stride of the pass and the number of groups (with a
+        // power of two of groups the strides are powers of two and this is the smallest of them; with 3 * 2^k groups
+        // and the like the strides past 2^k wrap to odd multiples of 2^k)
         uint32_t s0 = 0;
         for (int k = a; k < b; ++k)
-            if (s[k] && (!s0 || s[k] < s0)) s0 = s[k];
-        if (!s0) s0 = groups / cap;  // only contiguous-block stages: any class structure works, take full windows
+            if (s[k]) {
+                const uint32_t low = s[k] & (~s[k] + 1u);
+                if (!s0 || low < s0) s0 = low;
+            }
+        if (s0 > groups_pow2) s0 = groups_pow2;
+        if (!s0) {  // only contiguous-block stages: any class structure works, take full windows
+            s0 = groups_pow2;
+            while (s0 > 1 && groups / s0 < cap) s0 /= 2;
+        }
         p.first = a;
         p.count = b - a;
         p.single = 0;
@@ -100,13 +117,15 @@ std::vector<FusedPass> plan_fused(const ncn_shape* sh, int first, int count, boo
             p.sub_stride[k - a] = s[k] / s0;
             sum += s[k] / s0;
         }
-        if (p.ring <= cap) {  // closed: cap / ring whole rings of adjacent classes per window
+        if (p.ring <= cap_rows / nc) {  // closed: whole rings of adjacent classes, a power of two of them per window
+            uint32_t rings = floor_pow2((cap_rows / nc) / p.ring);
+            if (rings > s0) rings = s0;
             p.closed = 1;
-            p.window = cap;
+            p.window = rings * p.ring;
             p.halo = 0;
-            p.own = cap;
+            p.own = p.window;
             p.tiles_per_ring = 1;
-            p.class_groups = s0 / (cap / p.ring);
+            p.class_groups = s0 / rings;
             return 2.0;
         }
         p.closed = 0;
@@ -228,6 +247,7 @@ hipError_t launch_fused(Pass pass, FusedArgs& a, const ncn_shape* sh, const Fuse
     a.n_stages = p.count;
     a.class_stride = p.class_stride;
     a.ring = p.ring;
+    a.ring_magic = (p.ring & (p.ring - 1)) == 0 ? 0u : (uint32_t)(((1ull << 32) + p.ring - 1) / p.ring);
     a.window = p.window;
     a.halo = p.halo;
     a.own = p.own;

@@ -77,11 +77,12 @@ struct FusedArgs {
     const int32_t* ctx_len;  // LENGTHS builds: [batch] live slots per batch entry (in the group order of each stage)
     int64_t N, E;
     int32_t n_head, n_stages;
-    int32_t in_dtype, g_dtype, out_dtype, reserved;
+    int32_t in_dtype, g_dtype, out_dtype;
+    uint32_t ring_magic;      // 0 when `ring` is a power of two, else ceil(2^32 / ring): closed passes divide by the ring
     // RADIX builds read: class_stride = n^a in rows, ring = n^k rows per window, window = rows / n_cache,
     // class_groups = workgroup-loads per batch entry, sub_stride[j] = n^j in rows, closed = 1
     uint32_t class_stride;    // S0, in blocks
-    uint32_t ring;            // sub-blocks per class = groups / S0 (power of two)
+    uint32_t ring;            // sub-blocks per class = groups / S0 (a power of two, or an odd number times one)
     uint32_t window;          // sub-blocks held in LDS
     uint32_t halo;            // sub-blocks of halo on each side (0 for a closed pass)
     uint32_t own;             // owned sub-blocks per window (= ring for a closed pass)
@@ -101,6 +102,38 @@ struct FusedItem {
 };
 
 __device__ __forceinline__ uint32_t log2u(uint32_t v) { return 31u - (uint32_t)__clz((int)v); }
+
+// Closed passes hold whole rings side by side in a window: number of the ring that window position q lies in
+// (q < 2^16: a window has at most a few thousand positions, which keeps the multiply-high exact).
+__device__ __forceinline__ uint32_t ring_index(const FusedArgs& A, uint32_t q) {
+    return A.ring_magic == 0u ? q >> log2u(A.ring) : __umulhi(q, A.ring_magic);
+}
+// Window position of the sub-block `add` places after q on q's own ring (closed passes; add < 4 * ring).
+__device__ __forceinline__ uint32_t ring_wrap(const FusedArgs& A, uint32_t q, uint32_t add) {
+    if (A.ring_magic == 0u) return (q & ~(A.ring - 1u)) | ((q + add) & (A.ring - 1u));
+    // rings of 3 * 2^k and the like.  The ring's first position does not change from stage to stage, but it is made
+    // afresh each time (the empty statement hides q from the optimiser): kept in a register across the stages of a
+    // pass it would cost the kernels that run at their register limit a spill.
+    uint32_t qq = q;
+    asm volatile("" : "+v"(qq));
+    const uint32_t base = __umulhi(qq, A.ring_magic) * A.ring;
+    uint32_t t = qq - base + add;
+    t -= __umulhi(t, A.ring_magic) * A.ring;
+    return base + t;
+}
+// (sub-block on the ring, class) of window position qi
+__device__ __forceinline__ void ring_place(const FusedArgs& A, uint32_t sub0, uint32_t cls0, uint32_t qi, uint32_t& sub,
+                                           uint32_t& cls) {
+    if (A.closed) {       // whole rings of adjacent classes, the first sub-block of each first
+        const uint32_t ri = ring_index(A, qi);
+        sub = qi - ri * A.ring;
+        cls = cls0 + ri;
+    } else {              // a stretch of one ring, shorter than the ring: wraps at most once
+        sub = sub0 + qi;
+        if (sub >= A.ring) sub -= A.ring;
+        cls = cls0;
+    }
+}
 
 template <int NC, int EC, bool RADIX>
 __device__ __forceinline__ FusedItem fused_item(const FusedArgs& A, uint32_t item) {
@@ -123,7 +156,8 @@ __device__ __forceinline__ FusedItem fused_item(const FusedArgs& A, uint32_t ite
         it.own_cnt = A.window;
     } else {
         it.cls = cg;
-        it.sub0 = (k * A.own + A.ring - A.halo) & (A.ring - 1u);
+        it.sub0 = k * A.own + A.ring - A.halo;   // k * own < ring
+        if (it.sub0 >= A.ring) it.sub0 -= A.ring;
         it.own_lo = A.halo;
         const uint32_t left = A.ring - k * A.own;
         it.own_cnt = left < A.own ? left : A.own;
@@ -144,8 +178,8 @@ __device__ __forceinline__ int64_t fused_row_offset(const FusedArgs& A, const Fu
         return it.base + pos * A.E;
     }
     const uint32_t qi = lr / NC, o = lr - qi * NC;
-    const uint32_t sub = (it.sub0 + qi) & (A.ring - 1u);
-    const uint32_t cls = A.closed ? it.cls + (qi >> log2u(A.ring)) : it.cls;   // rings are powers of two
+    uint32_t sub, cls;
+    ring_place(A, it.sub0, it.cls, qi, sub, cls);
     const uint32_t blk = sub * A.class_stride + cls;
     return it.base + ((int64_t)blk * NC + o) * A.E;
 }
@@ -171,8 +205,7 @@ __device__ __forceinline__ uint32_t fused_lds_row(const FusedArgs& A, uint32_t q
         const uint32_t wq = qg >> (lg_span - lg_nc), g = qg & (gpw - 1u);
         return fused_lds_place<NC>((wq << lg_span) + ((g >> lg_sj) << (lg_sj + lg_nc)) + (i << lg_sj) + (g & (sstride - 1u)));
     }
-    uint32_t qi = qg + i * sstride;
-    if (A.closed) qi = (qg & ~(A.ring - 1u)) | (qi & (A.ring - 1u));  // wrap inside the group's own ring
+    const uint32_t qi = A.closed ? ring_wrap(A, qg, i * sstride) : qg + i * sstride;  // closed: inside the group's own ring
     return fused_lds_place<NC>(qi * NC + i);
 }
 
@@ -181,8 +214,8 @@ __device__ __forceinline__ uint32_t fused_lds_row(const FusedArgs& A, uint32_t q
 // number * NC + 0 .. NC-1 (ncn_triton/ncn_triton_old.py:66, 93-96).
 template <int NC>
 __device__ __forceinline__ int fused_live_rows(const FusedArgs& A, const FusedItem& it, uint32_t qg, int32_t len) {
-    const uint32_t sub = (it.sub0 + qg) & (A.ring - 1u);
-    const uint32_t cls = A.closed ? it.cls + (qg >> log2u(A.ring)) : it.cls;
+    uint32_t sub, cls;
+    ring_place(A, it.sub0, it.cls, qg, sub, cls);
     const int64_t r = (int64_t)len - (int64_t)(sub * A.class_stride + cls) * NC;
     return (int)max((int64_t)0, min(r, (int64_t)NC));
 }
@@ -370,7 +403,7 @@ __global__ void __launch_bounds__(64 * kFusedWavesFwd) fused_forward_kernel(cons
 }
 
 template <int NC, int EC, int R, int F, bool TANH_ONLY, bool RADIX = false, bool LENGTHS = false>
-__global__ void __launch_bounds__(64 * kFusedWavesBwd, TANH_ONLY ? 4 : 1) fused_backward_kernel(const FusedArgs A) {
+__global__ void __launch_bounds__(64 * kFusedWavesBwd, TANH_ONLY ? (R * F <= 8 ? 4 : 2) : 1) fused_backward_kernel(const FusedArgs A) {
     static_assert(!(RADIX && LENGTHS), "context lengths go with the stride permutation");
     constexpr int NW = kFusedWavesBwd;
     using T = Tile<NC, EC, R, F>;

@@ -8,10 +8,6 @@ namespace ncn {
 
 namespace {
 
-// the shapes of the plain multi-stage passes
-#define NCN_FOR_EACH_FUSED_CONFIG(X) \
-    X(2, 16) X(4, 16) X(2, 32) X(4, 32)
-
 template <int NC, int EC>
 hipError_t launch_t(Pass pass, const FusedArgs& a, int grid, size_t lds, hipStream_t s) {
     constexpr TileShape t = fast_tile(NC, EC);

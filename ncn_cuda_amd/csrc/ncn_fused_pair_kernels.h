@@ -101,9 +101,7 @@ __device__ __forceinline__ void pair_commit_slot1(const uint4 (&raw)[K], int dty
 
 // window position of the sub-block that holds slot 1 of the group whose slot 0 is sub-block q
 __device__ __forceinline__ uint32_t pair_partner(const FusedArgs& A, uint32_t q, uint32_t ss) {
-    uint32_t qi = q + ss;
-    if (A.closed) qi = (q & ~(A.ring - 1u)) | (qi & (A.ring - 1u));   // wrap inside the group's own ring
-    return qi;
+    return A.closed ? ring_wrap(A, q, ss) : q + ss;   // closed: inside the group's own ring
 }
 
 // a lane's F features of an LDS row (or of a weight vector): its H chunks of 4

@@ -11,8 +11,7 @@ namespace ncn {
 namespace {
 
 // shapes with a radix build: digits are extracted with shifts, so n_cache is 2 or 4 (tile shapes of the one-stage table)
-#define NCN_FOR_EACH_RADIX_CONFIG(X) \
-    X(2, 16) X(4, 16) X(2, 32) X(4, 32)
+#define NCN_FOR_EACH_RADIX_CONFIG(X) NCN_FOR_EACH_FUSED_CONFIG(X)
 
 constexpr int kRadixMaxGrid = 4096;
 

@@ -29,6 +29,15 @@ CASES = [
     (2, 256, 64, 2, 2, 1000003, 3),  # a very high first stage: 2^(stage-1) mod groups is 0 from stage log2(groups)+1 on
     (3, 2048, 64, 4, 2, 0, 10),    # n = 2, head width 16 (16 groups per wave tile, windows of 512 groups)
     (2, 16, 32, 1, 2, 0, 3),       # n = 2, 8 groups: a window smaller than one wave tile per wave
+    (3, 2048, 16, 2, 2, 0, 10),    # n = 2, head width 8 (one lane per group, 64 groups per wave tile)
+    (2, 2048, 128, 2, 2, 0, 11),   # n = 2, head width 64 (windows of 64 groups, backward passes of 3 stages)
+    (2, 1024, 32, 4, 4, 0, 6),     # n = 4, head width 8
+    (2, 512, 128, 2, 4, 0, 6),     # n = 4, head width 64 (windows of 16 groups)
+    (2, 3 * 512, 64, 2, 2, 0, 12),   # 768 groups = 3 * 2^8: strides wrap to 256 and 512 in turn, closed passes on rings of 3, 6, ..
+    (2, 96, 32, 4, 4, 0, 6),         # n = 4, 24 groups = 3 * 8
+    (1, 3 * 4096, 128, 4, 2, 0, 13), # 6144 groups: halo passes on a ring that is no power of two, then closed ones
+    (2, 5 * 256, 64, 2, 2, 0, 9),    # 640 groups = 5 * 2^7
+    (2, 7 * 64, 32, 2, 4, 2, 5),     # n = 4, 112 groups = 7 * 16, from stage 2
 ]
 
 
@@ -46,6 +55,13 @@ def test_multi_stage_matches_single_stage_and_oracle(M, case):
     for l in range(L):
         cx, cxa = M.forward(cx, cxa, gWs[l], alpha, 0, n, C, first + l)
         outs.append((cx, cxa))
+    # groups of 2 and 4 rows at heads of 8 to 64 features, an even number of groups: the call really uses LDS passes
+    if n in (2, 4) and E // C in (8, 16, 32, 64) and (N // n) % 2 == 0:
+        import ctypes
+        from ncn_cuda_amd import _lib
+        shape = _lib.NcnShape(batch, N, E, C, n)
+        for backward in (0, 1):
+            assert _lib.load().ncn_plan_passes(ctypes.byref(shape), first, L, 0, backward, None, 0) >= 1
     # one call for all stages
     y, ya = M.forward_stages(gx, gxa, Wst, alpha, 0, n, C, first, L)
     # same arithmetic up to where the powers of m are folded in (per stage vs per pass): rounding-level agreement
@@ -182,8 +198,8 @@ def _stage_by_stage_dW(M, outs, gdy, gdya, gWs, alpha, act, n, C, first):
 
 
 @pytest.mark.parametrize("case", [
-    (2, 256, 16, 2, 2, 0, 11),      # more stages in one call than one reduction job holds (8): two jobs
-                                    # (heads of 8 features: no LDS passes, one launch per stage)
+    (2, 256, 8, 2, 2, 0, 11),       # more stages in one call than one reduction job holds (8): two jobs
+                                    # (heads of 4 features: no LDS passes, one launch per stage)
     (8192, 64, 128, 4, 16, 0, 2),   # 16384 partial rows per stage: the buffer holds one stage, a job per stage
     (640, 256, 128, 4, 8, 1, 3),    # 5120 rows per stage: three stages side by side (15360 rows), one job
 ], ids=lambda c: "b%d_N%d_E%d_C%d_n%d_s%d_L%d" % c)

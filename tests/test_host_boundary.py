@@ -108,7 +108,11 @@ def test_entry_points_reject_bad_arguments_before_touching_the_gpu(lib):
     args = [p, p, 0, p, p, 0, p, p, 0, z, z, p, p]
     assert h.ncn_backward(*args, z, ctypes.c_size_t(0), ctypes.byref(sh), 0, 1, 0.9, 0.9, 0, z) == -5
     assert h.ncn_backward(*args, p, ctypes.c_size_t(ws - 1), ctypes.byref(sh), 0, 1, 0.9, 0.9, 0, z) == -5
-    assert h.ncn_backward(*args, p, ctypes.c_size_t(ws), ctypes.byref(sh), 0, 2, 0.9, 0.9, 0, z) == -8  # needs x_rec
+    # two stages without x_rec, xa_rec and without room in the workspace for the state between them (groups of 8 rows:
+    # one launch per stage; shapes with multi-stage passes may run two stages as one closed pass, which carries nothing)
+    sh8 = _shape(lib, 2, 64, 32, 4, 8)
+    ws8 = h.ncn_workspace_bytes(ctypes.byref(sh8))
+    assert h.ncn_backward(*args, p, ctypes.c_size_t(ws8), ctypes.byref(sh8), 0, 2, 0.9, 0.9, 0, z) == -8  # needs x_rec
 
 
 def test_indexed_entry_points_reject_bad_arguments_before_touching_the_gpu(lib):
@@ -286,7 +290,11 @@ def _passes(lib, shape, first, count, backward):
 
 @pytest.mark.parametrize("backward", [False, True])
 @pytest.mark.parametrize("dims", [(128, 8192, 128, 4, 2, 0, 13), (32, 1024, 128, 4, 4, 0, 5), (3, 1024, 64, 2, 2, 0, 11),
-                                  (2, 2048, 64, 2, 2, 3, 6), (5, 64, 128, 4, 4, 0, 3), (1, 1 << 16, 32, 1, 2, 0, 20)])
+                                  (2, 2048, 64, 2, 2, 3, 6), (5, 64, 128, 4, 4, 0, 3), (1, 1 << 16, 32, 1, 2, 0, 20),
+                                  (3, 2048, 16, 2, 2, 0, 10), (2, 2048, 128, 2, 2, 0, 11), (2, 1024, 32, 4, 4, 0, 6),
+                                  (2, 512, 128, 2, 4, 0, 6),                      # heads of 8 and of 64 features
+                                  (2, 3 * 512, 64, 2, 2, 0, 12), (2, 96, 32, 4, 4, 0, 6), (2, 3 * 4096, 128, 4, 2, 0, 14),
+                                  (2, 5 * 256, 64, 2, 2, 0, 9), (2, 7 * 64, 32, 2, 4, 2, 5)])  # 3, 5, 7 times a power of two
 def test_multi_stage_plan_invariants(lib, dims, backward):
     """The pass planner (host logic): passes tile the stage range in order; a halo window owns what its halo leaves,
     and the halo is (n_cache - 1) * sum of the pass's strides in sub-blocks; closed passes own their whole window."""
@@ -299,22 +307,24 @@ def test_multi_stage_plan_invariants(lib, dims, backward):
     for (p_first, p_count, kind, s0, window, halo, own, cgroups) in passes:
         assert p_first == nxt and p_count >= 1
         nxt += p_count
-        strides = [(0 if (first + p_first + k) == 0 else (1 << (first + p_first + k - 1)) % groups) for k in range(p_count)]
+        strides = [(0 if (first + p_first + k) == 0 else pow(2, first + p_first + k - 1, groups)) for k in range(p_count)]
         if kind == 0:
             assert p_count == 1
             continue
         assert p_count >= 2 and p_count <= 8
-        assert window & (window - 1) == 0 and window <= groups
+        assert window <= groups
         nz = [s for s in strides if s]
-        assert all(s % s0 == 0 for s in nz)
+        assert s0 & (s0 - 1) == 0 and groups % s0 == 0 and all(s % s0 == 0 for s in nz)   # classes: residues modulo S0
         ring = groups // s0
         # rows a workgroup keeps in LDS: groups of two rows leave their slot-0 rows in registers
         lds_bytes = window * (1 if n == 2 else n) * (E // C) * 4 * (4 if backward else 2)
         assert lds_bytes <= 64 * 1024
         if kind == 2:
-            assert ring <= window and halo == 0 and own == window and cgroups * (window // ring) == s0
+            assert window % ring == 0 and halo == 0 and own == window and cgroups * (window // ring) == s0
+            rings = window // ring
+            assert rings & (rings - 1) == 0                       # whole rings, a power of two of them
         else:
-            assert ring > window and cgroups == s0
+            assert ring > window and cgroups == s0 and window & (window - 1) == 0
             assert halo == (n - 1) * sum(s // s0 for s in strides)
             assert own == window - 2 * halo and 4 * own >= 3 * window
     assert nxt == count
@@ -322,7 +332,8 @@ def test_multi_stage_plan_invariants(lib, dims, backward):
 
 def test_multi_stage_plan_declines_ineligible_shapes(lib):
     assert _passes(lib, _shape(lib, 128, 4096, 128, 4, 16), 0, 3, False) == []   # n_cache = 16: arithmetic-bound
-    assert _passes(lib, _shape(lib, 2, 96, 32, 4, 4), 0, 3, False) == []         # 24 groups: not a power of two
+    assert _passes(lib, _shape(lib, 2, 60, 32, 4, 4), 0, 3, False) == []         # 15 groups: no power of two divides them
+    assert _passes(lib, _shape(lib, 2, 96, 32, 4, 4), 0, 3, False) != []         # 24 groups = 3 * 8: classes modulo 2, 4, 8
     assert _passes(lib, _shape(lib, 2, 1024, 128, 4, 2), 0, 1, False) == []      # a single stage
     # the deep configuration: three passes forward, four at most backward, closed rings last
     fwd = _passes(lib, _shape(lib, 128, 8192, 128, 4, 2), 0, 13, False)
