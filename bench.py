@@ -4,6 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg3|cfg2|cfg4|cfg5] [--no-cpu]
                     [--grouping closed|stride-table|radix-table|ragged|radix] [--save-every K] [--scalar-heads]
                     [--no-surface]
+    python bench.py --record-traffic <dir>      (turns rocprofv3 counter files into profiles/traffic.json, see there)
 
 One step = forward of all L stages (each stage saving its outputs, like the reference's autograd
 node) + reversible backward of all L stages producing dx, dxa and every dW_l, on inputs that are
@@ -71,7 +72,81 @@ def measured_traffic(config, grouping, version):
     return entry.get("bytes")
 
 
+def record_traffic(prof_dir):
+    """Turns the counter files of two rocprofv3 runs of this script into the entry of profiles/traffic.json that
+    `roofline.traffic` is read from.  prof_dir holds f/ and w/ (the output directories of
+        rocprofv3 --pmc FETCH_SIZE --output-format csv -d <prof_dir>/f -o p -- python3 bench.py --config C --steps 2
+                  --warmup 1 --no-cpu --no-surface --copy-probe > <prof_dir>/f.log
+    and the same with WRITE_SIZE and w) and the two logs.  Each counter is scaled by what it reads for the 1 GiB copy
+    of --copy-probe (1048576 KiB read and written).  The library version, build id and workload of the entry are those
+    the profiled runs printed, so an entry can only claim what was measured."""
+    import csv
+    import glob
+
+    runs = {}
+    for d in ("f", "w"):
+        with open(os.path.join(prof_dir, d + ".log")) as fh:
+            lines = [l for l in fh if l.startswith("{")]
+        runs[d] = json.loads(lines[-1])
+    meta = runs["f"]
+    for key in ("ncn_version", "build_id", "kernel"):
+        if runs["w"]["roofline"][key] != meta["roofline"][key]:
+            raise SystemExit(f"the two runs disagree on {key}")
+    workload = meta["config"]["workload"]
+    config = workload.split(":")[0]
+    grouping = workload.rsplit("grouping ", 1)[1]
+    steps = meta["steps"] + meta["warmup"]
+    per_call = "backward call" in meta["roofline"]["kernel"]
+    sizes, factors, names = {}, {}, {}
+    for d, counter in (("f", "FETCH_SIZE"), ("w", "WRITE_SIZE")):
+        rows = []
+        for f in glob.glob(os.path.join(prof_dir, d, "**", "*counter_collection.csv"), recursive=True):
+            with open(f) as fh:
+                rows += [r for r in csv.DictReader(fh) if r["Counter_Name"] == counter]
+        copy = max(float(r["Counter_Value"]) for r in rows if "copyBuffer" in r["Kernel_Name"])
+        factors[d] = 1048576.0 / copy
+        per_dispatch = {}
+        for r in rows:   # one row per dispatch and XCD set: sum what belongs to one dispatch
+            if "ncn::" in r["Kernel_Name"]:
+                k = (r["Kernel_Name"], r["Dispatch_Id"])
+                per_dispatch[k] = per_dispatch.get(k, 0.0) + float(r["Counter_Value"])
+        if per_call:    # every backward-side launch of a call (passes, one-stage launches, dW reduction), per call
+            mine = {k: v for k, v in per_dispatch.items() if "backward" in k[0] or "reduce_" in k[0]}
+            n_calls = steps * meta["config"]["backward_calls_per_step"]
+            sizes[d] = sum(mine.values()) / n_calls * factors[d] * 1024.0
+            counts = {}
+            for (name, _), _v in mine.items():
+                counts[name] = counts.get(name, 0) + 1
+            short = lambda n: n.replace("(anonymous namespace)::", "").split("(")[0].replace("void ", "")
+            names[d] = ", ".join(f"{c / n_calls:g} x {short(n)}" for n, c in sorted(counts.items()))
+        else:           # the one-stage backward kernel, per launch
+            mine = [v for k, v in per_dispatch.items() if "stage_backward_kernel" in k[0]]
+            sizes[d] = sum(mine) / len(mine) * factors[d] * 1024.0
+            names[d] = sorted({k[0] for k in per_dispatch if "stage_backward_kernel" in k[0]})[0].split("(")[0].replace("void ", "")
+    try:
+        with open(TRAFFIC_FILE) as fh:
+            rec = json.load(fh)
+    except (OSError, ValueError):
+        rec = {"entries": {}}
+    rec["comment"] = ("HBM bytes per launch (or per backward call over a segment) of the dominant kernel of bench.py, from "
+                      "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, written by `python bench.py --record-traffic <dir>` from the "
+                      "counter files and logs of the profiled runs; bench.py reports an entry only for the library version "
+                      "it was measured on")
+    rec["entries"][f"{config}/{grouping}"] = {
+        "ncn_version": meta["roofline"]["ncn_version"], "build_id": meta["roofline"]["build_id"],
+        "kernel": names["f"], "bytes": round(sizes["f"] + sizes["w"]), "read_bytes": round(sizes["f"]),
+        "written_bytes": round(sizes["w"]), "fetch_size_factor": round(factors["f"], 4),
+        "write_size_factor": round(factors["w"], 4), "workload": workload}
+    with open(TRAFFIC_FILE, "w") as fh:
+        json.dump(rec, fh, indent=1)
+        fh.write("\n")
+    print(json.dumps(rec["entries"][f"{config}/{grouping}"]))
+
+
 def main():
+    if len(sys.argv) == 3 and sys.argv[1] == "--record-traffic":
+        record_traffic(sys.argv[2])
+        return
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
@@ -170,8 +245,8 @@ def main():
                 saved.append((sy, sya))
             elif bf16 and cnt == 1:
                 # bf16 outputs plus what their rounding took away (a second bf16 plane): what the backward inverts
-                cx, cxa, ys, yas = M.forward_stages(cx, cxa, Wst[a], alpha, 0, n, C, a, 1, save_residual=True,
-                                                    ctx_len=lens)
+                # (float32 copies instead where only the generic kernels take the shape: --scalar-heads)
+                cx, cxa, ys, yas = M.forward_stages_saving(cx, cxa, Wst[a], alpha, 0, n, C, a, ctx_len=lens)
                 saved.append((ys, yas))
             else:
                 cx, cxa = M.forward_stages(cx, cxa, Wst[a:a + cnt], alpha, 0, n, C, a, cnt, out_dtype=torch.float32,
@@ -237,22 +312,10 @@ def main():
     del src, dst
 
     # what this GPU sustains on plain float32 FMAs (no packed instructions, as the library is built): a stream of
-    # independent v_fma_f32, 8 waves per SIMD, timed here with events on the launch stream
+    # independent v_fma_f32, 8 waves per SIMD, timed with events on the launch stream
+    from ncn_cuda_amd import probe
     lib = M._lib.load()
-    cus = torch.cuda.get_device_properties(dev).multi_processor_count
-    fma_blocks, fma_iters = 8 * cus, 2048
-    probe_out = torch.empty(fma_blocks * 256, dtype=torch.float32, device=dev)
-    stream_ptr = torch.cuda.current_stream(dev).cuda_stream
-    M._lib.check(lib.ncn_probe_fma_stream(probe_out.data_ptr(), fma_blocks, fma_iters, stream_ptr), "ncn_probe_fma_stream")
-    f0, f1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    f0.record()
-    for _ in range(3):
-        M._lib.check(lib.ncn_probe_fma_stream(probe_out.data_ptr(), fma_blocks, fma_iters, stream_ptr), "ncn_probe_fma_stream")
-    f1.record()
-    torch.cuda.synchronize()
-    fma_flops = 2.0 * lib.ncn_probe_fma_per_thread(fma_iters) * fma_blocks * 256
-    attainable_valu = 3 * fma_flops / (f0.elapsed_time(f1) * 1e-3) / 1e12
-    del probe_out
+    attainable_valu = probe.fma_stream_tflops(device=dev)
 
     # The same workload through the autograd surface the reference times (NCNNetTestCuda(...)(x, xa); yi.backward(dyi),
     # grad_test_bench.py:116-134: one node per stage) and through the one-node form of the stack; then the timed step
@@ -377,7 +440,7 @@ def main():
             "attainable_valu_TFLOPs": attainable_valu, "valu_frac_of_attainable": valu_achieved / attainable_valu,
             "hbm_achieved_GBps": hbm_achieved, "hbm_frac": hbm_achieved / HBM_PEAK_GBS,
             "attainable_copy_GBps": copy_gbps, "hbm_frac_of_attainable_copy": hbm_achieved / copy_gbps,
-            "ncn_version": version}
+            "ncn_version": version, "build_id": lib.ncn_build_id().decode()}
     result = {
         "metric": f"NCN fwd+bwd tokens/sec and achieved HBM GB/s (% roofline), B={tokens} D={N} g={n}",
         "value": value,
@@ -394,7 +457,8 @@ def main():
         "config": {"workload": f"{args.config}: B={tokens} D={N} g={n} -> x[batch={batch},N={N},E={E}], "
                                f"{C} heads of {E // C}, n_cache={n}, {L} stages, alpha=0.9, m=0.9, tanh, "
                                f"{cfg['dtype']} storage, outputs saved every {save_every} stage(s), "
-                               f"grouping {args.grouping}", "positions_per_s": batch * N / (ms_per_step * 1e-3)},
+                               f"grouping {args.grouping}", "positions_per_s": batch * N / (ms_per_step * 1e-3),
+                   "backward_calls_per_step": len(segs)},
         "roofline": roof,
         "stack": {"median_ms_per_step": median_step_ms,
                   "min_ms_per_step": per_step_ms[0], "max_ms_per_step": per_step_ms[-1],

@@ -16,7 +16,7 @@ EXPORTS = ("ncn_forward", "ncn_backward", "ncn_inverse", "ncn_forward_indexed", 
            "ncn_inverse_indexed", "ncn_inverse_ws", "ncn_forward_radix", "ncn_backward_radix", "ncn_inverse_radix", "ncn_plan_radix", "ncn_workspace_bytes", "ncn_workspace_bytes_stages",
            "ncn_plan_passes", "ncn_kernel_path",
            "ncn_check_shape", "ncn_error_string", "ncn_version", "ncn_backward_static", "ncn_static_scratch_bytes", "ncn_kernel_path_scalars",
-           "ncn_build_id", "ncn_probe_fma_stream", "ncn_probe_fma_per_thread")
+           "ncn_build_id", "ncn_probe_issue", "ncn_probe_issue_info")
 
 
 class NcnShape(ctypes.Structure):
@@ -112,10 +112,10 @@ def load():
     lib.ncn_version.argtypes = []
     lib.ncn_build_id.restype = ctypes.c_char_p
     lib.ncn_build_id.argtypes = []
-    lib.ncn_probe_fma_stream.restype = i
-    lib.ncn_probe_fma_stream.argtypes = [vp, i, i, vp]
-    lib.ncn_probe_fma_per_thread.restype = i
-    lib.ncn_probe_fma_per_thread.argtypes = [i]
+    lib.ncn_probe_issue.restype = i
+    lib.ncn_probe_issue.argtypes = [i, i, i, i, vp, vp]
+    lib.ncn_probe_issue_info.restype = i
+    lib.ncn_probe_issue_info.argtypes = [i, ctypes.POINTER(i), ctypes.POINTER(i)]
     _lib = lib
     return lib
 

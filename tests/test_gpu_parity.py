@@ -336,3 +336,14 @@ def test_backward_with_more_tiles_than_waves_loops_and_agrees_with_smaller_calls
     for k in range(4):
         assert O.rel_err(whole[k], torch.cat([parts[0][k], parts[1][k]])) < 1e-6
     assert O.rel_err(whole[4], parts[0][4] + parts[1][4]) < 1e-6
+
+
+def test_issue_rate_probe_runs(M):
+    """The measurement aid behind bench.py's attainable_valu_TFLOPs: a stream of plain v_fma_f32 lands between half and
+    all of the 78.6 TFLOP/s that 16 lanes per SIMD and clock give, and a stream of v_exp_f32 issues at about half the
+    rate of the FMAs (one operation each where an FMA counts two)."""
+    from ncn_cuda_amd import probe
+    fma = probe.fma_stream_tflops(iters=512)
+    assert 40.0 < fma < 82.0
+    ms, instr, flops = probe.time_launch(3, 8, 8, 256)
+    assert 0.35 * fma / 2 < flops / (ms * 1e-3) / 1e12 < 0.65 * fma / 2

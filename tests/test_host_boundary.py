@@ -430,3 +430,17 @@ def test_python_validation_rejects_scalars_no_kernel_takes(lib):
     M.validate(torch.zeros(1, 16, 64), torch.zeros(1, 16, 64), torch.zeros(128), 4, 2, 0, alpha=1e-5)   # generic
     with pytest.raises(ValueError, match="generic kernels"):
         M.validate(x, x, W, 4, 2, 0, alpha=1e-5, m=0.9)
+
+
+def test_probe_entry_points_validate_their_arguments(lib):
+    """The measurement aid: modes are described without a GPU, bad arguments are refused before any launch."""
+    h = lib.load()
+    valu, flops = ctypes.c_int(0), ctypes.c_int(0)
+    assert h.ncn_probe_issue_info(0, ctypes.byref(valu), ctypes.byref(flops)) == 8 and (valu.value, flops.value) == (1, 2)
+    assert h.ncn_probe_issue_info(8, ctypes.byref(valu), ctypes.byref(flops)) == 8 and (valu.value, flops.value) == (20, 28)
+    assert h.ncn_probe_issue_info(99, None, None) == -2
+    p = ctypes.c_void_p(4096)
+    assert h.ncn_probe_issue(0, 8, 8, 16, None, None) == -1
+    assert h.ncn_probe_issue(99, 8, 8, 16, p, None) == -2
+    assert h.ncn_probe_issue(0, 3, 8, 16, p, None) == -2      # chains: 1, 4 or 8
+    assert h.ncn_probe_issue(0, 8, 3, 16, p, None) == -2      # waves per SIMD: 1, 2, 4 or 8
