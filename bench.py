@@ -425,14 +425,18 @@ def main():
     # limited by their HBM round trips
     valu_bound = n >= 8
     version = lib.ncn_version().decode()
-    kernel = (f"stage_backward_kernel<{n},{E // C}>" + (" (indexed build)" if tables else "") if not lds_passes else
+    import ctypes
+    on_register_kernels = lib.ncn_kernel_path(ctypes.byref(M._lib.NcnShape(batch, N, E, C, n))) == 2
+    kernel = ((f"stage_backward_kernel<{n},{E // C}>" if on_register_kernels else
+               f"generic_backward_kernel (n_cache {n}, heads of {E // C}: no register-tile build)") +
+              (" (indexed build)" if tables else "") if not lds_passes else
               f"backward call over a segment of up to {save_every} stages (multi-stage passes)")
     roof = {"bound": "fp32_valu" if valu_bound else "hbm",
             "achieved": valu_achieved if valu_bound else hbm_achieved,
             "peak": VALU_PEAK_TFLOPS if valu_bound else HBM_PEAK_GBS,
             "unit": "TFLOP/s" if valu_bound else "GB/s",
             "frac": (valu_achieved / VALU_PEAK_TFLOPS) if valu_bound else (hbm_achieved / HBM_PEAK_GBS),
-            "traffic": measured_traffic(args.config, args.grouping, version),
+            "traffic": None if args.scalar_heads else measured_traffic(args.config, args.grouping, version),
             "kernel": kernel, "avg_launch_ms": bwd_ms,
             "algorithmic_flops_per_launch": flops_bwd_unit,
             "algorithmic_bytes_per_launch": bytes_bwd_launch,
