@@ -36,11 +36,14 @@ def test_net_test_cuda_like_reference_script(pkg):
     assert O.rel_err(yi, ref_yi) < 1e-5
     assert O.rel_err(ya, ref_ya) < 1e-5
     # n_cache = 32 amplifies inversion rounding by (1/0.9)^32 = 29: the reference's own check uses atol=1e-2
-    # (grad_test_bench.py:161); float32 still lands near 1e-5 relative
-    assert O.rel_err(gx.grad, ref_dx) < 5e-5
-    assert O.rel_err(gxa.grad, ref_dxa) < 5e-5
+    # (grad_test_bench.py:161); float32 still lands near 1e-5 relative (measured: dx 4.1e-6, worst dW 1.5e-5)
+    from conftest import record_errors
+    record_errors("reference_script_shape", n=n, amp=(1 / 0.9) ** n, dx=O.rel_err(gx.grad, ref_dx),
+                  dxa=O.rel_err(gxa.grad, ref_dxa), dW=max(O.rel_err(gWs[l].grad, ref_dWs[l]) for l in range(L)))
+    assert O.rel_err(gx.grad, ref_dx) < 3e-5
+    assert O.rel_err(gxa.grad, ref_dxa) < 3e-5
     for l in range(L):
-        assert O.rel_err(gWs[l].grad, ref_dWs[l]) < 5e-5
+        assert O.rel_err(gWs[l].grad, ref_dWs[l]) < 3e-5
 
 
 def test_net_cuda_module_list_and_state_dict(pkg):

@@ -99,11 +99,15 @@ def test_forward_backward_inverse_vs_oracle(M, shape):
     assert O.rel_err(outs[-1][1], ref_ya) < TOL_F32
     # the reversible backward divides by m at each of the n steps of a stage: float32 rounding grows like
     # (1/m)^n (5x at n = 16, 29x at n = 32, 850x at n = 64), which only matters above n = 16
-    # (n <= 16, the group sizes of the benchmark configurations, are held to 1e-5; every step rounds about 1e-7
-    # relative, which the steps that follow amplify: 5e-6 per unit of amplification covers n = 32 and 64)
-    tol_inv = max(TOL_F32, 5e-6 * (1 / 0.9) ** n)
-    tol_bwd = TOL_F32 if n <= 16 else tol_inv
+    # (groups of up to 32 rows are held to 1e-5 on the gradients: measured 9.0e-6 at n = 32 on these shapes; at
+    # n = 64 the worst gradient is 1.7e-6 per unit of amplification, the inverse 2.8e-6 at n = 32)
+    tol_inv = max(TOL_F32, 4e-6 * (1 / 0.9) ** n)
+    tol_bwd = TOL_F32 if n <= 32 else 3e-6 * (1 / 0.9) ** n
     xr, xar, dx, dxa, dWs = _stack_backward(M, outs, gdyi, gdya, gWs, alpha, n, C)
+    if n >= 32:
+        from conftest import record_errors
+        record_errors("parity_shapes", n=n, amp=(1 / 0.9) ** n, dx=O.rel_err(dx, ref_dx), dxa=O.rel_err(dxa, ref_dxa),
+                      dW=max(O.rel_err(dWs[l], ref_dWs[l]) for l in range(L)))
     assert O.rel_err(dx, ref_dx) < tol_bwd
     assert O.rel_err(dxa, ref_dxa) < tol_bwd
     for l in range(L):
@@ -113,6 +117,9 @@ def test_forward_backward_inverse_vs_oracle(M, shape):
     ix, ixa = M.inverse(outs[-1][0], outs[-1][1], gWs[-1], alpha, 0, n, C, L - 1)
     # (at n = 64 the step Jacobians add to that: the round trip only keeps about two digits)
     tol_rt = tol_inv if n <= 32 else 1e-1
+    if n >= 32:
+        from conftest import record_errors
+        record_errors("parity_inverse", n=n, amp=(1 / 0.9) ** n, x=O.rel_err(ix, prev[0]), xa=O.rel_err(ixa, prev[1]))
     assert O.rel_err(ix, prev[0]) < tol_rt
     assert O.rel_err(ixa, prev[1]) < tol_rt
 

@@ -60,11 +60,14 @@ def test_random_problem(M, case):
     W = torch.stack(Ws).cuda()
     amp_stage = (1 / 0.9) ** n
     # float32 rounding of the inversion grows like (1/m)^n per stage: 5x at n = 16, 29x at n = 32, 850x at n = 64
-    # (where the reference's own check uses atol = 1e-2, grad_test_bench.py:161)
-    # (n <= 16, the group sizes of the benchmark configurations, are held to 1e-5 whatever the amplification; above,
-    # the sign-regime inputs of relu / leaky relu reach 9e-6 per unit of amplification at n = 64)
-    gtol = (2e-5 if n >= 64 else 1e-5) * amp_stage if n >= 32 else 1e-5
-    rtol = max(3e-5, 1e-5 * amp_stage) if n < 64 else 2e-1
+    # (where the reference's own check uses atol = 1e-2, grad_test_bench.py:161).  n <= 16, the group sizes of the
+    # benchmark configurations, are held to 1e-5 whatever the amplification.  Above, the bounds are a margin over the
+    # worst case measured on these 96 shapes, per unit of amplification: gradients 5.0e-7 at n = 32 (dW; dx, dxa
+    # 2.0e-7), 6.6e-6 at n = 64 (1.4e-5 on the sign-regime inputs of relu / leaky relu); reconstructed inputs 3.9e-6
+    # at n = 32, and 0.057 absolute at n = 64 (0.13 on the sign-regime inputs).
+    signed = act in (1, 3)
+    gtol = 1e-5 if n < 32 else max(1e-5, 1e-6 * amp_stage) if n < 64 else (2e-5 if signed else 1e-5) * amp_stage
+    rtol = max(3e-5, 6e-6 * amp_stage) if n < 64 else (2e-1 if signed else 1e-1)
     # one call per stage, every stage saving its outputs
     outs, cx, cxa = [], gx, gxa
     for l in range(L):
@@ -72,11 +75,18 @@ def test_random_problem(M, case):
         outs.append((cx, cxa))
     assert O.rel_err(cx, ref[0]) < 1e-5 and O.rel_err(cxa, ref[1]) < 1e-5
     g, h = gdy, gdya
+    worst_dw = worst_rec = 0.0
     for l in range(L - 1, -1, -1):
         xr, xar, g, h, dW = M.backward_stages(outs[l][0], outs[l][1], g, h, W[l], alpha, act, n, C, first + l, 1)
-        assert O.rel_err(dW[0], ref[4][l]) < gtol, f"dW{l}"
         prev = outs[l - 1] if l else (gx, gxa)
+        worst_dw = max(worst_dw, O.rel_err(dW[0], ref[4][l]))
+        worst_rec = max(worst_rec, O.rel_err(xr, prev[0]), O.rel_err(xar, prev[1]))
+        assert O.rel_err(dW[0], ref[4][l]) < gtol, f"dW{l}"
         assert O.rel_err(xr, prev[0]) < rtol and O.rel_err(xar, prev[1]) < rtol
+    if n >= 32:
+        from conftest import record_errors
+        record_errors("random_problem", n=n, act=act, amp=amp_stage, dW=worst_dw, rec=worst_rec,
+                      dx=O.rel_err(g, ref[2]), dxa=O.rel_err(h, ref[3]))
     assert O.rel_err(g, ref[2]) < gtol and O.rel_err(h, ref[3]) < gtol
     # the same stages in one call (multi-stage passes where the shape allows), forward only compared tightly
     y, ya = M.forward_stages(gx, gxa, W, alpha, act, n, C, first, L)
