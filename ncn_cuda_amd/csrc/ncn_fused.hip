@@ -89,7 +89,24 @@ std::vector<FusedPass> plan_fused(const ncn_shape* sh, int first, int count, boo
         const int fit = fixed < budget ? (int)((budget - fixed) / per_stage) : 0;
         if (fit >= 2 && fit < max_stages) max_stages = fit;
     }
-    // stages [a, b) as one pass; returns its cost in "full passes over the data" (read + write), or < 0 if impossible
+    // What a pass costs, in the time one array of the activations' size takes to cross HBM at copy speed.  Traffic: the
+    // pass reads `arrays_in` arrays of its windows (window / own times the data) and writes `arrays_out` arrays of its
+    // owned rows; in the backward the pass that holds the call's first stage runs last and writes the two gradients
+    // only (callers that want the reconstructed inputs pay two arrays more than priced here).  Issue: every stage costs
+    // `per_stage` such units of instruction issue on all groups of its windows (measured per kernel family on
+    // x[128, 8192, 128]: a two-row backward stage 0.143 ms against 0.102 ms per array, a two-row forward stage 0.078 ms;
+    // the four-row kernels in proportion to their instruction counts).  The two overlap, better the more they differ:
+    // the cube root of the sum of cubes follows the measured pass times to 5 % (a closed backward pass, whose windows
+    // are the most scattered in memory, takes 1.1 times that).
+    const double arrays_in = backward ? 4.0 : 2.0;
+    const double per_stage = nc == 2 ? (backward ? 1.4 : 0.76) : (backward ? 3.6 : 2.0);
+    auto priced = [&](int a, double redundancy, int stages, bool closed) -> double {
+        const double arrays_out = backward ? (a == 0 ? 2.0 : 4.0) : 2.0;
+        const double traffic = arrays_in * redundancy + arrays_out;
+        const double issue = per_stage * stages * redundancy;
+        return std::cbrt(traffic * traffic * traffic + issue * issue * issue) * (closed && backward ? 1.1 : 1.0);
+    };
+    // stages [a, b) as one pass; returns its cost (see above), or < 0 if impossible
     auto make = [&](int a, int b, FusedPass& p) -> double {
         if (b - a > max_stages || b - a < 2) return -1.0;
         // S0: the largest power of two that divides every non-zero stride of the pass and the number of groups (with a
@@ -126,7 +143,7 @@ std::vector<FusedPass> plan_fused(const ncn_shape* sh, int first, int count, boo
             p.own = p.window;
             p.tiles_per_ring = 1;
             p.class_groups = s0 / rings;
-            return 2.0;
+            return priced(a, 1.0, b - a, true);
         }
         p.closed = 0;
         p.window = cap;
@@ -136,17 +153,18 @@ std::vector<FusedPass> plan_fused(const ncn_shape* sh, int first, int count, boo
         if (p.own * 4 < cap * 3) return -1.0;  // more than a third of the window would be redundant work
         p.tiles_per_ring = (p.ring + p.own - 1) / p.own;
         p.class_groups = s0;
-        return 1.0 + (double)cap / p.own;
+        return priced(a, (double)cap / p.own, b - a, false);
     };
 
-    // cheapest cut of the range into passes (a one-stage launch costs one read + one write = 2)
+    // cheapest cut of the range into passes (a one-stage launch is bound by its traffic: every array once)
     std::vector<double> best(count + 1, 1e30);
     std::vector<int> from(count + 1, -1);
     std::vector<FusedPass> how(count + 1);
     best[0] = 0.0;
     for (int b = 1; b <= count; ++b) {
-        if (best[b - 1] + 2.0 < best[b]) {
-            best[b] = best[b - 1] + 2.0;
+        const double single = arrays_in + (backward ? (b == 1 ? 2.0 : 4.0) : 2.0);
+        if (best[b - 1] + single < best[b]) {
+            best[b] = best[b - 1] + single;
             from[b] = b - 1;
             FusedPass p{};
             p.first = b - 1;

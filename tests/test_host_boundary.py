@@ -76,9 +76,9 @@ def test_kernel_path_and_workspace(lib):
     P4 = 128 * 8192 * 128 * 4
     assert h.ncn_workspace_bytes_stages(ctypes.byref(deep), 0, 13, 0, 0) == 2 * P4
     # backward: the four arrays and a dW partial row per window and stage of every pass (stages 6-12 in 4096 closed
-    # windows per head, stages 0-3 in 128 x 36 halo windows that own 114 of their 128 groups, stages 4-5 in 128 x 8 x 5
+    # windows per head, stages 3-5 in 128 x 4 x 9 halo windows that own 114 of their 128 groups, stages 0-2 in 128 x 34
     # that own 122), plus their chunk sums (one row per 32, + 8)
-    rows = 7 * 4096 + 4 * 4608 + 2 * 5120
+    rows = 7 * 4096 + 3 * 4608 + 3 * 4352
     assert h.ncn_workspace_bytes_stages(ctypes.byref(deep), 0, 13, 0, 1) == (rows + rows // 32 + 8) * 2 * 128 * 4 + 4 * P4
     assert (rows + rows // 32 + 8) * 2 * 128 * 4 > h.ncn_workspace_bytes(ctypes.byref(deep))
     assert h.ncn_workspace_bytes_stages(ctypes.byref(deep), 0, 1, 0, 0) == 0
