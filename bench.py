@@ -17,10 +17,9 @@ backward call over a segment of stages where several stages run per launch) agai
 it: float32 vector arithmetic for groups of 8 rows and more (each element takes n_cache sequential tanh
 steps per stage), HBM bandwidth for smaller groups.  Its duration is measured with HIP events on the
 launch stream inside the timed region; the figures for the other roof ride along as hbm_* / valu_*.
-`roofline.frac` is against the published peak (157.3 TFLOP/s, which counts packed FP32 instructions; 8 TB/s); what
-this GPU sustains is measured in the same run and quoted beside it: `attainable_valu_TFLOPs` (a stream of independent
-plain v_fma_f32, the library's ncn_probe_fma_stream; the library is built without packed FP32) and
-`attainable_copy_GBps` (a 1 GiB device copy).
+`roofline.frac` is against the published peak (157.3 TFLOP/s; 8 TB/s); what this GPU sustains is measured in the
+same run and quoted beside it: `attainable_valu_TFLOPs` (a stream of independent v_fma_f32 on vector registers, the
+library's ncn_probe_issue; the library is built without packed FP32) and `attainable_copy_GBps` (a 1 GiB device copy).
 `stack.autograd_*` time the same workload through the reference's own surface (NCNNetTestCuda + yi.backward(dyi),
 grad_test_bench.py:116-134) and through the one-node form of the stack, `stack.graph_ms_per_step` replays the timed
 step from a HIP graph; all three outside the headline timed region.
@@ -48,7 +47,7 @@ CONFIGS = {
     "cfg5": dict(batch=64, N=2048, E=128, C=4, n=8, L=4, dtype="f32", w_scale=0.1),
 }
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
-VALU_PEAK_TFLOPS = 157.3   # MI355X FP32 vector peak, which counts packed FP32 instructions
+VALU_PEAK_TFLOPS = 157.3   # MI355X FP32 vector peak
 # float32 operations per element and step of the kernels as written in ncn_stage_kernels.h (FMA = 2, exp2 and
 # rcp = 1 each), without the per-row and per-lane bookkeeping: forward 5 FMA (row sum, z, two for xa, x) + the
 # +1 before the reciprocal + exp2 + rcp = 13; backward 12 FMA (inversion of x, row sum, z, two for xa, F'/4, the
@@ -311,8 +310,8 @@ def main():
     copy_gbps = 5 * 2.0 * src.numel() * 4 / (c0.elapsed_time(c1) * 1e-3) / 1e9
     del src, dst
 
-    # what this GPU sustains on plain float32 FMAs (no packed instructions, as the library is built): a stream of
-    # independent v_fma_f32, 8 waves per SIMD, timed with events on the launch stream
+    # what this GPU sustains on float32 FMAs without packed instructions (as the library is built): a stream of
+    # independent v_fma_f32 whose sources are vector registers, 8 waves per SIMD, timed with events on the launch stream
     from ncn_cuda_amd import probe
     lib = M._lib.load()
     attainable_valu = probe.fma_stream_tflops(device=dev)
@@ -440,7 +439,7 @@ def main():
             "kernel": kernel, "avg_launch_ms": bwd_ms,
             "algorithmic_flops_per_launch": flops_bwd_unit,
             "algorithmic_bytes_per_launch": bytes_bwd_launch,
-            "valu_achieved_TFLOPs": valu_achieved, "valu_frac_of_packed_peak": valu_achieved / VALU_PEAK_TFLOPS,
+            "valu_achieved_TFLOPs": valu_achieved, "valu_frac_of_peak": valu_achieved / VALU_PEAK_TFLOPS,
             "attainable_valu_TFLOPs": attainable_valu, "valu_frac_of_attainable": valu_achieved / attainable_valu,
             "hbm_achieved_GBps": hbm_achieved, "hbm_frac": hbm_achieved / HBM_PEAK_GBS,
             "attainable_copy_GBps": copy_gbps, "hbm_frac_of_attainable_copy": hbm_achieved / copy_gbps,

@@ -349,16 +349,16 @@ const char* ncn_build_id(void);
 
 /* Measurement aid, no part of the layer and no reference counterpart: kernels that only issue one kind of vector
  * instruction, or a mix shaped like the step code of the NCN kernels, built like the rest of the library (no packed
- * FP32).  bench.py quotes the plain-FMA rate they sustain beside the published 157.3 TFLOP/s (which counts packed FP32
- * instructions), and `python -m ncn_cuda_amd.probe` prints the whole table.
+ * FP32).  bench.py quotes the rate of a stream of v_fma_f32 on vector registers beside the published 157.3 TFLOP/s,
+ * and `python -m ncn_cuda_amd.probe` prints the whole table.
  * ncn_probe_issue launches `waves_per_simd` (1, 2, 4, 8) workgroups of 256 threads per CU, one wave per SIMD each (the
  * dynamic LDS they ask for keeps a CU from taking more); every lane runs `chains` (1, 4, 8) independent dependency
  * chains of iters * G groups of instructions, G = the return value of ncn_probe_issue_info, which also gives the
  * vector instructions and the floating-point operations one group counts.  out: 8 * CUs * 256 floats.  The caller
  * times the launch with events on `stream`. */
-#define NCN_PROBE_FMA 0           /* v_fma_f32 */
-#define NCN_PROBE_ADD 1           /* v_add_f32 */
-#define NCN_PROBE_MUL 2           /* v_mul_f32 */
+#define NCN_PROBE_FMA 0           /* v_fma_f32, every source a vector register */
+#define NCN_PROBE_ADD 1           /* v_add_f32, likewise */
+#define NCN_PROBE_MUL 2           /* v_mul_f32, likewise */
 #define NCN_PROBE_EXP2 3          /* v_exp_f32 */
 #define NCN_PROBE_RCP 4           /* v_rcp_f32 */
 #define NCN_PROBE_EXP2_ADD_RCP 5  /* 1 / (1 + 2^x): the activation of a step */
@@ -368,7 +368,11 @@ const char* ncn_build_id(void);
 #define NCN_PROBE_FORWARD_MIX 9   /* 5 fma, 2 add (1 across lanes), exp2, rcp: one element-step of the forward */
 #define NCN_PROBE_MFMA 10         /* v_mfma_f32_16x16x4_f32 */
 #define NCN_PROBE_FMA_AND_MFMA 11 /* 4 v_fma_f32 and one independent v_mfma_f32_16x16x4_f32: do they overlap? */
-#define NCN_PROBE_MODES 12
+#define NCN_PROBE_FMA_SGPR 12     /* v_fmac_f32 with a scalar-register source, every instruction */
+#define NCN_PROBE_FMA_SGPR_1_IN_4 13 /* the same, three v_fma_f32 on vector registers between two of them */
+#define NCN_PROBE_EXP2_1_IN_8 14  /* one v_exp_f32 and seven v_fma_f32: what a transcendental costs inside other work */
+#define NCN_PROBE_DPP_1_IN_2 15   /* v_add_f32 with a DPP operand and v_fma_f32 in turns */
+#define NCN_PROBE_MODES 16
 int ncn_probe_issue(int mode, int chains, int waves_per_simd, int iters, float* out, void* stream);
 int ncn_probe_issue_info(int mode, int* valu_per_group, int* flops_per_group);
 

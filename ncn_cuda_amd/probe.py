@@ -2,8 +2,9 @@
 
     python -m ncn_cuda_amd.probe [--iters N]
 
-Prints, for each instruction kind (and two mixes shaped like one element-step of the forward and of the backward step
-code), the time of a launch that issues nothing else, at 1, 2, 4 and 8 resident waves per SIMD and 1, 4 and 8
+Prints, for each instruction kind (in the operand forms that matter: sources in vector registers, a scalar-register
+source, a DPP operand; two mixes shaped like one element-step of the forward and of the backward step code; one
+instruction kind among FMAs), the time of a launch that issues nothing else, at 1, 2, 4 and 8 resident waves per SIMD and 1, 4 and 8
 independent dependency chains per lane:
 
     cycles = launch time x 2.4 GHz / (wave instructions issued per SIMD)     (2.4 GHz: the GPU's peak engine clock)
@@ -19,9 +20,10 @@ import torch
 
 from . import _lib
 
-MODES = ["v_fma_f32", "v_add_f32", "v_mul_f32", "v_exp_f32", "v_rcp_f32", "exp2, +1, rcp", "v_add_f32 dpp quad_perm",
-         "ds_swizzle + v_add_f32", "backward step mix", "forward step mix", "v_mfma_f32_16x16x4_f32",
-         "4 v_fma_f32 + 1 independent mfma"]
+MODES = ["v_fma_f32 (vector registers)", "v_add_f32", "v_mul_f32", "v_exp_f32", "v_rcp_f32", "exp2, +1, rcp",
+         "v_add_f32 dpp quad_perm", "ds_swizzle + v_add_f32", "backward step mix", "forward step mix",
+         "v_mfma_f32_16x16x4_f32", "4 v_fma_f32 + 1 independent mfma", "v_fmac_f32 with a scalar source",
+         "1 scalar-source fmac : 3 v_fma_f32", "1 v_exp_f32 : 7 v_fma_f32", "1 dpp add : 1 v_fma_f32"]
 PEAK_CLOCK_HZ = 2.4e9
 
 
@@ -54,7 +56,8 @@ def time_launch(mode, chains, waves, iters, reps=3, device=None):
 
 
 def fma_stream_tflops(iters=2048, device=None):
-    """Plain v_fma_f32, 8 chains per lane, 8 waves per SIMD: the float32 vector rate without packed instructions."""
+    """v_fma_f32 on vector registers, 8 chains per lane, 8 waves per SIMD: the float32 vector rate without packed
+    instructions."""
     ms, _, flops = time_launch(0, 8, 8, iters, device=device)
     return flops / (ms * 1e-3) / 1e12
 
@@ -73,8 +76,9 @@ def main():
         for waves in (1, 2, 4, 8):
             for chains in (1, 4, 8):
                 ms, instr, flops = time_launch(mode, chains, waves, args.iters)
-                print(f"{name:34s} {waves:10d} {chains:6d} {ms:8.3f} {ms * 1e-3 * PEAK_CLOCK_HZ / instr:12.2f} "
-                      f"{flops / (ms * 1e-3) / 1e12:8.2f}", flush=True)
+                rate = f"{flops / (ms * 1e-3) / 1e12:8.2f}" if flops else f"{'-':>8s}"
+                print(f"{name:34s} {waves:10d} {chains:6d} {ms:8.3f} {ms * 1e-3 * PEAK_CLOCK_HZ / instr:12.2f} {rate}",
+                      flush=True)
 
 
 if __name__ == "__main__":

@@ -438,6 +438,8 @@ def test_probe_entry_points_validate_their_arguments(lib):
     valu, flops = ctypes.c_int(0), ctypes.c_int(0)
     assert h.ncn_probe_issue_info(0, ctypes.byref(valu), ctypes.byref(flops)) == 8 and (valu.value, flops.value) == (1, 2)
     assert h.ncn_probe_issue_info(8, ctypes.byref(valu), ctypes.byref(flops)) == 8 and (valu.value, flops.value) == (20, 28)
+    assert h.ncn_probe_issue_info(15, ctypes.byref(valu), ctypes.byref(flops)) == 8 and (valu.value, flops.value) == (1, 0)
+    assert h.ncn_probe_issue_info(16, None, None) == -2
     assert h.ncn_probe_issue_info(99, None, None) == -2
     p = ctypes.c_void_p(4096)
     assert h.ncn_probe_issue(0, 8, 8, 16, None, None) == -1
