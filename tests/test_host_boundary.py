@@ -288,6 +288,18 @@ def _passes(lib, shape, first, count, backward):
     return [tuple(buf[8 * j:8 * j + 8]) for j in range(k)]
 
 
+def test_planner_puts_stages_where_they_cost_least(lib):
+    """The 13 stages of the deep configuration.  Backward: the pass that runs last (stages 0-2) writes gradients only
+    and is bound by instruction issue, the middle pass by its traffic, where a third stage is free: stages 3-5 go
+    there, not a fourth stage into the last pass (both cuts move the same bytes).  Forward: two passes."""
+    shape = _shape(lib, 128, 8192, 128, 4, 2)
+    bwd = _passes(lib, shape, 0, 13, True)
+    assert [(p[0], p[1], p[2]) for p in bwd] == [(0, 3, 1), (3, 3, 1), (6, 7, 2)]      # (first, count, 1 halo / 2 closed)
+    assert [(p[4], p[6]) for p in bwd] == [(128, 122), (128, 114), (128, 128)]         # (window, owned groups)
+    fwd = _passes(lib, shape, 0, 13, False)
+    assert [(p[0], p[1], p[2]) for p in fwd] == [(0, 5, 1), (5, 8, 2)]
+
+
 @pytest.mark.parametrize("backward", [False, True])
 @pytest.mark.parametrize("dims", [(128, 8192, 128, 4, 2, 0, 13), (32, 1024, 128, 4, 4, 0, 5), (3, 1024, 64, 2, 2, 0, 11),
                                   (2, 2048, 64, 2, 2, 3, 6), (5, 64, 128, 4, 4, 0, 3), (1, 1 << 16, 32, 1, 2, 0, 20),
