@@ -358,7 +358,7 @@ hipError_t static_scratch(float** out) {
 
 extern "C" {
 
-const char* ncn_version(void) { return "0.12"; }
+const char* ncn_version(void) { return "0.13"; }
 
 int ncn_plan_passes(const ncn_shape* shape, int first_stage, int n_stages, int activation, int backward, int32_t* out,
                     int max_passes) {

@@ -15,4 +15,4 @@
 // lengths and for the radix-n levels alike.  Groups of 8 rows and more are bound by arithmetic even stage by stage
 // (measured 10 % slower through LDS) and have none.
 #define NCN_FOR_EACH_FUSED_CONFIG(X) \
-    X(2, 8) X(4, 8) X(2, 16) X(4, 16) X(2, 32) X(4, 32) X(2, 64) X(4, 64)
+    X(2, 8) X(4, 8) X(2, 16) X(4, 16) X(2, 32) X(4, 32) X(2, 64) X(4, 64) X(2, 128) X(4, 128)

@@ -81,7 +81,8 @@ std::vector<FusedPass> plan_fused(const ncn_shape* sh, int first, int count, boo
     for (int k = 0; k < count; ++k) s[k] = stage_stride_of(first + k, groups);
 
     // backward keeps a dW slot per wave and stage in LDS: 7 stages leave room for two workgroups per CU at heads of up
-    // to 32 features; the two-row kernels at wider heads take as many stages as still let two workgroups share a CU
+    // to 32 features; the two-row kernels at heads of 64 take as many stages as still let two workgroups share a CU
+    // (3), at heads of 128 not even two stages would and a CU runs one workgroup of up to 7 stages
     int max_stages = backward ? kFusedMaxStages - 1 : kFusedMaxStages;
     if (backward && nc == 2) {
         const size_t budget = 80 * 1024, fixed = pair_state_bytes(true) / 2 + (size_t)kFusedMaxStages * 2 * ec * sizeof(float);

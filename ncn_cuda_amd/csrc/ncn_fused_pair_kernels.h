@@ -259,13 +259,13 @@ __global__ void __launch_bounds__(64 * kFusedWavesFwd, NCN_PAIR_FWD_WAVES) pair_
 // DPP moves whose write masks pick the side and one add.  (Summing every value in every lane costs one instruction
 // per value and level: 3 levels x 16 values against 33 instructions here at 4 lanes per group.)
 template <int LF>
-constexpr int pair_scatter_levels() { return LF <= 4 ? 4 : 3; }   // lane bits 5, 4, 3 and, when it is a group bit, 2
+constexpr int pair_scatter_levels() { return LF <= 4 ? 4 : LF == 8 ? 3 : 2; }   // lane bits 5, 4 and, where they are group bits, 3 and 2
 template <int LF, int NV>
 constexpr int pair_scatter_left() { return NV >> pair_scatter_levels<LF>(); }
 
 template <int LF, int NV>
 __device__ __forceinline__ int pair_scatter_sum(float (&v)[NV], int lane) {
-    static_assert(LF == 1 || LF == 2 || LF == 4 || LF == 8, "lanes per group");
+    static_assert(LF == 1 || LF == 2 || LF == 4 || LF == 8 || LF == 16, "lanes per group");
     static_assert(NV == 16, "two rows of 8 weights");
     // lane bit 5: lower half-wave keeps v[0..8), upper v[8..16)
 #pragma unroll
@@ -279,15 +279,18 @@ __device__ __forceinline__ int pair_scatter_sum(float (&v)[NV], int lane) {
         const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v[i]), __float_as_uint(v[i + 4]), false, false);
         v[i] = __uint_as_float(r[0]) + __uint_as_float(r[1]);
     }
-    // lane bit 3: banks 0,1 of a row keep v[0..2), banks 2,3 keep v[2..4); row_ror:8 reads lane (l + 8) mod 16
+    int first = ((lane >> 5) & 1) * 8 + ((lane >> 4) & 1) * 4;
+    if constexpr (LF <= 8) {
+        // lane bit 3: banks 0,1 of a row keep v[0..2), banks 2,3 keep v[2..4); row_ror:8 reads lane (l + 8) mod 16
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int lo = __float_as_int(v[i]), hi = __float_as_int(v[i + 2]);
-        const int t = __builtin_amdgcn_update_dpp(hi, lo, 0x128, 0xF, 0x3, false);   // banks 0,1: partner's lo; 2,3: own hi
-        const int u = __builtin_amdgcn_update_dpp(lo, hi, 0x128, 0xF, 0xC, false);   // banks 2,3: partner's hi; 0,1: own lo
-        v[i] = __int_as_float(t) + __int_as_float(u);
+        for (int i = 0; i < 2; ++i) {
+            const int lo = __float_as_int(v[i]), hi = __float_as_int(v[i + 2]);
+            const int t = __builtin_amdgcn_update_dpp(hi, lo, 0x128, 0xF, 0x3, false);   // banks 0,1: partner's lo; 2,3: own hi
+            const int u = __builtin_amdgcn_update_dpp(lo, hi, 0x128, 0xF, 0xC, false);   // banks 2,3: partner's hi; 0,1: own lo
+            v[i] = __int_as_float(t) + __int_as_float(u);
+        }
+        first += ((lane >> 3) & 1) * 2;
     }
-    int first = ((lane >> 5) & 1) * 8 + ((lane >> 4) & 1) * 4 + ((lane >> 3) & 1) * 2;
     if constexpr (LF <= 4) {
         // lane bit 2: banks 0,2 keep v[0], banks 1,3 keep v[1]; row_shl:4 reads lane l + 4, row_shr:4 lane l - 4
         const int lo = __float_as_int(v[0]), hi = __float_as_int(v[1]);

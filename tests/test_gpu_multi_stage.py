@@ -38,6 +38,8 @@ CASES = [
     (1, 3 * 4096, 128, 4, 2, 0, 13), # 6144 groups: halo passes on a ring that is no power of two, then closed ones
     (2, 5 * 256, 64, 2, 2, 0, 9),    # 640 groups = 5 * 2^7
     (2, 7 * 64, 32, 2, 4, 2, 5),     # n = 4, 112 groups = 7 * 16, from stage 2
+    (2, 2048, 256, 2, 2, 0, 11),     # n = 2, head width 128 (16 lanes per row, windows of 32 groups)
+    (2, 1024, 128, 1, 4, 5, 4),      # n = 4, head width 128: closed passes on the rings of the high stages
 ]
 
 
@@ -55,8 +57,8 @@ def test_multi_stage_matches_single_stage_and_oracle(M, case):
     for l in range(L):
         cx, cxa = M.forward(cx, cxa, gWs[l], alpha, 0, n, C, first + l)
         outs.append((cx, cxa))
-    # groups of 2 and 4 rows at heads of 8 to 64 features, an even number of groups: the call really uses LDS passes
-    if n in (2, 4) and E // C in (8, 16, 32, 64) and (N // n) % 2 == 0:
+    # groups of 2 and 4 rows at heads of 8 to 128 features, an even number of groups: the call really uses LDS passes
+    if n in (2, 4) and E // C in (8, 16, 32, 64, 128) and (N // n) % 2 == 0:
         import ctypes
         from ncn_cuda_amd import _lib
         shape = _lib.NcnShape(batch, N, E, C, n)

@@ -305,6 +305,7 @@ def test_planner_puts_stages_where_they_cost_least(lib):
                                   (2, 2048, 64, 2, 2, 3, 6), (5, 64, 128, 4, 4, 0, 3), (1, 1 << 16, 32, 1, 2, 0, 20),
                                   (3, 2048, 16, 2, 2, 0, 10), (2, 2048, 128, 2, 2, 0, 11), (2, 1024, 32, 4, 4, 0, 6),
                                   (2, 512, 128, 2, 4, 0, 6),                      # heads of 8 and of 64 features
+                                  (2, 2048, 256, 2, 2, 0, 11), (2, 1024, 128, 1, 4, 5, 4),   # heads of 128 features
                                   (2, 3 * 512, 64, 2, 2, 0, 12), (2, 96, 32, 4, 4, 0, 6), (2, 3 * 4096, 128, 4, 2, 0, 14),
                                   (2, 5 * 256, 64, 2, 2, 0, 9), (2, 7 * 64, 32, 2, 4, 2, 5)])  # 3, 5, 7 times a power of two
 def test_multi_stage_plan_invariants(lib, dims, backward):
