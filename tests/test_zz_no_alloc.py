@@ -119,3 +119,61 @@ def test_backward_static_needs_the_state_buffers_for_several_stages():
                                  0.9, 0.9, 0, None)
     torch.cuda.synchronize()
     assert rc == 0 and torch.isfinite(out[0]).all() and torch.isfinite(dW[0]).all()
+
+
+def test_backward_static_under_graph_capture():
+    """What the entry point is for: after one warm-up call (which resolves the scratch's address and is not
+    capturable), a call recorded into a HIP graph replays on new inputs like the eager ncn_backward."""
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from ncn_cuda_amd import _lib
+    lib = _lib.load()
+    batch, N, E, C, n = 4, 256, 128, 4, 16
+    dev = torch.device("cuda:0")
+    sh = _lib.NcnShape(batch, N, E, C, n)
+    sets = [O.make_inputs(batch, N, E, 1, n, seed=70 + k, xa_zero=False) for k in range(3)]
+    W = sets[0][2][0].to(dev)
+    y, ya, dy, dya = (torch.empty(batch, N, E, device=dev) for _ in range(4))
+    dx, dxa = torch.empty_like(y), torch.empty_like(y)
+    dW = torch.empty(1, 2 * E, device=dev)
+
+    def load(k):   # the stage outputs of input set k, and its upstream gradients
+        x, xa = sets[k][0].to(dev), sets[k][1].to(dev)
+        rc = lib.ncn_forward(x.data_ptr(), xa.data_ptr(), 0, y.data_ptr(), ya.data_ptr(), 0, None, None, W.data_ptr(), None, 0,
+                             ctypes.byref(sh), 0, 1, 0.9, 0.9, 0, None)
+        assert rc == 0
+        dy.copy_(sets[k][3]); dya.copy_(sets[k][4])
+
+    def static_call(stream):
+        return lib.ncn_backward_static(y.data_ptr(), ya.data_ptr(), 0, dy.data_ptr(), dya.data_ptr(), 0, dx.data_ptr(),
+                                       dxa.data_ptr(), 0, None, None, W.data_ptr(), dW.data_ptr(), ctypes.byref(sh), 0, 1,
+                                       0.9, 0.9, 0, stream)
+
+    load(0)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        assert static_call(ctypes.c_void_p(side.cuda_stream)) == 0      # warm-up, outside any capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        before = torch.cuda.memory_allocated()
+        assert static_call(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)) == 0
+        assert torch.cuda.memory_allocated() == before
+    ws_bytes = lib.ncn_workspace_bytes(ctypes.byref(sh))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    for k in (1, 2, 0, 1):
+        load(k)
+        dx.fill_(float("nan")); dxa.fill_(float("nan")); dW.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [dx.clone(), dxa.clone(), dW.clone()]
+        ex, exa, eW = torch.empty_like(dx), torch.empty_like(dx), torch.empty_like(dW)    # eager work between the replays
+        rc = lib.ncn_backward(y.data_ptr(), ya.data_ptr(), 0, dy.data_ptr(), dya.data_ptr(), 0, ex.data_ptr(), exa.data_ptr(), 0,
+                              None, None, W.data_ptr(), eW.data_ptr(), ws.data_ptr(), ctypes.c_size_t(ws_bytes),
+                              ctypes.byref(sh), 0, 1, 0.9, 0.9, 0, None)
+        assert rc == 0
+        torch.cuda.synchronize()
+        assert torch.equal(got[0], ex) and torch.equal(got[1], exa)
+        assert O.rel_err(got[2], eW) < 1e-5 and torch.isfinite(got[2]).all()
