@@ -51,13 +51,18 @@ VALU_PEAK_TFLOPS = 157.3   # MI355X FP32 vector peak
 # float32 operations per element and step of the kernels as written in ncn_stage_kernels.h (FMA = 2, exp2 and
 # rcp = 1 each), without the per-row and per-lane bookkeeping: forward 5 FMA (row sum, z, two for xa, x) + the
 # +1 before the reciprocal + exp2 + rcp = 13; backward 12 FMA (inversion of x, row sum, z, two for xa, F'/4, the
-# row's <U, x_j>, the pivot row's sum, two for G, dWi, P) + the +1 + P F'/4 + exp2 + rcp = 28.
+# row's <U, x_j>, the pivot row's sum, two for G, dWi, P) + the +1 + P F'/4 + exp2 + rcp = 28.  (Heads of one feature,
+# ncn_headwise_kernels.h: the same 13, and 29 with the products that are no longer shared by a row; counted as 28.)
 FLOPS_FWD_PER_ELEM_STEP = 13.0
 FLOPS_BWD_PER_ELEM_STEP = 28.0
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
 
 
-def measured_traffic(config, grouping, version):
+def traffic_key(config, grouping, scalar_heads=False):
+    return f"{config}/{grouping}" + ("/scalar-heads" if scalar_heads else "")
+
+
+def measured_traffic(config, grouping, version, scalar_heads=False):
     """HBM bytes per launch (or per backward call over a segment) of the dominant kernel, from the profile record of
     this library version; None when there is none."""
     try:
@@ -65,7 +70,7 @@ def measured_traffic(config, grouping, version):
             rec = json.load(fh)
     except (OSError, ValueError):
         return None
-    entry = rec.get("entries", {}).get(f"{config}/{grouping}")
+    entry = rec.get("entries", {}).get(traffic_key(config, grouping, scalar_heads))
     if not entry or entry.get("ncn_version") != version:
         return None
     return entry.get("bytes")
@@ -94,6 +99,8 @@ def record_traffic(prof_dir):
     workload = meta["config"]["workload"]
     config = workload.split(":")[0]
     grouping = workload.rsplit("grouping ", 1)[1]
+    key = traffic_key(config, grouping, " heads of 1," in workload)
+    one_stage = ("stage_backward_kernel", "headwise_backward_kernel")
     steps = meta["steps"] + meta["warmup"]
     per_call = "backward call" in meta["roofline"]["kernel"]
     sizes, factors, names = {}, {}, {}
@@ -119,9 +126,9 @@ def record_traffic(prof_dir):
             short = lambda n: n.replace("(anonymous namespace)::", "").split("(")[0].replace("void ", "")
             names[d] = ", ".join(f"{c / n_calls:g} x {short(n)}" for n, c in sorted(counts.items()))
         else:           # the one-stage backward kernel, per launch
-            mine = [v for k, v in per_dispatch.items() if "stage_backward_kernel" in k[0]]
+            mine = [v for k, v in per_dispatch.items() if any(o in k[0] for o in one_stage)]
             sizes[d] = sum(mine) / len(mine) * factors[d] * 1024.0
-            names[d] = sorted({k[0] for k in per_dispatch if "stage_backward_kernel" in k[0]})[0].split("(")[0].replace("void ", "")
+            names[d] = sorted({k[0] for k in per_dispatch if any(o in k[0] for o in one_stage)})[0].split("(")[0].replace("void ", "")
     try:
         with open(TRAFFIC_FILE) as fh:
             rec = json.load(fh)
@@ -131,7 +138,7 @@ def record_traffic(prof_dir):
                       "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, written by `python bench.py --record-traffic <dir>` from the "
                       "counter files and logs of the profiled runs; bench.py reports an entry only for the library version "
                       "it was measured on")
-    rec["entries"][f"{config}/{grouping}"] = {
+    rec["entries"][key] = {
         "ncn_version": meta["roofline"]["ncn_version"], "build_id": meta["roofline"]["build_id"],
         "kernel": names["f"], "bytes": round(sizes["f"] + sizes["w"]), "read_bytes": round(sizes["f"]),
         "written_bytes": round(sizes["w"]), "fetch_size_factor": round(factors["f"], 4),
@@ -139,7 +146,7 @@ def record_traffic(prof_dir):
     with open(TRAFFIC_FILE, "w") as fh:
         json.dump(rec, fh, indent=1)
         fh.write("\n")
-    print(json.dumps(rec["entries"][f"{config}/{grouping}"]))
+    print(json.dumps(rec["entries"][key]))
 
 
 def main():
@@ -165,7 +172,7 @@ def main():
                          "modules.default_save_every)")
     ap.add_argument("--scalar-heads", action="store_true",
                     help="the literal scalar reading of x[B, D]: one feature per head (n_head = E), a different shape "
-                         "from the one the metric is quoted on; runs on the generic kernels")
+                         "from the one the metric is quoted on; register kernels that hold four heads per lane")
     ap.add_argument("--no-surface", action="store_true",
                     help="skip the legs outside the timed region that go through the autograd surface and a HIP graph")
     ap.add_argument("--copy-probe", action="store_true",
@@ -244,7 +251,7 @@ def main():
                 saved.append((sy, sya))
             elif bf16 and cnt == 1:
                 # bf16 outputs plus what their rounding took away (a second bf16 plane): what the backward inverts
-                # (float32 copies instead where only the generic kernels take the shape: --scalar-heads)
+                # (float32 copies instead where only the generic kernels take the shape)
                 cx, cxa, ys, yas = M.forward_stages_saving(cx, cxa, Wst[a], alpha, 0, n, C, a, ctx_len=lens)
                 saved.append((ys, yas))
             else:
@@ -426,7 +433,8 @@ def main():
     version = lib.ncn_version().decode()
     import ctypes
     on_register_kernels = lib.ncn_kernel_path(ctypes.byref(M._lib.NcnShape(batch, N, E, C, n))) == 2
-    kernel = ((f"stage_backward_kernel<{n},{E // C}>" if on_register_kernels else
+    kernel = ((f"headwise_backward_kernel<{n}> (one feature per head, four heads to a lane)" if on_register_kernels and C == E else
+               f"stage_backward_kernel<{n},{E // C}>" if on_register_kernels else
                f"generic_backward_kernel (n_cache {n}, heads of {E // C}: no register-tile build)") +
               (" (indexed build)" if tables else "") if not lds_passes else
               f"backward call over a segment of up to {save_every} stages (multi-stage passes)")
@@ -435,7 +443,7 @@ def main():
             "peak": VALU_PEAK_TFLOPS if valu_bound else HBM_PEAK_GBS,
             "unit": "TFLOP/s" if valu_bound else "GB/s",
             "frac": (valu_achieved / VALU_PEAK_TFLOPS) if valu_bound else (hbm_achieved / HBM_PEAK_GBS),
-            "traffic": None if args.scalar_heads else measured_traffic(args.config, args.grouping, version),
+            "traffic": measured_traffic(args.config, args.grouping, version, args.scalar_heads),
             "kernel": kernel, "avg_launch_ms": bwd_ms,
             "algorithmic_flops_per_launch": flops_bwd_unit,
             "algorithmic_bytes_per_launch": bytes_bwd_launch,

@@ -20,10 +20,17 @@ bool known_dtype(int d) { return d == NCN_F32 || d == NCN_BF16; }
 bool known_dtype_or_x2(int d, int n_stages, int path) { return known_dtype(d) || (d == NCN_BF16X2 && n_stages == 1 && path == 2); }
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// Heads of one feature (E == n_head) run on the register kernels of ncn_headwise_kernels.h, four adjacent heads to a lane.
+bool headwise_shape(const ncn_shape* sh) {
+    const int w = headwise_width(sh->E);
+    return sh->E == sh->n_head && w != 0 && sh->n_cache <= 64 && fast_tile(sh->n_cache, w).r != 0;
+}
+
 // 2 = register kernels, 1 = generic LDS kernels, 0 = unsupported
 int kernel_path(const ncn_shape* sh, int /*activation*/) {
     if (sh->n_cache < 1 || sh->n_cache > 64) return 0;
     const int64_t ec = sh->E / sh->n_head;
+    if (headwise_shape(sh)) return 2;
     if (ec <= 128 && fast_tile(sh->n_cache, (int)ec).r != 0) return 2;
     if (ec <= kGenericMaxHeadDim) return 1;
     return 0;
@@ -228,6 +235,28 @@ hipError_t launch_ragged_rest(Pass pass, StageArgs a, const ncn_shape* sh, int p
 }
 int edge_rows(const ncn_shape* sh) { return (int)(sh->batch < kEdgeGridX ? sh->batch : kEdgeGridX); }
 
+// A call on heads of one feature that the register kernels take (path 2) is planned and launched with the geometry
+// of E / w heads of w = headwise_width(E) features, which `as_wide` receives: same tiles, grids and partial rows as
+// for such heads, other kernels.
+bool headwise_call(const ncn_shape* sh, int path, ncn_shape* as_wide) {
+    if (path != 2 || !headwise_shape(sh)) return false;
+    *as_wide = *sh;
+    as_wide->n_head = (int)(sh->E / headwise_width(sh->E));
+    return true;
+}
+
+// one stage on the register kernels: the plain builds know the stride permutation only, the others read the
+// launch's table, radix level and context lengths
+hipError_t run_forward_kernel(Pass pass, const StageArgs& a, bool plain, bool headwise, int n_head, int grid,
+                              hipStream_t s) {
+    if (headwise) return plain ? launch_headwise_forward(pass, a, grid, s) : launch_headwise_forward_indexed(pass, a, grid, s);
+    return plain ? launch_fast_forward(pass, a, n_head, grid, s) : launch_fast_forward_indexed(pass, a, n_head, grid, s);
+}
+hipError_t run_backward_kernel(const StageArgs& a, bool plain, bool headwise, int n_head, int grid, hipStream_t s) {
+    if (headwise) return plain ? launch_headwise_backward(a, grid, s) : launch_headwise_backward_indexed(a, grid, s);
+    return plain ? launch_fast_backward(a, n_head, grid, s) : launch_fast_backward_indexed(a, n_head, grid, s);
+}
+
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 // rows of chunk sums that the launches of one reduction job can need when they fill row_cap partial rows
@@ -358,7 +387,7 @@ hipError_t static_scratch(float** out) {
 
 extern "C" {
 
-const char* ncn_version(void) { return "0.13"; }
+const char* ncn_version(void) { return "0.14"; }
 
 int ncn_plan_passes(const ncn_shape* shape, int first_stage, int n_stages, int activation, int backward, int32_t* out,
                     int max_passes) {
@@ -441,6 +470,9 @@ static int forward_impl(const void* x, const void* xa, int in_dtype, void* y, vo
     if ((y32 == nullptr) != (ya32 == nullptr)) return NCN_ERR_NULL;
     const int path = kernel_path_for(shape, activation, alpha, m);
     if (path == 0) return NCN_ERR_UNSUPPORTED;
+    ncn_shape as_wide;
+    const bool headwise = headwise_call(shape, path, &as_wide);
+    if (headwise) shape = &as_wide;
     if (!known_dtype(in_dtype) || !known_dtype_or_x2(out_dtype, n_stages, path)) return NCN_ERR_DTYPE;
     if (!aligned16(x) || !aligned16(xa) || !aligned16(y) || !aligned16(ya) || !aligned16(W) || !aligned16(y32) ||
         !aligned16(ya32) || !aligned16(workspace))
@@ -451,7 +483,8 @@ static int forward_impl(const void* x, const void* xa, int in_dtype, void* y, vo
 
     // several stages: LDS-resident passes when the shape allows and the buffers permit the ping-pong
     std::vector<FusedPass> passes;
-    if (grouping.permutation()) passes = multi_stage_plan(shape, first_stage, n_stages, activation, false, path);
+    // (heads of one feature have no multi-stage kernels: one launch per stage)
+    if (grouping.permutation() && !headwise) passes = multi_stage_plan(shape, first_stage, n_stages, activation, false, path);
     const size_t np = passes.size();
     // one stage of the range with the one-stage kernel (and, with lengths, the launch for the rows past them)
     auto run_stage = [&](int k, const void* i0, const void* i1, int i_dtype, void* o0, void* o1, int o_dtype,
@@ -462,8 +495,7 @@ static int forward_impl(const void* x, const void* xa, int in_dtype, void* y, vo
         a.out0 = o0; a.out1 = o1; a.out_dtype = o_dtype;
         a.aux0 = with_copies ? y32 : nullptr; a.aux1 = with_copies ? ya32 : nullptr;
         a.W = W + k * wstride;
-        hipError_t err = grouping.plain() ? launch_fast_forward(kForward, a, shape->n_head, p.grid_fwd, s)
-                                          : launch_fast_forward_indexed(kForward, a, shape->n_head, p.grid_fwd, s);
+        hipError_t err = run_forward_kernel(kForward, a, grouping.plain(), headwise, shape->n_head, p.grid_fwd, s);
         if (err == hipSuccess && grouping.ctx_len) err = launch_ragged_rest(kForward, a, shape, p.path, 0, s);
         return err;
     };
@@ -546,9 +578,8 @@ static int forward_impl(const void* x, const void* xa, int in_dtype, void* y, vo
         a.aux0 = last ? y32 : nullptr;
         a.aux1 = last ? ya32 : nullptr;
         a.W = W + k * wstride;
-        hipError_t err = (p.path != 2)      ? launch_generic(kForward, a, shape->n_head, p.grid_fwd, s)
-                         : grouping.plain() ? launch_fast_forward(kForward, a, shape->n_head, p.grid_fwd, s)
-                                            : launch_fast_forward_indexed(kForward, a, shape->n_head, p.grid_fwd, s);
+        hipError_t err = (p.path != 2) ? launch_generic(kForward, a, shape->n_head, p.grid_fwd, s)
+                                       : run_forward_kernel(kForward, a, grouping.plain(), headwise, shape->n_head, p.grid_fwd, s);
         if (err == hipSuccess && grouping.ctx_len) err = launch_ragged_rest(kForward, a, shape, p.path, 0, s);
         if (err != hipSuccess) return (int)err;
     }
@@ -565,6 +596,9 @@ static int inverse_impl(const void* y, const void* ya, int in_dtype, void* x, vo
     if (!x || !xa || !y || !ya || !W) return NCN_ERR_NULL;
     const int path = kernel_path_for(shape, activation, alpha, m);
     if (path == 0) return NCN_ERR_UNSUPPORTED;
+    ncn_shape as_wide;
+    const bool headwise = headwise_call(shape, path, &as_wide);
+    if (headwise) shape = &as_wide;
     if (!known_dtype_or_x2(in_dtype, n_stages, path) || !known_dtype(out_dtype)) return NCN_ERR_DTYPE;
     if (!aligned16(x) || !aligned16(xa) || !aligned16(y) || !aligned16(ya) || !aligned16(W) || !aligned16(workspace))
         return NCN_ERR_ALIGN;
@@ -575,7 +609,7 @@ static int inverse_impl(const void* y, const void* ya, int in_dtype, void* x, vo
     // first pass to run goes from y, ya to x, xa and the others work in place on x, xa, which a halo pass must not,
     // so the stages of such a pass are undone by one-stage launches (closed passes and one-stage launches may).
     std::vector<FusedPass> passes;
-    if (grouping.permutation() && (out_dtype == NCN_F32 || n_stages == 1))
+    if (grouping.permutation() && !headwise && (out_dtype == NCN_F32 || n_stages == 1))
         passes = multi_stage_plan(shape, first_stage, n_stages, activation, false, path);
     auto run_stage = [&](int k, const void* i0, const void* i1, int i_dtype, void* o0, void* o1, int o_dtype) -> hipError_t {
         StageArgs a{};
@@ -583,8 +617,7 @@ static int inverse_impl(const void* y, const void* ya, int in_dtype, void* x, vo
         a.in0 = i0; a.in1 = i1; a.in_dtype = i_dtype;
         a.out0 = o0; a.out1 = o1; a.out_dtype = o_dtype;
         a.W = W + (int64_t)k * 2 * shape->E;
-        hipError_t err = grouping.plain() ? launch_fast_forward(kInverse, a, shape->n_head, p.grid_fwd, s)
-                                          : launch_fast_forward_indexed(kInverse, a, shape->n_head, p.grid_fwd, s);
+        hipError_t err = run_forward_kernel(kInverse, a, grouping.plain(), headwise, shape->n_head, p.grid_fwd, s);
         if (err == hipSuccess && grouping.ctx_len) err = launch_ragged_rest(kInverse, a, shape, p.path, 0, s);
         return err;
     };
@@ -663,9 +696,8 @@ static int inverse_impl(const void* y, const void* ya, int in_dtype, void* x, vo
         a.out1 = xa;
         a.out_dtype = out_dtype;
         a.W = W + (int64_t)k * 2 * shape->E;
-        hipError_t err = (p.path != 2)      ? launch_generic(kInverse, a, shape->n_head, p.grid_fwd, s)
-                         : grouping.plain() ? launch_fast_forward(kInverse, a, shape->n_head, p.grid_fwd, s)
-                                            : launch_fast_forward_indexed(kInverse, a, shape->n_head, p.grid_fwd, s);
+        hipError_t err = (p.path != 2) ? launch_generic(kInverse, a, shape->n_head, p.grid_fwd, s)
+                                       : run_forward_kernel(kInverse, a, grouping.plain(), headwise, shape->n_head, p.grid_fwd, s);
         if (err == hipSuccess && grouping.ctx_len) err = launch_ragged_rest(kInverse, a, shape, p.path, 0, s);
         if (err != hipSuccess) return (int)err;
     }
@@ -685,6 +717,9 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
     if ((x_rec == nullptr) != (xa_rec == nullptr)) return NCN_ERR_NULL;
     const int path = kernel_path_for(shape, activation, alpha, m);
     if (path == 0) return NCN_ERR_UNSUPPORTED;
+    ncn_shape as_wide;
+    const bool headwise = headwise_call(shape, path, &as_wide);
+    if (headwise) shape = &as_wide;
     if (!known_dtype_or_x2(y_dtype, n_stages, path) || !known_dtype(dy_dtype) || !known_dtype(dx_dtype)) return NCN_ERR_DTYPE;
     if (n_stages > 1 && dx_dtype != NCN_F32) return NCN_ERR_ALIAS;
     if (!workspace || workspace_bytes < partial_buffer_bytes(shape, row_cap)) return NCN_ERR_WORKSPACE;
@@ -707,7 +742,7 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
     // several stages: LDS-resident passes, last pass of the range first; the state ping-pongs between the
     // output arrays and four float32 arrays behind the dW scratch (their grids count on kMaxGridX partial rows)
     std::vector<FusedPass> passes;
-    if (grouping.permutation() && row_cap == kMaxGridX)
+    if (grouping.permutation() && !headwise && row_cap == kMaxGridX)
         passes = multi_stage_plan(shape, first_stage, n_stages, activation, true, path);
     const size_t np = passes.size();
     bool fused_ok = np > 0;
@@ -758,8 +793,7 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
                 a.aux0 = dxr; a.aux1 = dxar;
                 a.W = W + ps.first * wstride;
                 a.dw_partials = region;
-                err = grouping.plain() ? launch_fast_backward(a, shape->n_head, p.grid_x, s)
-                                       : launch_fast_backward_indexed(a, shape->n_head, p.grid_x, s);
+                err = run_backward_kernel(a, grouping.plain(), headwise, shape->n_head, p.grid_x, s);
                 if (err == hipSuccess && grouping.ctx_len)
                     err = launch_ragged_rest(kBackward, a, shape, p.path, p.partial_rows, s);
             } else {
@@ -809,9 +843,8 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
         a.aux1 = (no_rec && k == 0) ? nullptr : xa_rec;
         a.W = W + (int64_t)k * 2 * shape->E;
         a.dw_partials = region;
-        err = (p.path != 2)      ? launch_generic(kBackward, a, shape->n_head, p.grid_x, s)
-              : grouping.plain() ? launch_fast_backward(a, shape->n_head, p.grid_x, s)
-                                 : launch_fast_backward_indexed(a, shape->n_head, p.grid_x, s);
+        err = (p.path != 2) ? launch_generic(kBackward, a, shape->n_head, p.grid_x, s)
+                            : run_backward_kernel(a, grouping.plain(), headwise, shape->n_head, p.grid_x, s);
         if (err == hipSuccess && grouping.ctx_len) err = launch_ragged_rest(kBackward, a, shape, p.path, p.partial_rows, s);
         if (err != hipSuccess) return (int)err;
         reducer.add(region, p.partial_rows + extra_rows, 1, dW + k * wstride);
@@ -906,10 +939,13 @@ int ncn_forward_radix(const void* x, const void* xa, int in_dtype, void* y, void
         return NCN_ERR_ALIGN;
     const int path = kernel_path_for(shape, activation, alpha, m);
     if (path == 0) return NCN_ERR_UNSUPPORTED;
+    ncn_shape as_wide;
+    const bool headwise = headwise_call(shape, path, &as_wide);
+    if (headwise) shape = &as_wide;
     const Plan p = make_plan(shape, path);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int64_t wstride = 2 * shape->E;
-    const std::vector<RadixPass> passes = plan_radix(shape, first_level, n_levels, false, path == 2);
+    const std::vector<RadixPass> passes = plan_radix(shape, first_level, n_levels, false, path == 2 && !headwise);
     // every pass is closed: the first reads x, xa and the later ones run in place on y, ya; passes of several levels
     // keep their state in float32 LDS and convert on the way out
     for (size_t k = 0; k < passes.size(); ++k) {
@@ -925,7 +961,7 @@ int ncn_forward_radix(const void* x, const void* xa, int in_dtype, void* y, void
             a.aux0 = last ? y32 : nullptr; a.aux1 = last ? ya32 : nullptr;
             a.W = W + ps.first * wstride;
             err = (p.path != 2) ? launch_generic(kForward, a, shape->n_head, p.grid_fwd, s)
-                                : launch_fast_forward_indexed(kForward, a, shape->n_head, p.grid_fwd, s);
+                                : run_forward_kernel(kForward, a, false, headwise, shape->n_head, p.grid_fwd, s);
         } else {
             FusedArgs a{};
             a.in0 = first ? x : y; a.in1 = first ? xa : ya; a.in_dtype = first ? in_dtype : out_dtype;
@@ -968,12 +1004,15 @@ int ncn_backward_radix(const void* y, const void* ya, int y_dtype, const void* d
         return NCN_ERR_ALIGN;
     const int path = kernel_path_for(shape, activation, alpha, m);
     if (path == 0) return NCN_ERR_UNSUPPORTED;
+    ncn_shape as_wide;
+    const bool headwise = headwise_call(shape, path, &as_wide);
+    if (headwise) shape = &as_wide;
     const Plan p = make_plan(shape, path);
     hipStream_t s = static_cast<hipStream_t>(stream);
     float* partials = static_cast<float*>(workspace);
     float* level1 = partials + (int64_t)kMaxGridX * 2 * shape->E;
     const int64_t wstride = 2 * shape->E;
-    const std::vector<RadixPass> passes = plan_radix(shape, first_level, n_levels, true, path == 2);
+    const std::vector<RadixPass> passes = plan_radix(shape, first_level, n_levels, true, path == 2 && !headwise);
     // last pass first; the first one to run reads y, ya, dy, dya, the others run in place on x_rec, xa_rec, dx, dxa
     DwReducer reducer(partials, level1, wstride, s);
     for (size_t e = 0; e < passes.size(); ++e) {
@@ -995,7 +1034,7 @@ int ncn_backward_radix(const void* y, const void* ya, int y_dtype, const void* d
             a.W = W + ps.first * wstride;
             a.dw_partials = region;
             err = (p.path != 2) ? launch_generic(kBackward, a, shape->n_head, p.grid_x, s)
-                                : launch_fast_backward_indexed(a, shape->n_head, p.grid_x, s);
+                                : run_backward_kernel(a, false, headwise, shape->n_head, p.grid_x, s);
         } else {
             FusedArgs a{};
             a.in0 = top ? y : x_rec; a.in1 = top ? ya : xa_rec; a.in_dtype = top ? y_dtype : NCN_F32;
@@ -1025,10 +1064,13 @@ int ncn_inverse_radix(const void* y, const void* ya, int in_dtype, void* x, void
     if (!aligned16(x) || !aligned16(xa) || !aligned16(y) || !aligned16(ya) || !aligned16(W)) return NCN_ERR_ALIGN;
     const int path = kernel_path_for(shape, activation, alpha, m);
     if (path == 0) return NCN_ERR_UNSUPPORTED;
+    ncn_shape as_wide;
+    const bool headwise = headwise_call(shape, path, &as_wide);
+    if (headwise) shape = &as_wide;
     const Plan p = make_plan(shape, path);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int64_t wstride = 2 * shape->E;
-    const std::vector<RadixPass> passes = plan_radix(shape, first_level, n_levels, false, path == 2);
+    const std::vector<RadixPass> passes = plan_radix(shape, first_level, n_levels, false, path == 2 && !headwise);
     for (size_t e = 0; e < passes.size(); ++e) {   // last pass first; every pass is closed: in place after the first
         const RadixPass& ps = passes[passes.size() - 1 - e];
         const bool top = (e == 0);
@@ -1041,7 +1083,7 @@ int ncn_inverse_radix(const void* y, const void* ya, int in_dtype, void* x, void
             a.out0 = x; a.out1 = xa; a.out_dtype = out_dtype;
             a.W = W + ps.first * wstride;
             err = (p.path != 2) ? launch_generic(kInverse, a, shape->n_head, p.grid_fwd, s)
-                                : launch_fast_forward_indexed(kInverse, a, shape->n_head, p.grid_fwd, s);
+                                : run_forward_kernel(kInverse, a, false, headwise, shape->n_head, p.grid_fwd, s);
         } else {
             FusedArgs a{};
             a.in0 = top ? y : x; a.in1 = top ? ya : xa; a.in_dtype = top ? in_dtype : out_dtype;

@@ -74,6 +74,20 @@ hipError_t launch_fast_backward_once(const StageArgs& a, int n_head, int grid_x,
 hipError_t launch_fast_forward_indexed(Pass pass, const StageArgs& a, int n_head, int grid_x, hipStream_t s);
 hipError_t launch_fast_backward_indexed(const StageArgs& a, int n_head, int grid_x, hipStream_t s);
 hipError_t launch_fast_backward_indexed_once(const StageArgs& a, int n_head, int grid_x, hipStream_t s);
+// Heads of one feature (ncn_headwise_kernels.h): `a` carries the geometry of E / w heads of w features, w =
+// headwise_width(E), for which the grid was planned as well; the second form honours a.table, a.radix_stride and
+// a.ctx_len.
+constexpr int kHeadwiseMaxWidth = 32;
+// adjacent one-feature heads that the lanes of a row hold together: the largest of 32, 16, 8, 4 that divides E (0: none)
+constexpr int headwise_width(int64_t E) {
+    for (int w = kHeadwiseMaxWidth; w >= 4; w /= 2)
+        if (E % w == 0) return w;
+    return 0;
+}
+hipError_t launch_headwise_forward(Pass pass, const StageArgs& a, int grid_x, hipStream_t s);
+hipError_t launch_headwise_forward_indexed(Pass pass, const StageArgs& a, int grid_x, hipStream_t s);
+hipError_t launch_headwise_backward(const StageArgs& a, int grid_x, hipStream_t s);
+hipError_t launch_headwise_backward_indexed(const StageArgs& a, int grid_x, hipStream_t s);
 hipError_t launch_generic(Pass pass, const StageArgs& a, int n_head, int grid_x, hipStream_t s);
 // Rows past the context length of their batch entry: copied through (a.ctx_len must be set).
 hipError_t launch_pass_through(Pass pass, const StageArgs& a, int64_t batch, hipStream_t s);

@@ -74,9 +74,9 @@ def _check(got, ref, x, xa, tol=TOL, n=4):
 
 
 SHAPES = [(3, 64, 32, 2, 4, 3), (2, 256, 128, 4, 16, 2), (3, 36, 20, 2, 3, 3), (5, 128, 64, 2, 8, 2),
-          (2, 64, 256, 2, 8, 2), (2, 128, 8, 2, 32, 1)]
+          (2, 64, 256, 2, 8, 2), (2, 128, 8, 2, 32, 1), (3, 64, 8, 8, 4, 3), (2, 128, 16, 16, 16, 2)]
 IDS = ["register_n4_Ec16", "register_n16_Ec32", "generic_n3_Ec10", "register_n8_Ec32", "register_n8_Ec128",
-       "register_n32_Ec4"]
+       "register_n32_Ec4", "register_n4_Ec1", "register_n16_Ec1"]
 
 
 @pytest.mark.parametrize("kind", ["stride", "radix", "random"])

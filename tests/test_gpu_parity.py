@@ -81,6 +81,15 @@ SHAPES = [
     (2, 36, 20, 2, 3, 3),      # generic kernel: n=3, Ec=10
     (1, 128, 6, 2, 64, 2),     # generic kernel: n=64, Ec=3
     (2, 14, 12, 4, 1, 2),      # generic kernel: n=1
+    (3, 40, 8, 8, 2, 3),       # one feature per head (E == n_head), four heads to a lane: n=2, 8 heads to a row, partial wave tile
+    (2, 64, 16, 16, 4, 4),     # one feature per head, n=4, 16 heads to a row
+    (2, 64, 12, 12, 8, 2),     # one feature per head, n=8, E = 3 * 4: 4 heads to a row
+    (2, 256, 128, 128, 16, 3), # one feature per head, n=16, 32 heads to a row
+    (1, 64, 32, 32, 32, 2),    # one feature per head, n=32
+    (1, 128, 4, 4, 64, 2),     # one feature per head, n=64, E = 4
+    (1, 128, 32, 32, 64, 1),   # one feature per head, n=64, 32 heads to a row: eight heads to a lane
+    (2, 32, 48, 48, 2, 2),     # one feature per head, E = 3 * 16
+    (2, 32, 6, 6, 4, 2),       # one feature per head, E not a multiple of 4: generic kernel
 ]
 
 
@@ -150,6 +159,29 @@ def test_multi_stage_calls_match_single_stage_calls(M):
     assert O.rel_err(ix, xr) < 5e-7 * amp  # two kernels, same inversion, different rounding
 
 
+@pytest.mark.parametrize("shape", [(2, 64, 16, 16, 2, 5), (2, 128, 64, 64, 4, 3)], ids=["n2_16_heads", "n4_64_heads"])
+def test_multi_stage_calls_on_one_feature_heads(M, shape):
+    """Several stages in one call on heads of one feature: the library lays them out as heads of 16 and 32 features, for
+    which small groups have multi-stage passes, and must still run them with the kernels for one-feature heads."""
+    batch, N, E, C, n, L = shape
+    alpha = 0.8
+    x, xa, Ws, dyi, dya = O.make_inputs(batch, N, E, L, n, seed=6, xa_zero=False)
+    gx, gxa, gdyi, gdya = _dev(x, xa, dyi, dya)
+    Wst = torch.stack(_dev(*Ws))
+    d = torch.float64
+    ref_y, ref_ya, ref_dx, ref_dxa, ref_dWs = O.net_autograd(x.to(d), xa.to(d), [w.to(d) for w in Ws], dyi.to(d),
+                                                             dya.to(d), alpha, n, C)
+    y, ya = M.forward_stages(gx, gxa, Wst, alpha, 0, n, C, 0, L)
+    assert O.rel_err(y, ref_y) < TOL_F32 and O.rel_err(ya, ref_ya) < TOL_F32
+    xr, xar, dx, dxa, dW = M.backward_stages(y, ya, gdyi, gdya, Wst, alpha, 0, n, C, 0, L)
+    assert O.rel_err(dx, ref_dx) < TOL_F32 and O.rel_err(dxa, ref_dxa) < TOL_F32
+    for l in range(L):
+        assert O.rel_err(dW[l], ref_dWs[l]) < TOL_F32
+    assert O.rel_err(xr, x) < TOL_F32
+    ix, ixa = M.inverse_stages(y, ya, Wst, alpha, 0, n, C, 0, L)
+    assert O.rel_err(ix, x) < TOL_F32 and O.rel_err(ixa, xa) < TOL_F32
+
+
 def test_dya_none_equals_zeros(M):
     batch, N, E, C, n = 2, 64, 32, 4, 4
     x, xa, Ws, dyi, _ = O.make_inputs(batch, N, E, 1, n, seed=3)
@@ -161,8 +193,8 @@ def test_dya_none_equals_zeros(M):
         assert torch.equal(u, v)
 
 
-@pytest.mark.parametrize("shape", [(2, 32, 16, 2, 4, 3), (2, 128, 128, 4, 16, 2), (2, 36, 20, 2, 3, 3)],
-                         ids=["register_n4_Ec8", "register_n16_Ec32", "generic_n3_Ec10"])
+@pytest.mark.parametrize("shape", [(2, 32, 16, 2, 4, 3), (2, 128, 128, 4, 16, 2), (2, 36, 20, 2, 3, 3), (2, 64, 16, 16, 8, 2)],
+                         ids=["register_n4_Ec8", "register_n16_Ec32", "generic_n3_Ec10", "register_n8_Ec1"])
 @pytest.mark.parametrize("act", [1, 2, -1, 3], ids=["relu", "sigmoid", "linear", "leaky_relu"])
 def test_other_activations_vs_oracle(M, act, shape):
     """relu / sigmoid / linear (codes of ncn_fwd_cuda_kernel.cu:86-95) and the Triton kernels' leaky relu
@@ -200,13 +232,14 @@ def test_other_activations_vs_oracle(M, act, shape):
         assert O.rel_err(dWs[l], ref_dWs[l]) < TOL_F32
 
 
+@pytest.mark.parametrize("heads", [4, 128], ids=["Ec32", "Ec1"])
 @pytest.mark.parametrize("save", ["two_bf16_planes", "float32_copies"])
-def test_bf16_storage_fp32_arithmetic(M, save):
+def test_bf16_storage_fp32_arithmetic(M, save, heads):
     """bf16 activations and weights, float32 arithmetic: compared with the oracle run in float32 on the
     same bf16-rounded inputs.  Tolerance 2e-2 relative.  The saved outputs are the bf16 outputs plus what their
     rounding took away (a second bf16 plane), or float32 copies; the two reconstructions must agree to the 16 bits the
     planes hold."""
-    batch, N, E, C, n, L = 4, 256, 128, 4, 16, 3
+    batch, N, E, C, n, L = 4, 256, 128, heads, 16, 3
     alpha = 0.9
     x, xa, Ws, dyi, dya = O.make_inputs(batch, N, E, L, n, seed=0, xa_zero=True, dtype=torch.bfloat16)
     f = torch.float32

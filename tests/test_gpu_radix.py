@@ -42,6 +42,8 @@ CASES = [
     (2, 512, 32, 2, 8, 0, 3),      # n = 8: no LDS passes, closed-form positions in the one-stage register kernels
     (2, 81, 10, 2, 3, 0, 4),       # n = 3, head width 5: generic kernel
     (2, 128, 256, 2, 2, 2, 3),     # head width 128: register kernels, one level per launch
+    (2, 64, 16, 16, 2, 0, 6),      # one feature per head: register kernels, four heads to a lane, one level per launch
+    (2, 512, 8, 8, 8, 0, 3),       # the same at n = 8
 ]
 
 

@@ -68,6 +68,11 @@ def test_kernel_path_and_workspace(lib):
     assert h.ncn_kernel_path(ctypes.byref(_shape(lib, 1, 256, 32, 4, 2))) == 2        # config 1 (Ec = 8)
     assert h.ncn_kernel_path(ctypes.byref(_shape(lib, 1, 24, 10, 2, 3))) == 1         # n = 3, Ec = 5: generic
     assert h.ncn_kernel_path(ctypes.byref(_shape(lib, 1, 256, 32, 4, 128))) == 0
+    # one feature per head: register kernels (four heads to a lane) when E is a multiple of 4 and n_cache a power of two
+    assert h.ncn_kernel_path(ctypes.byref(_shape(lib, 2, 256, 128, 128, 16))) == 2
+    assert h.ncn_kernel_path_scalars(ctypes.byref(_shape(lib, 2, 256, 128, 128, 16)), 1e-4, 0.9) == 1
+    assert h.ncn_kernel_path(ctypes.byref(_shape(lib, 2, 256, 6, 6, 16))) == 1
+    assert h.ncn_kernel_path(ctypes.byref(_shape(lib, 2, 240, 128, 128, 3))) == 1
     ws = h.ncn_workspace_bytes(ctypes.byref(_shape(lib, 128, 4096, 128, 4, 16)))
     assert ws > 0 and ws % 16 == 0 and ws < (1 << 25)
     assert h.ncn_workspace_bytes(ctypes.byref(_shape(lib, 1, 65, 32, 4, 4))) == 0

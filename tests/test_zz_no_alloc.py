@@ -69,7 +69,8 @@ def test_backward_static_matches_backward_on_two_calls_in_a_row():
         assert torch.equal(u, v)                         # dx, dxa, x_rec, xa_rec do not depend on the grid
     assert O.rel_err(b[4], a[4]) < 1e-5 and torch.isfinite(b[4]).all()   # the same terms summed over fewer partial rows
     # the capped grid is rounded to whole multiples of n_head waves: three heads (blocks in threes) and two
-    for shape5 in ((40, 4096, 96, 3, 16), (40, 4096, 64, 2, 16)):
+    # (and one feature per head: 16 lanes' worth of heads, waves in sixteens)
+    for shape5 in ((40, 4096, 96, 3, 16), (40, 4096, 64, 2, 16), (40, 4096, 64, 64, 16)):
         a, b = _call_both(lib, _lib, shape5, 1, seed=6)
         for u, v in zip(a[:4], b[:4]):
             assert torch.equal(u, v)
