@@ -39,8 +39,25 @@ def _cases(seed, count, acts=None):
     return out
 
 
-# the last 16: relu and leaky relu (codes 1 and 3) on inputs that stay away from the kink
-CASES = _cases(2024, 40) + _cases(7, 40) + _cases(11, 16, acts=(1, 3))
+def _one_feature_cases(seed, count):
+    """Heads of one feature (E == n_head) on the group sizes and widths their register kernels exist for, and some
+    they do not (E not a multiple of 4, n_cache not a power of two: generic kernels)."""
+    rng = random.Random(seed)
+    out = []
+    while len(out) < count:
+        n = rng.choice([2, 2, 4, 4, 8, 16, 16, 32, 64, 3])
+        E = rng.choice([4, 8, 12, 16, 20, 24, 32, 48, 64, 96, 128, 6])
+        groups = rng.choice([1, 2, 3, 4, 6, 8, 16, 24, 32])
+        if n * groups * E > 1 << 16:
+            continue
+        batch = rng.choice([1, 2, 3, 5])
+        L = rng.randint(1, 4 if n >= 8 else 6)
+        out.append((batch, n * groups, E, E, n, rng.choice([0, 0, 1, 3]), L, rng.choice([0, 0, 0, 2, -1, 3])))
+    return out
+
+
+# 16 of them: relu and leaky relu (codes 1 and 3) on inputs that stay away from the kink; the last 24: one feature per head
+CASES = _cases(2024, 40) + _cases(7, 40) + _cases(11, 16, acts=(1, 3)) + _one_feature_cases(5, 24)
 
 
 @pytest.mark.parametrize("case", CASES, ids=lambda c: "b%d_N%d_E%d_C%d_n%d_s%d_L%d_a%d" % c)
