@@ -433,7 +433,8 @@ def main():
     version = lib.ncn_version().decode()
     import ctypes
     on_register_kernels = lib.ncn_kernel_path(ctypes.byref(M._lib.NcnShape(batch, N, E, C, n))) == 2
-    kernel = ((f"headwise_backward_kernel<{n}> (one feature per head, four heads to a lane)" if on_register_kernels and C == E else
+    wide = next((w for w in (32, 16, 8, 4) if E % w == 0), 0)   # adjacent one-feature heads that a row's lanes hold
+    kernel = ((f"headwise_backward_kernel<{n},{wide}> (one feature per head)" if on_register_kernels and C == E else
                f"stage_backward_kernel<{n},{E // C}>" if on_register_kernels else
                f"generic_backward_kernel (n_cache {n}, heads of {E // C}: no register-tile build)") +
               (" (indexed build)" if tables else "") if not lds_passes else

@@ -323,8 +323,9 @@ int ncn_plan_passes(const ncn_shape* shape, int first_stage, int n_stages, int a
 /* 2: hand-tuned register kernel, 1: generic LDS kernel, 0: not supported (n_cache > 64, or the
  * head width does not fit the generic kernel's LDS).  Register kernels exist for n_cache 2, 4, 8, 16, 32, 64 with
  * head widths 4 .. 128 (powers of two; 128 up to n_cache 16, 64 up to 32), and for heads of one feature
- * (E == n_head, the recurrence on rows of scalars) when E is a multiple of 4: those run one launch per stage under
- * every grouping (no multi-stage passes).  No reference counterpart. */
+ * (E == n_head, the recurrence on rows of scalars) when E is a multiple of 4: the library lays those out as heads of
+ * 32, 16, 8 or 4 adjacent ones (the largest that divides E), with the multi-stage passes of such heads for n_cache 2
+ * and 4 when E is a multiple of 8.  No reference counterpart. */
 int ncn_kernel_path(const ncn_shape* shape);
 
 /* The same for a call with these scalars: the register kernels carry their state times alpha and 1 - m, so values

@@ -24,7 +24,8 @@ BUILD_DIR = os.path.join(PKG_DIR, "build")
 LOCK_PATH = os.path.join(PKG_DIR, ".build.lock")
 ID_SOURCE = "ncn_build_id.hip"
 SOURCES = ["ncn_api.hip", "ncn_fwd.hip", "ncn_bwd.hip", "ncn_bwd_once.hip", "ncn_fwd_indexed.hip", "ncn_bwd_indexed.hip", "ncn_bwd_indexed_once.hip",
-           "ncn_headwise.hip", "ncn_headwise_indexed.hip", "ncn_headwise_bwd.hip", "ncn_headwise_bwd_indexed.hip", "ncn_generic.hip", "ncn_fused.hip", "ncn_fused_radix.hip", "ncn_fused_lengths.hip", "ncn_probe.hip", ID_SOURCE]
+           "ncn_headwise.hip", "ncn_headwise_indexed.hip", "ncn_headwise_bwd.hip", "ncn_headwise_bwd_indexed.hip", "ncn_generic.hip", "ncn_fused.hip", "ncn_fused_radix.hip", "ncn_fused_lengths.hip", "ncn_fused_headwise.hip", "ncn_fused_headwise_lengths.hip",
+           "ncn_fused_radix_headwise.hip", "ncn_probe.hip", ID_SOURCE]
 # packed-fp32 VALU instructions are switched off for device code on purpose (flag is device-only;
 # the host pass prints a harmless "not a recognized feature" note).
 HIPCC_FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17",
@@ -38,6 +39,8 @@ ID_MARKER = "NCN_BUILD_ID="    # the library holds this marker followed by the 1
 # tiles is bound by issue slots and does not care, its form without the loop gains 2.5 % at 16 rows per group.
 MAX_ILP = ["-mllvm", "-amdgpu-sched-strategy=max-ilp"]
 EXTRA_FLAGS = {"ncn_fused.hip": MAX_ILP, "ncn_fused_radix.hip": MAX_ILP, "ncn_fused_lengths.hip": MAX_ILP,
+               "ncn_fused_headwise.hip": MAX_ILP, "ncn_fused_headwise_lengths.hip": MAX_ILP,
+               "ncn_fused_radix_headwise.hip": MAX_ILP,
                "ncn_fwd.hip": MAX_ILP, "ncn_fwd_indexed.hip": MAX_ILP, "ncn_bwd_indexed.hip": MAX_ILP,
                "ncn_bwd_once.hip": MAX_ILP, "ncn_bwd_indexed_once.hip": MAX_ILP,
                "ncn_headwise.hip": MAX_ILP, "ncn_headwise_indexed.hip": MAX_ILP, "ncn_headwise_bwd.hip": MAX_ILP,

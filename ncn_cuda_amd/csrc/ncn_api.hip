@@ -245,6 +245,11 @@ bool headwise_call(const ncn_shape* sh, int path, ncn_shape* as_wide) {
     return true;
 }
 
+// the shape that the passes of a call on `sh` are planned for (the queries take no scalars: register kernels assumed)
+const ncn_shape* planning_shape(const ncn_shape* sh, ncn_shape* as_wide) {
+    return headwise_call(sh, 2, as_wide) ? as_wide : sh;
+}
+
 // one stage on the register kernels: the plain builds know the stride permutation only, the others read the
 // launch's table, radix level and context lengths
 hipError_t run_forward_kernel(Pass pass, const StageArgs& a, bool plain, bool headwise, int n_head, int grid,
@@ -387,12 +392,14 @@ hipError_t static_scratch(float** out) {
 
 extern "C" {
 
-const char* ncn_version(void) { return "0.14"; }
+const char* ncn_version(void) { return "0.15"; }
 
 int ncn_plan_passes(const ncn_shape* shape, int first_stage, int n_stages, int activation, int backward, int32_t* out,
                     int max_passes) {
     int rc = check_shape(shape, first_stage, n_stages, activation);
     if (rc != NCN_OK) return rc;
+    ncn_shape as_wide;
+    shape = planning_shape(shape, &as_wide);
     const std::vector<FusedPass> passes = multi_stage_plan(shape, first_stage, n_stages, activation, backward != 0);
     int k = 0;
     for (const FusedPass& p : passes) {
@@ -447,6 +454,8 @@ size_t ncn_workspace_bytes(const ncn_shape* shape) {
 
 size_t ncn_workspace_bytes_stages(const ncn_shape* shape, int first_stage, int n_stages, int activation, int backward) {
     if (check_shape(shape, first_stage, n_stages, activation) != NCN_OK) return 0;
+    ncn_shape as_wide;
+    shape = planning_shape(shape, &as_wide);
     const std::vector<FusedPass> passes = multi_stage_plan(shape, first_stage, n_stages, activation, backward != 0);
     const size_t base = !backward ? 0 : passes.empty() ? base_workspace_bytes(shape)
                                                         : partial_buffer_bytes(shape, fused_rows_wanted(shape, passes));
@@ -483,8 +492,7 @@ static int forward_impl(const void* x, const void* xa, int in_dtype, void* y, vo
 
     // several stages: LDS-resident passes when the shape allows and the buffers permit the ping-pong
     std::vector<FusedPass> passes;
-    // (heads of one feature have no multi-stage kernels: one launch per stage)
-    if (grouping.permutation() && !headwise) passes = multi_stage_plan(shape, first_stage, n_stages, activation, false, path);
+    if (grouping.permutation()) passes = multi_stage_plan(shape, first_stage, n_stages, activation, false, path);
     const size_t np = passes.size();
     // one stage of the range with the one-stage kernel (and, with lengths, the launch for the rows past them)
     auto run_stage = [&](int k, const void* i0, const void* i1, int i_dtype, void* o0, void* o1, int o_dtype,
@@ -526,7 +534,7 @@ static int forward_impl(const void* x, const void* xa, int in_dtype, void* y, vo
                 a.W = W + ps.first * wstride;
                 a.ctx_len = grouping.ctx_len;
                 fill_step_table(a.tab, shape->n_cache, alpha, m, activation);
-                err = launch_fused(kForward, a, shape, ps, s);
+                err = launch_fused(kForward, a, shape, ps, s, kMaxGridX, headwise);
             }
             if (err != hipSuccess) return (int)err;
         }
@@ -557,7 +565,7 @@ static int forward_impl(const void* x, const void* xa, int in_dtype, void* y, vo
                 a.W = W + ps.first * wstride;
                 a.ctx_len = grouping.ctx_len;
                 fill_step_table(a.tab, shape->n_cache, alpha, m, activation);
-                err = launch_fused(kForward, a, shape, ps, s);
+                err = launch_fused(kForward, a, shape, ps, s, kMaxGridX, headwise);
             }
             if (err != hipSuccess) return (int)err;
             cur0 = d0; cur1 = d1; cur_dtype = d_dtype;
@@ -609,7 +617,7 @@ static int inverse_impl(const void* y, const void* ya, int in_dtype, void* x, vo
     // first pass to run goes from y, ya to x, xa and the others work in place on x, xa, which a halo pass must not,
     // so the stages of such a pass are undone by one-stage launches (closed passes and one-stage launches may).
     std::vector<FusedPass> passes;
-    if (grouping.permutation() && !headwise && (out_dtype == NCN_F32 || n_stages == 1))
+    if (grouping.permutation() && (out_dtype == NCN_F32 || n_stages == 1))
         passes = multi_stage_plan(shape, first_stage, n_stages, activation, false, path);
     auto run_stage = [&](int k, const void* i0, const void* i1, int i_dtype, void* o0, void* o1, int o_dtype) -> hipError_t {
         StageArgs a{};
@@ -650,7 +658,7 @@ static int inverse_impl(const void* y, const void* ya, int in_dtype, void* x, vo
                 a.W = W + ps.first * wstride;
                 a.ctx_len = grouping.ctx_len;
                 fill_step_table(a.tab, shape->n_cache, alpha, m, activation);
-                err = launch_fused(kInverse, a, shape, ps, s);
+                err = launch_fused(kInverse, a, shape, ps, s, kMaxGridX, headwise);
             }
             if (err != hipSuccess) return (int)err;
             cur0 = d0; cur1 = d1; cur_dtype = NCN_F32;
@@ -678,7 +686,7 @@ static int inverse_impl(const void* y, const void* ya, int in_dtype, void* x, vo
                 a.W = W + ps.first * wstride;
                 a.ctx_len = grouping.ctx_len;
                 fill_step_table(a.tab, shape->n_cache, alpha, m, activation);
-                hipError_t err = launch_fused(kInverse, a, shape, ps, s);
+                hipError_t err = launch_fused(kInverse, a, shape, ps, s, kMaxGridX, headwise);
                 if (err != hipSuccess) return (int)err;
             }
         }
@@ -742,7 +750,7 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
     // several stages: LDS-resident passes, last pass of the range first; the state ping-pongs between the
     // output arrays and four float32 arrays behind the dW scratch (their grids count on kMaxGridX partial rows)
     std::vector<FusedPass> passes;
-    if (grouping.permutation() && !headwise && row_cap == kMaxGridX)
+    if (grouping.permutation() && row_cap == kMaxGridX)
         passes = multi_stage_plan(shape, first_stage, n_stages, activation, true, path);
     const size_t np = passes.size();
     bool fused_ok = np > 0;
@@ -806,7 +814,7 @@ static int backward_impl(const void* y, const void* ya, int y_dtype, const void*
                 a.dw_partials = region;
                 a.ctx_len = grouping.ctx_len;
                 fill_step_table(a.tab, shape->n_cache, alpha, m, activation);
-                err = launch_fused(kBackward, a, shape, ps, s, fused_cap);
+                err = launch_fused(kBackward, a, shape, ps, s, fused_cap, headwise);
             }
             if (err != hipSuccess) return (int)err;
             reducer.add(region, rows, ps.count, dW + ps.first * wstride);
@@ -945,7 +953,7 @@ int ncn_forward_radix(const void* x, const void* xa, int in_dtype, void* y, void
     const Plan p = make_plan(shape, path);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int64_t wstride = 2 * shape->E;
-    const std::vector<RadixPass> passes = plan_radix(shape, first_level, n_levels, false, path == 2 && !headwise);
+    const std::vector<RadixPass> passes = plan_radix(shape, first_level, n_levels, false, path == 2);
     // every pass is closed: the first reads x, xa and the later ones run in place on y, ya; passes of several levels
     // keep their state in float32 LDS and convert on the way out
     for (size_t k = 0; k < passes.size(); ++k) {
@@ -969,7 +977,7 @@ int ncn_forward_radix(const void* x, const void* xa, int in_dtype, void* y, void
             a.aux0 = last ? y32 : nullptr; a.aux1 = last ? ya32 : nullptr;
             a.W = W + ps.first * wstride;
             fill_step_table(a.tab, shape->n_cache, alpha, m, activation);
-            err = launch_fused_radix(kForward, a, shape, ps, s);
+            err = launch_fused_radix(kForward, a, shape, ps, s, headwise);
         }
         if (err != hipSuccess) return (int)err;
     }
@@ -1012,7 +1020,7 @@ int ncn_backward_radix(const void* y, const void* ya, int y_dtype, const void* d
     float* partials = static_cast<float*>(workspace);
     float* level1 = partials + (int64_t)kMaxGridX * 2 * shape->E;
     const int64_t wstride = 2 * shape->E;
-    const std::vector<RadixPass> passes = plan_radix(shape, first_level, n_levels, true, path == 2 && !headwise);
+    const std::vector<RadixPass> passes = plan_radix(shape, first_level, n_levels, true, path == 2);
     // last pass first; the first one to run reads y, ya, dy, dya, the others run in place on x_rec, xa_rec, dx, dxa
     DwReducer reducer(partials, level1, wstride, s);
     for (size_t e = 0; e < passes.size(); ++e) {
@@ -1044,7 +1052,7 @@ int ncn_backward_radix(const void* y, const void* ya, int y_dtype, const void* d
             a.W = W + ps.first * wstride;
             a.dw_partials = region;
             fill_step_table(a.tab, shape->n_cache, alpha, m, activation);
-            err = launch_fused_radix(kBackward, a, shape, ps, s);
+            err = launch_fused_radix(kBackward, a, shape, ps, s, headwise);
         }
         if (err != hipSuccess) return (int)err;
         reducer.add(region, rows, ps.count, dW + ps.first * wstride);
@@ -1070,7 +1078,7 @@ int ncn_inverse_radix(const void* y, const void* ya, int in_dtype, void* x, void
     const Plan p = make_plan(shape, path);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int64_t wstride = 2 * shape->E;
-    const std::vector<RadixPass> passes = plan_radix(shape, first_level, n_levels, false, path == 2 && !headwise);
+    const std::vector<RadixPass> passes = plan_radix(shape, first_level, n_levels, false, path == 2);
     for (size_t e = 0; e < passes.size(); ++e) {   // last pass first; every pass is closed: in place after the first
         const RadixPass& ps = passes[passes.size() - 1 - e];
         const bool top = (e == 0);
@@ -1090,7 +1098,7 @@ int ncn_inverse_radix(const void* y, const void* ya, int in_dtype, void* x, void
             a.out0 = x; a.out1 = xa; a.out_dtype = out_dtype;
             a.W = W + ps.first * wstride;
             fill_step_table(a.tab, shape->n_cache, alpha, m, activation);
-            err = launch_fused_radix(kInverse, a, shape, ps, s);
+            err = launch_fused_radix(kInverse, a, shape, ps, s, headwise);
         }
         if (err != hipSuccess) return (int)err;
     }
@@ -1103,6 +1111,8 @@ int ncn_plan_radix(const ncn_shape* shape, int first_level, int n_levels, int ac
     if (rc != NCN_OK) return rc;
     rc = check_radix(shape, first_level, n_levels);
     if (rc != NCN_OK) return rc;
+    ncn_shape as_wide;
+    shape = planning_shape(shape, &as_wide);
     const std::vector<RadixPass> passes = plan_radix(shape, first_level, n_levels, backward != 0);
     int k = 0;
     for (const RadixPass& p : passes) {

@@ -3,9 +3,7 @@
 #include <cmath>
 #include <vector>
 
-#include "ncn_fused_kernels.h"
-#include "ncn_fused_pair_kernels.h"
-#include "ncn_launch.h"
+#include "ncn_fused_dispatch.h"
 
 namespace ncn {
 
@@ -187,57 +185,6 @@ std::vector<FusedPass> plan_fused(const ncn_shape* sh, int first, int count, boo
     return passes;
 }
 
-template <int NC, int EC>
-static hipError_t launch_fused_t(Pass pass, const FusedArgs& a, int grid, size_t lds, hipStream_t s) {
-    const bool backward = pass == kBackward;
-    constexpr TileShape t = fast_tile(NC, EC);
-    static_assert(t.r != 0, "multi-stage shapes must be one-stage shapes too");
-    hipError_t err;
-    const bool tanh_only = a.tab.activation == NCN_ACT_TANH;
-    if constexpr (NC == 2) {
-        static_assert(t.r == 2, "the two-row kernels keep both rows of a group in one lane");
-        if (!backward && (uint32_t)grid != a.total_items) return hipErrorInvalidConfiguration;   // one window each
-        if (backward) {
-            // a workgroup per window when the dW scratch has the rows for it, else workgroups that loop over windows
-            const bool loop = (uint32_t)grid < a.total_items;
-            auto k = tanh_only ? (loop ? pair_backward_kernel<EC, true, false, true> : pair_backward_kernel<EC, true, false, false>)
-                               : (loop ? pair_backward_kernel<EC, false, false, true> : pair_backward_kernel<EC, false, false, false>);
-            err = ensure_dynamic_lds(reinterpret_cast<const void*>(k), lds);
-            if (err != hipSuccess) return err;
-            hipLaunchKernelGGL(k, dim3(grid), dim3(64 * kPairWavesBwd), lds, s, a);
-        } else if (pass == kInverse) {
-            auto k = tanh_only ? pair_forward_kernel<EC, true, true> : pair_forward_kernel<EC, false, true>;
-            err = ensure_dynamic_lds(reinterpret_cast<const void*>(k), lds);
-            if (err != hipSuccess) return err;
-            hipLaunchKernelGGL(k, dim3(grid), dim3(64 * kFusedWavesFwd), lds, s, a);
-        } else {
-            auto k = tanh_only ? pair_forward_kernel<EC, true> : pair_forward_kernel<EC, false>;
-            err = ensure_dynamic_lds(reinterpret_cast<const void*>(k), lds);
-            if (err != hipSuccess) return err;
-            hipLaunchKernelGGL(k, dim3(grid), dim3(64 * kFusedWavesFwd), lds, s, a);
-        }
-        return hipGetLastError();
-    } else
-    if (backward) {
-        auto k = tanh_only ? fused_backward_kernel<NC, EC, t.r, t.f, true> : fused_backward_kernel<NC, EC, t.r, t.f, false>;
-        err = ensure_dynamic_lds(reinterpret_cast<const void*>(k), lds);
-        if (err != hipSuccess) return err;
-        hipLaunchKernelGGL(k, dim3(grid), dim3(64 * kFusedWavesBwd), lds, s, a);
-    } else if (pass == kInverse) {
-        auto k = tanh_only ? fused_forward_kernel<NC, EC, t.r, t.f, true, false, true>
-                           : fused_forward_kernel<NC, EC, t.r, t.f, false, false, true>;
-        err = ensure_dynamic_lds(reinterpret_cast<const void*>(k), lds);
-        if (err != hipSuccess) return err;
-        hipLaunchKernelGGL(k, dim3(grid), dim3(64 * kFusedWavesFwd), lds, s, a);
-    } else {
-        auto k = tanh_only ? fused_forward_kernel<NC, EC, t.r, t.f, true> : fused_forward_kernel<NC, EC, t.r, t.f, false>;
-        err = ensure_dynamic_lds(reinterpret_cast<const void*>(k), lds);
-        if (err != hipSuccess) return err;
-        hipLaunchKernelGGL(k, dim3(grid), dim3(64 * kFusedWavesFwd), lds, s, a);
-    }
-    return hipGetLastError();
-}
-
 int64_t fused_items(const ncn_shape* sh, const FusedPass& p) {
     return sh->batch * (int64_t)p.class_groups * p.tiles_per_ring * sh->n_head;
 }
@@ -257,7 +204,8 @@ int fused_grid(const ncn_shape* sh, const FusedPass& p, bool backward, int row_c
     return (int)g;
 }
 
-hipError_t launch_fused(Pass pass, FusedArgs& a, const ncn_shape* sh, const FusedPass& p, hipStream_t s, int row_cap) {
+hipError_t launch_fused(Pass pass, FusedArgs& a, const ncn_shape* sh, const FusedPass& p, hipStream_t s, int row_cap,
+                        bool headwise) {
     const bool backward = pass == kBackward;
     const int nc = sh->n_cache, ec = (int)(sh->E / sh->n_head);
     a.N = sh->N;
@@ -279,12 +227,9 @@ hipError_t launch_fused(Pass pass, FusedArgs& a, const ncn_shape* sh, const Fuse
     a.scale_up = (float)std::pow((double)a.tab.m, -(double)(nc * p.count));
     const int grid = fused_grid(sh, p, backward, row_cap);
     const size_t lds = fused_lds_bytes(nc, ec, backward, p.window, p.count);
+    if (headwise) return launch_fused_headwise(pass, a, nc, ec, grid, lds, s);
     if (a.ctx_len) return launch_fused_lengths(pass, a, nc, ec, grid, lds, s);
-#define NCN_CASE(NC, EC) \
-    if (nc == NC && ec == EC) return launch_fused_t<NC, EC>(pass, a, grid, lds, s);
-    NCN_FOR_EACH_FUSED_CONFIG(NCN_CASE)
-#undef NCN_CASE
-    return hipErrorInvalidConfiguration;
+    return launch_fused_shape<false, false, false>(pass, a, nc, ec, grid, lds, s);
 }
 
 }  // namespace ncn

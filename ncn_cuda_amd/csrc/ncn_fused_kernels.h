@@ -33,7 +33,7 @@
 // row of digit string d is d itself, and level a+j pairs the rows whose d differ in digit j.  (n_cache 2 and 4
 // only: every size below is a power of two and the digit arithmetic is shifts.)
 #pragma once
-#include "ncn_stage_kernels.h"
+#include "ncn_headwise_kernels.h"
 
 namespace ncn {
 
@@ -325,7 +325,10 @@ __device__ __forceinline__ void fused_load_weights(const FusedArgs& A, int head,
 // INVERSE: the same kernel undoes the stages instead, last one first (in0, in1 = y, ya; out0, out1 = x, xa).
 // LENGTHS: one context length per batch entry; the group a length cuts runs its live steps on its live rows, rows
 // past the length stay in LDS as they came (a row may be live in one stage of the pass and past the length in another).
-template <int NC, int EC, int R, int F, bool TANH_ONLY, bool RADIX = false, bool INVERSE = false, bool LENGTHS = false>
+// HEADWISE: heads of one feature laid out as heads of EC adjacent ones (ncn_headwise_kernels.h): the same windows, tiles
+// and weights, the step code without sums across a row's lanes.
+template <int NC, int EC, int R, int F, bool TANH_ONLY, bool RADIX = false, bool INVERSE = false, bool LENGTHS = false,
+          bool HEADWISE = false>
 __global__ void __launch_bounds__(64 * kFusedWavesFwd) fused_forward_kernel(const FusedArgs A) {
     static_assert(!(RADIX && LENGTHS), "context lengths go with the stride permutation");
     constexpr int NW = kFusedWavesFwd;
@@ -381,8 +384,13 @@ __global__ void __launch_bounds__(64 * kFusedWavesFwd) fused_forward_kernel(cons
                     lds_load_frag<F>(as + row[rr], a[rr]);
                 }
                 const int live = !LENGTHS ? NC : valid ? fused_live_rows<NC>(A, it, qg, len) : 0;
-                if (INVERSE) inverse_core<NC, EC, R, F, TANH_ONLY, LENGTHS, true>(x, a, wi, wj, A.tab, lane, slots, live);
-                else forward_core<NC, EC, R, F, TANH_ONLY, LENGTHS, true>(x, a, wi, wj, A.tab, lane, slots, live);
+                if constexpr (HEADWISE) {
+                    if (INVERSE) headwise_inverse_core<NC, EC, R, F, TANH_ONLY, LENGTHS, true>(x, a, wi, wj, A.tab, lane, slots, live);
+                    else headwise_forward_core<NC, EC, R, F, TANH_ONLY, LENGTHS, true>(x, a, wi, wj, A.tab, lane, slots, live);
+                } else {
+                    if (INVERSE) inverse_core<NC, EC, R, F, TANH_ONLY, LENGTHS, true>(x, a, wi, wj, A.tab, lane, slots, live);
+                    else forward_core<NC, EC, R, F, TANH_ONLY, LENGTHS, true>(x, a, wi, wj, A.tab, lane, slots, live);
+                }
                 if (valid) {
 #pragma unroll
                     for (int rr = 0; rr < R; ++rr) {
@@ -402,7 +410,7 @@ __global__ void __launch_bounds__(64 * kFusedWavesFwd) fused_forward_kernel(cons
     }
 }
 
-template <int NC, int EC, int R, int F, bool TANH_ONLY, bool RADIX = false, bool LENGTHS = false>
+template <int NC, int EC, int R, int F, bool TANH_ONLY, bool RADIX = false, bool LENGTHS = false, bool HEADWISE = false>
 __global__ void __launch_bounds__(64 * kFusedWavesBwd, TANH_ONLY ? (R * F <= 8 ? 4 : 2) : 1) fused_backward_kernel(const FusedArgs A) {
     static_assert(!(RADIX && LENGTHS), "context lengths go with the stride permutation");
     constexpr int NW = kFusedWavesBwd;
@@ -516,8 +524,12 @@ __global__ void __launch_bounds__(64 * kFusedWavesBwd, TANH_ONLY ? (R * F <= 8 ?
                         }
                     }
                 }
-                backward_core<NC, EC, R, F, true, TANH_ONLY, LENGTHS, true>(Y, B, G, P, wi, wj, dwi, dwj, own, A.tab,
-                                                                          (A.n_stages - 1 - st) * NC, lane, slots, live);
+                if constexpr (HEADWISE)
+                    headwise_backward_core<NC, EC, R, F, true, TANH_ONLY, LENGTHS, true>(
+                        Y, B, G, P, wi, wj, dwi, dwj, own, A.tab, (A.n_stages - 1 - st) * NC, lane, slots, live);
+                else
+                    backward_core<NC, EC, R, F, true, TANH_ONLY, LENGTHS, true>(Y, B, G, P, wi, wj, dwi, dwj, own, A.tab,
+                                                                              (A.n_stages - 1 - st) * NC, lane, slots, live);
                 if (valid) {
 #pragma unroll
                     for (int rr = 0; rr < R; ++rr) {

@@ -123,7 +123,7 @@ __device__ __forceinline__ void pair_lds_store(float* row, int fl, const float (
 }
 
 // forward, and with INVERSE the same passes undone (stages last to first)
-template <int EC, bool TANH_ONLY, bool INVERSE = false, bool LENGTHS = false>
+template <int EC, bool TANH_ONLY, bool INVERSE = false, bool LENGTHS = false, bool HEADWISE = false>
 __global__ void __launch_bounds__(64 * kFusedWavesFwd, NCN_PAIR_FWD_WAVES) pair_forward_kernel(const FusedArgs A) {
     using S = PairShape<EC>;
     constexpr int NC = 2, R = 2, F = S::F, H = S::H, NW = kFusedWavesFwd, KT = pair_tiles<EC>(false);
@@ -195,8 +195,13 @@ __global__ void __launch_bounds__(64 * kFusedWavesFwd, NCN_PAIR_FWD_WAVES) pair_
                     pair_lds_load<EC>(xs1 + row1, fl, x[k][1]);
                     pair_lds_load<EC>(as1 + row1, fl, a[k][1]);
                     const int live = !LENGTHS ? NC : fused_live_rows<NC>(A, it, q, len);
-                    if (INVERSE) inverse_core<NC, EC, R, F, TANH_ONLY, LENGTHS, true>(x[k], a[k], wi, wj, A.tab, lane, nullptr, live);
-                    else forward_core<NC, EC, R, F, TANH_ONLY, LENGTHS, true>(x[k], a[k], wi, wj, A.tab, lane, nullptr, live);
+                    if constexpr (HEADWISE) {
+                        if (INVERSE) headwise_inverse_core<NC, EC, R, F, TANH_ONLY, LENGTHS, true>(x[k], a[k], wi, wj, A.tab, lane, nullptr, live);
+                        else headwise_forward_core<NC, EC, R, F, TANH_ONLY, LENGTHS, true>(x[k], a[k], wi, wj, A.tab, lane, nullptr, live);
+                    } else {
+                        if (INVERSE) inverse_core<NC, EC, R, F, TANH_ONLY, LENGTHS, true>(x[k], a[k], wi, wj, A.tab, lane, nullptr, live);
+                        else forward_core<NC, EC, R, F, TANH_ONLY, LENGTHS, true>(x[k], a[k], wi, wj, A.tab, lane, nullptr, live);
+                    }
                     if (!LENGTHS || live > 1) {
                         pair_lds_store<EC>(xs1 + row1, fl, x[k][1]);
                         pair_lds_store<EC>(as1 + row1, fl, a[k][1]);
@@ -305,7 +310,7 @@ __device__ __forceinline__ int pair_scatter_sum(float (&v)[NV], int lane) {
     return first;
 }
 
-template <int EC, bool TANH_ONLY, bool LENGTHS = false, bool LOOP = false>
+template <int EC, bool TANH_ONLY, bool LENGTHS = false, bool LOOP = false, bool HEADWISE = false>
 __global__ void __launch_bounds__(64 * kPairWavesBwd, TANH_ONLY ? NCN_PAIR_BWD_WAVES : 1) pair_backward_kernel(const FusedArgs A) {
     using S = PairShape<EC>;
     constexpr int NC = 2, R = 2, F = S::F, H = S::H, NW = kPairWavesBwd, KT = pair_tiles<EC>(true);
@@ -448,8 +453,12 @@ __global__ void __launch_bounds__(64 * kPairWavesBwd, TANH_ONLY ? NCN_PAIR_BWD_W
 #pragma unroll
                         for (int f = 0; f < F; ++f) Y[k][1][f] = B[k][1][f] = G[k][1][f] = P[k][1][f] = 0.f;
                     }
-                    backward_core<NC, EC, R, F, true, TANH_ONLY, LENGTHS, true, false>(
-                        Y[k], B[k], G[k], P[k], wi, wj, dwi, dwj, own, A.tab, (A.n_stages - 1 - st) * NC, lane, nullptr, live);
+                    if constexpr (HEADWISE)
+                        headwise_backward_core<NC, EC, R, F, true, TANH_ONLY, LENGTHS, true, false>(
+                            Y[k], B[k], G[k], P[k], wi, wj, dwi, dwj, own, A.tab, (A.n_stages - 1 - st) * NC, lane, nullptr, live);
+                    else
+                        backward_core<NC, EC, R, F, true, TANH_ONLY, LENGTHS, true, false>(
+                            Y[k], B[k], G[k], P[k], wi, wj, dwi, dwj, own, A.tab, (A.n_stages - 1 - st) * NC, lane, nullptr, live);
                     if (!LENGTHS || live > 1) {
                         pair_lds_store<EC>(ys1 + row1, fl, Y[k][1]);
                         pair_lds_store<EC>(bs1 + row1, fl, B[k][1]);

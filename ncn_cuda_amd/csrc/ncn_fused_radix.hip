@@ -3,8 +3,7 @@
 #include <cmath>
 #include <vector>
 
-#include "ncn_fused_kernels.h"
-#include "ncn_launch.h"
+#include "ncn_fused_dispatch.h"
 
 namespace ncn {
 
@@ -30,35 +29,6 @@ size_t radix_lds_bytes(int nc, int ec, bool backward, uint32_t rows, int n_stage
     if (lr > 1) bytes += (size_t)nw * t.f * 64 * sizeof(float);
     if (backward) bytes += (size_t)nw * n_stages * 2 * ec * sizeof(float);
     return bytes;
-}
-
-template <int NC, int EC>
-hipError_t launch_t(Pass pass, const FusedArgs& a, int grid, size_t lds, hipStream_t s) {
-    const bool backward = pass == kBackward;
-    constexpr TileShape t = fast_tile(NC, EC);
-    static_assert(t.r != 0, "radix shapes must be one-stage shapes too");
-    const bool tanh_only = a.tab.activation == NCN_ACT_TANH;
-    hipError_t err;
-    if (backward) {
-        auto k = tanh_only ? fused_backward_kernel<NC, EC, t.r, t.f, true, true>
-                           : fused_backward_kernel<NC, EC, t.r, t.f, false, true>;
-        err = ensure_dynamic_lds(reinterpret_cast<const void*>(k), lds);
-        if (err != hipSuccess) return err;
-        hipLaunchKernelGGL(k, dim3(grid), dim3(64 * kFusedWavesBwd), lds, s, a);
-    } else if (pass == kInverse) {
-        auto k = tanh_only ? fused_forward_kernel<NC, EC, t.r, t.f, true, true, true>
-                           : fused_forward_kernel<NC, EC, t.r, t.f, false, true, true>;
-        err = ensure_dynamic_lds(reinterpret_cast<const void*>(k), lds);
-        if (err != hipSuccess) return err;
-        hipLaunchKernelGGL(k, dim3(grid), dim3(64 * kFusedWavesFwd), lds, s, a);
-    } else {
-        auto k = tanh_only ? fused_forward_kernel<NC, EC, t.r, t.f, true, true>
-                           : fused_forward_kernel<NC, EC, t.r, t.f, false, true>;
-        err = ensure_dynamic_lds(reinterpret_cast<const void*>(k), lds);
-        if (err != hipSuccess) return err;
-        hipLaunchKernelGGL(k, dim3(grid), dim3(64 * kFusedWavesFwd), lds, s, a);
-    }
-    return hipGetLastError();
 }
 
 int64_t ipow(int64_t b, int e) {
@@ -124,7 +94,8 @@ int radix_grid(const ncn_shape* sh, const RadixPass& p, bool backward) {
     return (int)g;
 }
 
-hipError_t launch_fused_radix(Pass pass, FusedArgs& a, const ncn_shape* sh, const RadixPass& p, hipStream_t s) {
+hipError_t launch_fused_radix(Pass pass, FusedArgs& a, const ncn_shape* sh, const RadixPass& p, hipStream_t s,
+                              bool headwise) {
     const bool backward = pass == kBackward;
     const int nc = sh->n_cache, ec = (int)(sh->E / sh->n_head);
     a.N = sh->N;
@@ -145,11 +116,8 @@ hipError_t launch_fused_radix(Pass pass, FusedArgs& a, const ncn_shape* sh, cons
     a.scale_up = (float)std::pow((double)a.tab.m, -(double)(nc * p.count));
     const int grid = radix_grid(sh, p, backward);
     const size_t lds = radix_lds_bytes(nc, ec, backward, p.rows, p.count);
-#define NCN_CASE(NC, EC) \
-    if (nc == NC && ec == EC) return launch_t<NC, EC>(pass, a, grid, lds, s);
-    NCN_FOR_EACH_RADIX_CONFIG(NCN_CASE)
-#undef NCN_CASE
-    return hipErrorInvalidConfiguration;
+    if (headwise) return launch_fused_radix_headwise(pass, a, nc, ec, grid, lds, s);
+    return launch_fused_shape<true, false, false>(pass, a, nc, ec, grid, lds, s);
 }
 
 }  // namespace ncn

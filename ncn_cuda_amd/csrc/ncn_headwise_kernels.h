@@ -17,10 +17,12 @@
 
 namespace ncn {
 
-template <int NC, int EC, int R, int F, bool TANH_ONLY, bool STEP_MASK>
+// The three functions take the template and call arguments of forward_core, inverse_core and backward_core, so that a
+// kernel picks one or the other by name (ROWS and KU_W have nothing to act on here).
+template <int NC, int EC, int R, int F, bool TANH_ONLY = true, bool STEP_MASK = false, bool ROWS = false>
 __device__ __forceinline__ void headwise_forward_core(float (&x)[R][F], float (&a)[R][F], const float (&wi)[F],
                                                       const float (&wj)[F], const StepTable& S, int lane, float4* slots,
-                                                      int live) {
+                                                      int live = NC) {
     using T = Tile<NC, EC, R, F>;
 #pragma unroll 1
     for (int jo = 0; jo < T::LR; ++jo) {
@@ -52,10 +54,10 @@ __device__ __forceinline__ void headwise_forward_core(float (&x)[R][F], float (&
     }
 }
 
-template <int NC, int EC, int R, int F, bool TANH_ONLY, bool STEP_MASK>
+template <int NC, int EC, int R, int F, bool TANH_ONLY, bool STEP_MASK = false, bool ROWS = false>
 __device__ __forceinline__ void headwise_inverse_core(float (&y)[R][F], float (&b)[R][F], const float (&wi)[F],
                                                       const float (&wj)[F], const StepTable& S, int lane, float4* slots,
-                                                      int live) {
+                                                      int live = NC) {
     using T = Tile<NC, EC, R, F>;
 #pragma unroll 1
     for (int jo = T::LR - 1; jo >= 0; --jo) {
@@ -93,24 +95,24 @@ __device__ __forceinline__ void headwise_inverse_core(float (&y)[R][F], float (&
 // The reversible backward of backward_core on the same scaled state (Y = xs, B = bh, G = g / m^t, P = p / m^t), with
 //   U_if = P_if F'/4,   rh_if = U_if xs_jf,   G_if += ku (U_if + rh_if Wi'_f),   dWi_f += krho[t] rh_if xs_if,
 //   pivot row:  G_jf += ku sum_i (rh_if Wj'_f + c_if U_if),   dWj_f += krho[t] (sum_i rh_if) xs_jf.
-template <int NC, int EC, int R, int F, bool TANH_ONLY, bool STEP_MASK>
+// step_base inversion steps were done before (several stages in a row keep counting); with MASKED the dW shares are
+// weighted by `own` (1, or 0 for a group whose dW another window accounts for).
+template <int NC, int EC, int R, int F, bool MASKED, bool TANH_ONLY = true, bool STEP_MASK = false, bool ROWS = false,
+          bool KU_W = true>
 __device__ __forceinline__ void headwise_backward_core(float (&Y)[R][F], float (&B)[R][F], float (&G)[R][F],
                                                        float (&P)[R][F], const float (&wi)[F], const float (&wj)[F],
-                                                       float (&dwi)[F], float (&dwj)[F], const StepTable& S, int lane,
-                                                       float4* slots, int live) {
+                                                       float (&dwi)[F], float (&dwj)[F], float own, const StepTable& S,
+                                                       int step_base, int lane, float4* slots, int live = NC) {
     using T = Tile<NC, EC, R, F>;
     const int rl = (lane / T::LF) % T::LR;
-    float wiku[F];
-#pragma unroll
-    for (int f = 0; f < F; ++f) wiku[f] = S.ku * wi[f];
 #pragma unroll 1
     for (int jo = T::LR - 1; jo >= 0; --jo) {
         const float selku = (T::LR == 1 || rl == jo) ? S.ku : 0.0f;  // this lane holds the pivot row
 #pragma unroll
         for (int jr = R - 1; jr >= 0; --jr) {
             if (STEP_MASK && jo * R + jr >= live) continue;
-            const int ts = (T::LR - 1 - jo) * R + (R - 1 - jr);   // inversion steps done so far
-            const float krho = S.krho[ts];
+            const int ts = step_base + (T::LR - 1 - jo) * R + (R - 1 - jr);   // inversion steps done so far
+            const float krho = MASKED ? S.krho[ts] * own : S.krho[ts];
 #pragma unroll
             for (int rr = 0; rr < R; ++rr)
 #pragma unroll
@@ -143,8 +145,7 @@ __device__ __forceinline__ void headwise_backward_core(float (&Y)[R][F], float (
                     v[f] = fmaf(c, U, v[f]);
                     rhs[f] += rh;
                     dwi[f] = fmaf(krho * rh, Y[rr][f], dwi[f]);
-                    G[rr][f] = fmaf(S.ku, U, G[rr][f]);
-                    G[rr][f] = fmaf(rh, wiku[f], G[rr][f]);
+                    G[rr][f] = fmaf(S.ku, fmaf(rh, wi[f], U), G[rr][f]);
                     if (rr != jr) P[rr][f] = fmaf(S.om, G[rr][f], P[rr][f]);
                 }
             }
@@ -155,7 +156,7 @@ __device__ __forceinline__ void headwise_backward_core(float (&Y)[R][F], float (
                 // every row lane of the group adds its share of sum_i rh_if: the sum over lanes at the end completes it
                 dwj[f] = fmaf(krho * rhs[f], xj[f], dwj[f]);
             }
-            lane_sum_n<T::LF, T::LPG, false, F>(t);   // over the group's row lanes
+            lane_sum_n<T::LF, T::LPG, ROWS, F>(t);   // over the group's row lanes
 #pragma unroll
             for (int f = 0; f < F; ++f) {
                 G[jr][f] = fmaf(selku, t[f], G[jr][f]);
@@ -278,7 +279,8 @@ __global__ void __launch_bounds__(kBlockThreads, (TANH_ONLY && !INDEXED && R * F
                     H[rr][f] *= isc;
                 }
             }
-        headwise_backward_core<NC, EC, R, F, TANH_ONLY, INDEXED>(Y, B, G, H, wi, wj, dwi, dwj, A.tab, lane, slots, live);
+        headwise_backward_core<NC, EC, R, F, false, TANH_ONLY, INDEXED>(Y, B, G, H, wi, wj, dwi, dwj, 1.0f, A.tab, 0, lane, slots,
+                                                                      live);
         const float dn = A.tab.m_pow_n;       // NC steps done: undo the scaling of the gradients
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) {

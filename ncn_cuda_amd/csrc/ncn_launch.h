@@ -107,10 +107,14 @@ std::vector<FusedPass> plan_fused(const ncn_shape* sh, int first, int count, boo
 int64_t fused_items(const ncn_shape* sh, const FusedPass& p);
 // row_cap: rows of the dW partial buffer a backward pass may fill (grid / n_head rows per stage)
 int fused_grid(const ncn_shape* sh, const FusedPass& p, bool backward, int row_cap = kMaxGridX);
+// headwise: `sh` is the layout of a call on heads of one feature (headwise_width(E) adjacent heads to a "head")
 hipError_t launch_fused(Pass pass, FusedArgs& a, const ncn_shape* sh, const FusedPass& p, hipStream_t s,
-                        int row_cap = kMaxGridX);
+                        int row_cap = kMaxGridX, bool headwise = false);
 // the builds with context lengths (a.ctx_len set), ncn_fused_lengths.hip; launch_fused goes there by itself
 hipError_t launch_fused_lengths(Pass pass, const FusedArgs& a, int nc, int ec, int grid, size_t lds, hipStream_t s);
+// the builds for heads of one feature (ncn_fused_headwise.hip; the first goes to the second when a.ctx_len is set)
+hipError_t launch_fused_headwise(Pass pass, const FusedArgs& a, int nc, int ec, int grid, size_t lds, hipStream_t s);
+hipError_t launch_fused_headwise_lengths(Pass pass, const FusedArgs& a, int nc, int ec, int grid, size_t lds, hipStream_t s);
 
 
 // ---- multi-stage passes over radix-n levels, ncn_fused_radix.hip ---------------------------------------------
@@ -126,6 +130,8 @@ bool radix_fused_supported(const ncn_shape* sh);
 // fused = false: one level per pass whatever the shape (calls whose scalars only the generic kernels take)
 std::vector<RadixPass> plan_radix(const ncn_shape* sh, int first, int count, bool backward, bool fused = true);
 int radix_grid(const ncn_shape* sh, const RadixPass& p, bool backward);
-hipError_t launch_fused_radix(Pass pass, FusedArgs& a, const ncn_shape* sh, const RadixPass& p, hipStream_t s);
+hipError_t launch_fused_radix(Pass pass, FusedArgs& a, const ncn_shape* sh, const RadixPass& p, hipStream_t s,
+                              bool headwise = false);
+hipError_t launch_fused_radix_headwise(Pass pass, const FusedArgs& a, int nc, int ec, int grid, size_t lds, hipStream_t s);
 
 }  // namespace ncn

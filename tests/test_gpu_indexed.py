@@ -154,7 +154,8 @@ LENGTH_PASS_CASES = [
     (3, 2048, 64, 2, 2, 3, 6),     # range that starts at stage 3
     (5, 64, 128, 4, 4, 0, 3),      # tiny ring
     (3, 2048, 64, 4, 2, 1, 9),     # n = 2, head width 16
-    (2, 32, 32, 1, 2, 0, 4),       # n = 2, 16 groups: windows smaller than the workgroup's tiles
+    (2, 32, 32, 1, 2, 0, 4),       # n = 2, 16 groups: windows smaller than the workgroup's tiles    (3, 1024, 64, 64, 2, 0, 11),   # heads of one feature (two "heads" of 32 adjacent ones), n = 2
+    (4, 1024, 16, 16, 4, 0, 5),    # heads of one feature, n = 4
 ]
 
 

@@ -39,7 +39,12 @@ CASES = [
     (2, 5 * 256, 64, 2, 2, 0, 9),    # 640 groups = 5 * 2^7
     (2, 7 * 64, 32, 2, 4, 2, 5),     # n = 4, 112 groups = 7 * 16, from stage 2
     (2, 2048, 256, 2, 2, 0, 11),     # n = 2, head width 128 (16 lanes per row, windows of 32 groups)
-    (2, 1024, 128, 1, 4, 5, 4),      # n = 4, head width 128: closed passes on the rings of the high stages
+    (2, 1024, 128, 1, 4, 5, 4),      # n = 4, head width 128: closed passes on the rings of the high stages    # heads of one feature (E == n_head), laid out as heads of 32, 16 and 8 adjacent ones: the same passes
+    (2, 8192, 128, 128, 2, 0, 13),   # the deep configuration's N on 128 one-feature heads (4 "heads" of 32)
+    (3, 1024, 48, 48, 2, 0, 11),     # E = 3 * 16
+    (2, 1024, 128, 128, 4, 0, 5),    # n = 4
+    (2, 512, 24, 24, 4, 1, 5),       # n = 4, E = 3 * 8
+    (2, 512, 12, 12, 2, 0, 6),       # E = 3 * 4: no LDS passes at four heads to a row, one launch per stage
 ]
 
 
@@ -58,7 +63,8 @@ def test_multi_stage_matches_single_stage_and_oracle(M, case):
         cx, cxa = M.forward(cx, cxa, gWs[l], alpha, 0, n, C, first + l)
         outs.append((cx, cxa))
     # groups of 2 and 4 rows at heads of 8 to 128 features, an even number of groups: the call really uses LDS passes
-    if n in (2, 4) and E // C in (8, 16, 32, 64, 128) and (N // n) % 2 == 0:
+    wide = next(w for w in (32, 16, 8, 4, 1) if E % w == 0) if C == E else E // C   # one-feature heads: adjacent heads per row
+    if n in (2, 4) and wide in (8, 16, 32, 64, 128) and (N // n) % 2 == 0:
         import ctypes
         from ncn_cuda_amd import _lib
         shape = _lib.NcnShape(batch, N, E, C, n)
@@ -111,8 +117,8 @@ def test_multi_stage_dya_none_and_bf16_input(M):
 
 
 @pytest.mark.parametrize("act", [1, 2, -1, 3], ids=["relu", "sigmoid", "linear", "leaky_relu"])
-@pytest.mark.parametrize("case", [(2, 1024, 64, 2, 2, 0, 9), (2, 512, 128, 4, 4, 1, 4)],
-                         ids=["n2_halo_and_closed", "n4_from_stage1"])
+@pytest.mark.parametrize("case", [(2, 1024, 64, 2, 2, 0, 9), (2, 512, 128, 4, 4, 1, 4), (2, 512, 64, 64, 4, 0, 4)],
+                         ids=["n2_halo_and_closed", "n4_from_stage1", "n4_one_feature_heads"])
 def test_multi_stage_other_activations(M, case, act):
     """The LDS passes in their runtime-activation build.  relu and leaky relu have a kink at T = 0, where a float32
     recomputation may pick the other slope: they run on inputs whose T keeps one sign per batch entry (both slopes,
@@ -291,6 +297,7 @@ def test_backward_with_the_smaller_workspace_loops_over_windows(M):
     (2, 1024, 128, 4, 4, 0, 5),    # multi-stage passes and one-stage launches mixed
     (2, 512, 32, 2, 8, 0, 4),      # one-stage launches only
     (2, 96, 20, 2, 3, 1, 3),       # the generic kernels
+    (3, 1024, 32, 32, 2, 0, 11),   # heads of one feature: several multi-stage passes
 ], ids=lambda c: "b%d_N%d_E%d_C%d_n%d_s%d_L%d" % c)
 @pytest.mark.parametrize("grouping", ["closed", "lengths", "table"])
 def test_backward_without_reconstructed_inputs(M, case, grouping):

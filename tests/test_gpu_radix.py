@@ -42,8 +42,9 @@ CASES = [
     (2, 512, 32, 2, 8, 0, 3),      # n = 8: no LDS passes, closed-form positions in the one-stage register kernels
     (2, 81, 10, 2, 3, 0, 4),       # n = 3, head width 5: generic kernel
     (2, 128, 256, 2, 2, 2, 3),     # head width 128: register kernels, one level per launch
-    (2, 64, 16, 16, 2, 0, 6),      # one feature per head: register kernels, four heads to a lane, one level per launch
-    (2, 512, 8, 8, 8, 0, 3),       # the same at n = 8
+    (2, 64, 16, 16, 2, 0, 6),      # one feature per head, laid out as one head of 16: levels in LDS like heads of 16
+    (2, 1024, 64, 64, 4, 0, 5),    # the same at n = 4, two "heads" of 32
+    (2, 512, 8, 8, 8, 0, 3),       # one feature per head at n = 8: one level per launch
 ]
 
 
