@@ -18,7 +18,8 @@
 namespace ncn {
 
 // The three functions take the template and call arguments of forward_core, inverse_core and backward_core, so that a
-// kernel picks one or the other by name (ROWS and KU_W have nothing to act on here).
+// kernel picks one or the other by name (ROWS only reaches the sum over a group's row lanes; KU_W has nothing to act
+// on here).
 template <int NC, int EC, int R, int F, bool TANH_ONLY = true, bool STEP_MASK = false, bool ROWS = false>
 __device__ __forceinline__ void headwise_forward_core(float (&x)[R][F], float (&a)[R][F], const float (&wi)[F],
                                                       const float (&wj)[F], const StepTable& S, int lane, float4* slots,
@@ -117,13 +118,46 @@ __device__ __forceinline__ void headwise_backward_core(float (&Y)[R][F], float (
             for (int rr = 0; rr < R; ++rr)
 #pragma unroll
                 for (int f = 0; f < F; ++f) Y[rr][f] = fmaf(S.im, Y[rr][f], -B[rr][f]);  // xs before this step
-            float xj[F], cj[F], v[F], rhs[F];
+            float xj[F], cj[F];
             row_lane_broadcast<T::LF, T::LR, F>(Y[jr], xj, jo, lane, slots);
 #pragma unroll
-            for (int f = 0; f < F; ++f) {
-                cj[f] = xj[f] * wj[f];
-                v[f] = rhs[f] = 0.f;
-            }
+            for (int f = 0; f < F; ++f) cj[f] = xj[f] * wj[f];
+            if constexpr (T::LR == 1) {
+                // The whole group is in this lane: every row's share of the pivot row's gradient,
+                // ku (rh_if Wj'_f + c_if U_if) = ku U_if (xs_jf Wj'_f + c_if), goes straight into it, and dWj takes the
+                // row's rh_if as dWi does (no sums to carry through the step: fewer registers).
+#pragma unroll
+                for (int rr = 0; rr < R; ++rr) {
+#pragma unroll
+                    for (int f = 0; f < F; ++f) {
+                        const float c = fmaf(Y[rr][f], wi[f], cj[f]);
+                        const float z = fmaf(c, xj[f], Y[rr][f]);
+                        float w;
+                        if constexpr (TANH_ONLY) {
+                            const float r = __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(z) + 1.0f);
+                            B[rr][f] = fmaf(S.bk1, r, fmaf(S.im, B[rr][f], S.bk0));   // bh before this step
+                            w = fmaf(-r, r, r);
+                        } else {
+                            float Fv;
+                            act_Fw(z, S.activation, Fv, w);
+                            B[rr][f] = fmaf(S.bk0, Fv, S.im * B[rr][f]);
+                        }
+                        const float U = P[rr][f] * w;
+                        const float rh = U * xj[f];
+                        const float krh = krho * rh;
+                        dwi[f] = fmaf(krh, Y[rr][f], dwi[f]);
+                        dwj[f] = fmaf(krh, xj[f], dwj[f]);
+                        G[rr][f] = fmaf(S.ku, fmaf(rh, wi[f], U), G[rr][f]);
+                        G[jr][f] = fmaf(S.ku * U, cj[f] + c, G[jr][f]);
+                        if (rr != jr) P[rr][f] = fmaf(S.om, G[rr][f], P[rr][f]);
+                    }
+                }
+#pragma unroll
+                for (int f = 0; f < F; ++f) P[jr][f] = fmaf(S.om, G[jr][f], P[jr][f]);
+            } else {
+            float v[F], rhs[F];
+#pragma unroll
+            for (int f = 0; f < F; ++f) v[f] = rhs[f] = 0.f;
 #pragma unroll
             for (int rr = 0; rr < R; ++rr) {
 #pragma unroll
@@ -161,6 +195,7 @@ __device__ __forceinline__ void headwise_backward_core(float (&Y)[R][F], float (
             for (int f = 0; f < F; ++f) {
                 G[jr][f] = fmaf(selku, t[f], G[jr][f]);
                 P[jr][f] = fmaf(S.om, G[jr][f], P[jr][f]);
+            }
             }
             __builtin_amdgcn_sched_barrier(0);
         }
