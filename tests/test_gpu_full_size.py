@@ -19,6 +19,12 @@ CONFIGS = {
     "cfg4": (128, 8192, 128, 4, 2, 13, torch.float32, 1.0),
     "cfg5": (64, 2048, 128, 4, 8, 4, torch.float32, 0.1),
 }
+# the tensors of cfg3 and cfg4 read as rows of scalars: one feature per head (bench.py --scalar-heads); compared whole
+ONE_FEATURE_HEADS = {
+    "cfg3_heads1": (128, 4096, 128, 128, 16, 3, torch.bfloat16, 1.0),
+    "cfg4_heads1": (128, 8192, 128, 128, 2, 13, torch.float32, 1.0),
+}
+ALL_CONFIGS = {**CONFIGS, **ONE_FEATURE_HEADS}
 
 
 @pytest.fixture(scope="module")
@@ -30,7 +36,7 @@ def M():
 
 
 def _inputs(name):
-    batch, N, E, C, n, L, dtype, wscale = CONFIGS[name]
+    batch, N, E, C, n, L, dtype, wscale = ALL_CONFIGS[name]
     g = torch.Generator(device="cuda").manual_seed(7)
     x = torch.randn(batch, N, E, device="cuda", generator=g).to(dtype)
     xa = (0.5 * torch.randn(batch, N, E, device="cuda", generator=g)).to(dtype)
@@ -183,14 +189,15 @@ def test_more_than_2_31_elements_per_array(M, case):
     torch.cuda.empty_cache()
 
 
-@pytest.mark.parametrize("name,entries", [("cfg2", None), ("cfg5", None), ("cfg3", None), ("cfg4", None)])
+@pytest.mark.parametrize("name,entries", [("cfg2", None), ("cfg5", None), ("cfg3", None), ("cfg4", None),
+                                          ("cfg3_heads1", None), ("cfg4_heads1", 16)])
 def test_whole_tensor_against_the_c_oracle(M, name, entries):
     """Every element, not a slice: the configuration as bench.py's timed step runs it (backward without reconstructed
     inputs) against the plain C restatement in float64
     (oracle/ncn_oracle.c on the host threads: about 25 s for the four configurations on 16 threads).  `entries` cuts
     the comparison to that many batch entries spread over the batch, for a machine where that is too long."""
     from oracle import c_oracle as CO
-    batch, N, E, C, n, L, dtype, _ = CONFIGS[name]
+    batch, N, E, C, n, L, dtype, _ = ALL_CONFIGS[name]
     x, xa, dy, W = _inputs(name)
     y, ya, dx, dxa, dW = _run(M, x, xa, dy, W, C, n, L, dtype)
     sel = list(range(batch)) if entries is None else sorted({(k * batch) // entries for k in range(entries)} | {batch - 1})
