@@ -91,8 +91,10 @@ def test_bf16_autograd(pkg):
 
 
 @pytest.mark.parametrize("cfg", [(2, 1024, 128, 4, 2, 9, torch.float32), (2, 512, 128, 4, 4, 7, torch.float32),
-                                 (2, 256, 128, 4, 16, 3, torch.bfloat16), (2, 512, 64, 2, 2, 6, torch.bfloat16)],
-                         ids=["n2_L9_f32", "n4_L7_f32", "n16_L3_bf16", "n2_L6_bf16"])
+                                 (2, 256, 128, 4, 16, 3, torch.bfloat16), (2, 512, 64, 2, 2, 6, torch.bfloat16),
+                                 (2, 512, 64, 64, 2, 7, torch.float32), (2, 256, 128, 128, 16, 3, torch.bfloat16)],
+                         ids=["n2_L9_f32", "n4_L7_f32", "n16_L3_bf16", "n2_L6_bf16", "n2_L7_f32_one_feature_heads",
+                              "n16_L3_bf16_one_feature_heads"])
 def test_whole_net_node_matches_oracle_and_per_stage_nodes(pkg, cfg):
     """NCNNetFunction (one node for the stack, checkpoints every save_every stages) against the oracle and against
     the reference-style chain of per-stage nodes."""
