@@ -305,6 +305,21 @@ def test_planner_puts_stages_where_they_cost_least(lib):
     assert [(p[0], p[1], p[2]) for p in fwd] == [(0, 5, 1), (5, 8, 2)]
 
 
+def test_one_feature_heads_are_planned_as_heads_of_adjacent_ones(lib):
+    """E == n_head: the passes, and the workspace that goes with them, are those of E / w heads of w features, w the
+    largest of 32, 16, 8, 4 that divides E; at w = 4 there are no multi-stage passes."""
+    h = lib.load()
+    for E, w in ((128, 32), (48, 16), (24, 8)):
+        one, wide = _shape(lib, 4, 8192, E, E, 2), _shape(lib, 4, 8192, E, E // w, 2)
+        for backward in (False, True):
+            assert _passes(lib, one, 0, 13, backward) == _passes(lib, wide, 0, 13, backward) != []
+        for b in (0, 1, 2):
+            assert (h.ncn_workspace_bytes_stages(ctypes.byref(one), 0, 13, 0, b)
+                    == h.ncn_workspace_bytes_stages(ctypes.byref(wide), 0, 13, 0, b))
+    assert _passes(lib, _shape(lib, 4, 8192, 12, 12, 2), 0, 13, True) == []     # four heads to a row: one launch per stage
+    assert _passes(lib, _shape(lib, 4, 8192, 6, 6, 2), 0, 13, True) == []       # generic kernels
+
+
 @pytest.mark.parametrize("backward", [False, True])
 @pytest.mark.parametrize("dims", [(128, 8192, 128, 4, 2, 0, 13), (32, 1024, 128, 4, 4, 0, 5), (3, 1024, 64, 2, 2, 0, 11),
                                   (2, 2048, 64, 2, 2, 3, 6), (5, 64, 128, 4, 4, 0, 3), (1, 1 << 16, 32, 1, 2, 0, 20),
