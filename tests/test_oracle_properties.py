@@ -191,10 +191,12 @@ def _scalar_act(t, code):
     return t
 
 
+@pytest.mark.parametrize("heads", [2, 4], ids=["heads_of_2", "heads_of_1"])
 @pytest.mark.parametrize("act", [0, 1, 2, 3, -1], ids=["tanh", "relu", "sigmoid", "leaky_relu", "linear"])
-def test_activations_against_scalar_loops(act):
-    """One stage on a tiny input, written out with Python floats only (no tensor op shared with the oracle)."""
-    B, N, E, C, n, stage, alpha, m = 2, 8, 4, 2, 4, 1, 0.8, 0.9
+def test_activations_against_scalar_loops(act, heads):
+    """One stage on a tiny input, written out with Python floats only (no tensor op shared with the oracle); with four
+    heads every feature is a head of its own (the recurrence on rows of scalars)."""
+    B, N, E, C, n, stage, alpha, m = 2, 8, 4, heads, 4, 1, 0.8, 0.9
     ce = E // C
     X, Xa, W = _rand(B, N, E, seed=31), _rand(B, N, E, seed=32), _rand(2 * E, seed=33, scale=0.7)
     y, ya = O.stage_forward(X, Xa, W, alpha, n, C, stage, m, activation=act)
