@@ -73,6 +73,7 @@ def test_headline_tile_matches_triton_vectors():
 @pytest.mark.parametrize("case", [
     (2, 32, 16, 2, 4, 0, 3, 0), (3, 48, 30, 3, 3, 1, 2, 3), (1, 256, 32, 1, 2, 0, 8, 0), (2, 64, 128, 4, 16, 2, 3, 2),
     (2, 24, 12, 2, 1, 0, 2, -1), (2, 40, 6, 2, 5, 1000003, 2, 1), (1, 64, 256, 2, 32, 3, 1, 0),
+    (2, 64, 16, 16, 2, 0, 5, 0), (2, 64, 8, 8, 16, 1, 2, 0),      # one feature per head
 ], ids=lambda c: "b%d_N%d_E%d_C%d_n%d_s%d_L%d_a%d" % c)
 def test_matches_python_oracle(case):
     batch, N, E, C, n, first, L, act = case
